@@ -1,0 +1,261 @@
+"""The cache manager: paged keys/values with a block table per request, and state slots.
+
+Layers with the same cache needs form a group; every group has its own pages, its own allocator
+and, per request, its own block table.  A group that keeps all keys frees a request's pages when
+the request ends; a group with a window also frees a page as soon as every key on it has fallen
+out of the window of all queries still to come.  Freed pages are used again.  Beside the pages
+there are slots for per-request state of fixed size.
+
+Page layout (one cache, i.e. one layer): keys ``[pages, kv_heads, page_size, head_dim]``, values
+transposed ``[pages, kv_heads, head_dim, page_size]``, so that both attention products read each
+lane's operand as one contiguous vector.  The reference keeps ``[layers, blocks, block_size,
+kv_heads, head_dim]`` for both (/root/reference/utils/kv_cache.py:84-89); its allocator
+semantics are in :mod:`.pages`.
+"""
+from __future__ import annotations
+
+import dataclasses
+import hashlib
+import json
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..parts.base import PagedKVSpec, StateSpec
+from .pages import CacheExhaustedError, CacheStateError, PagePool
+
+
+@dataclasses.dataclass
+class LayerCacheView:
+    """What a mixer gets for one call of the order."""
+    group: int
+    keys: Optional[torch.Tensor]
+    values: Optional[torch.Tensor]
+    page_size: int
+    writable: bool
+    state: Optional[torch.Tensor] = None     # [slots, *shape] for a mixer with per-request state
+
+
+class CacheGroup:
+    def __init__(self, index: int, spec: PagedKVSpec, caches: List[int], num_pages: int, page_size: int):
+        self.index, self.spec, self.caches = index, spec, caches
+        self.pool = PagePool(num_pages, page_size)
+        self.page_size = page_size
+        self.keys = None     # [len(caches), pages, kv_heads, page_size, head_dim]
+        self.values = None   # [len(caches), pages, kv_heads, head_dim, page_size]
+
+    def first_needed_block(self, num_computed: int) -> int:
+        """First logical block a query at position >= num_computed can still see."""
+        if self.spec.window is None:
+            return 0
+        return max(0, num_computed - self.spec.window + 1) // self.page_size
+
+
+class RequestCache:
+    def __init__(self, request_id, n_groups: int):
+        self.request_id = request_id
+        self.tables: List[List[int]] = [[] for _ in range(n_groups)]
+        self.state_slot = -1
+        self.num_computed = 0
+
+
+class CacheManager:
+    def __init__(self, cache_specs: Dict[int, object], page_size: int, num_pages, num_state_slots: int = 0,
+                 device=None, dtype=torch.float32, allocate_storage: bool = True, model_identity: str = "model"):
+        self.page_size = page_size
+        self.device, self.dtype = device, dtype
+        self.model_identity = model_identity
+        self.groups: List[CacheGroup] = []
+        self.group_of_cache: Dict[int, int] = {}
+        self.layer_in_group: Dict[int, int] = {}
+        self.state_specs: Dict[int, StateSpec] = {}
+        by_spec: Dict[PagedKVSpec, List[int]] = {}
+        for cache, spec in sorted(cache_specs.items()):
+            if isinstance(spec, PagedKVSpec):
+                by_spec.setdefault(spec, []).append(cache)
+            elif isinstance(spec, StateSpec):
+                self.state_specs[cache] = spec
+            else:
+                raise TypeError(f"cache {cache}: unknown cache spec {spec!r}")
+        for spec, caches in by_spec.items():
+            pages = num_pages[len(self.groups)] if isinstance(num_pages, (list, tuple)) else num_pages
+            group = CacheGroup(len(self.groups), spec, caches, pages, page_size)
+            for position, cache in enumerate(caches):
+                self.group_of_cache[cache] = group.index
+                self.layer_in_group[cache] = position
+            self.groups.append(group)
+        self.num_state_slots = num_state_slots if self.state_specs else 0
+        self.free_state_slots = list(range(self.num_state_slots - 1, -1, -1))
+        self.state: Dict[int, torch.Tensor] = {}
+        self.requests: Dict[object, RequestCache] = {}
+        self.prefix_caching_possible = bool(self.groups) and not self.state_specs and all(
+            group.spec.window is None for group in self.groups)
+        if allocate_storage:
+            self._allocate_storage()
+
+    def _allocate_storage(self):
+        for group in self.groups:
+            spec, n = group.spec, len(group.caches)
+            pages = group.pool.num_pages
+            group.keys = torch.zeros((n, pages, spec.n_kv_heads, self.page_size, spec.head_dim), device=self.device, dtype=self.dtype)
+            group.values = torch.zeros((n, pages, spec.n_kv_heads, spec.head_dim, self.page_size), device=self.device, dtype=self.dtype)
+        for cache, spec in self.state_specs.items():
+            self.state[cache] = torch.zeros((max(1, self.num_state_slots), *spec.shape), device=self.device,
+                                            dtype=getattr(torch, spec.dtype))
+
+    @staticmethod
+    def bytes_per_token(cache_specs: Dict[int, object], dtype: torch.dtype) -> int:
+        size = torch.empty(0, dtype=dtype).element_size()
+        return sum(2 * spec.n_kv_heads * spec.head_dim * size for spec in cache_specs.values() if isinstance(spec, PagedKVSpec))
+
+    # -- views for the model ---------------------------------------------------------------
+    def view(self, call) -> LayerCacheView:
+        cache = call.cache
+        if cache in self.group_of_cache:
+            group = self.groups[self.group_of_cache[cache]]
+            layer = self.layer_in_group[cache]
+            return LayerCacheView(group.index, None if group.keys is None else group.keys[layer],
+                                  None if group.values is None else group.values[layer], self.page_size, call.writes_cache)
+        if cache in self.state:
+            return LayerCacheView(-1, None, None, self.page_size, call.writes_cache, self.state[cache])
+        return LayerCacheView(-1, None, None, self.page_size, call.writes_cache)
+
+    # -- requests ------------------------------------------------------------------------
+    def open(self, request_id) -> RequestCache:
+        if request_id in self.requests:
+            raise CacheStateError(f"request {request_id!r} already has a cache")
+        record = RequestCache(request_id, len(self.groups))
+        if self.state_specs:
+            if not self.free_state_slots:
+                raise CacheExhaustedError(f"no state slot is free: num_state_slots: {self.num_state_slots}")
+            record.state_slot = self.free_state_slots.pop()
+            for tensor in self.state.values():
+                tensor[record.state_slot].zero_()
+        self.requests[request_id] = record
+        return record
+
+    def has(self, request_id) -> bool:
+        return request_id in self.requests
+
+    def record(self, request_id) -> RequestCache:
+        if request_id not in self.requests:
+            raise KeyError(f"Request does not have a cache: {request_id!r}")
+        return self.requests[request_id]
+
+    def pages_needed(self, request_id, num_tokens: int) -> List[int]:
+        """Pages each group must still allocate so that positions < num_tokens are covered."""
+        record = self.requests.get(request_id)
+        needed = []
+        for group in self.groups:
+            have = len(record.tables[group.index]) if record is not None else 0
+            needed.append(max(0, -(-num_tokens // self.page_size) - have))
+        return needed
+
+    def available_pages(self) -> List[int]:
+        return [group.pool.num_available for group in self.groups]
+
+    def ensure(self, request_id, num_tokens: int) -> None:
+        """Allocate pages so that positions ``< num_tokens`` have a place in every group.
+
+        All-or-nothing: if any group runs out, pages taken by this call are given back and
+        :class:`CacheExhaustedError` is raised.
+        """
+        record = self.record(request_id)
+        taken = []
+        try:
+            for group in self.groups:
+                table = record.tables[group.index]
+                wanted = -(-num_tokens // self.page_size)
+                while len(table) < wanted:
+                    page = group.pool.allocate()
+                    table.append(page)
+                    taken.append((group, page))
+        except CacheExhaustedError:
+            for group, page in reversed(taken):
+                table = record.tables[group.index]
+                assert table[-1] == page
+                table.pop()
+                group.pool.release(page)
+            raise
+
+    def advance(self, request_id, num_computed: int) -> None:
+        """Tokens ``< num_computed`` are in the cache; give back pages a window has passed."""
+        record = self.record(request_id)
+        record.num_computed = num_computed
+        for group in self.groups:
+            if group.spec.window is None:
+                continue
+            table = record.tables[group.index]
+            for block in range(min(group.first_needed_block(num_computed), len(table))):
+                if table[block] >= 0:
+                    group.pool.release(table[block])
+                    table[block] = -1
+
+    def close(self, request_id) -> None:
+        """The request ended (or is preempted): everything it holds is given back."""
+        record = self.record(request_id)
+        for group in self.groups:
+            group.pool.release_table(record.tables[group.index])
+        if record.state_slot >= 0:
+            self.free_state_slots.append(record.state_slot)
+            record.state_slot = -1
+        del self.requests[request_id]
+
+    # -- prefix caching (complete pages of prompt tokens) ------------------------------------
+    def digest(self, parent: str, tokens: Sequence[int]) -> str:
+        """Chained sha256 over (parent digest, page tokens, model, adapter), root parent "root"
+        (/root/reference/utils/engine.py:193-195)."""
+        payload = json.dumps([parent, list(tokens), self.model_identity, "none"], separators=(",", ":")).encode("utf-8")
+        return hashlib.sha256(payload).hexdigest()
+
+    def share_prefix(self, request_id, prompt: Sequence[int]) -> int:
+        """Attach the longest chain of cached complete pages; always leaves at least one prompt
+        token to compute (/root/reference/utils/engine.py:197-208).  Returns tokens covered."""
+        if not self.prefix_caching_possible:
+            return 0
+        record = self.record(request_id)
+        if any(record.tables[group.index] for group in self.groups):
+            raise CacheStateError("a prefix can only be shared into an empty block table")
+        parent, covered = "root", 0
+        for block in range((len(prompt) - 1) // self.page_size):
+            digest = self.digest(parent, prompt[block * self.page_size:(block + 1) * self.page_size])
+            if any(group.pool.find(digest) is None for group in self.groups):
+                break
+            for group in self.groups:
+                group.pool.share(digest, record.tables[group.index])
+            covered += self.page_size
+            parent = digest
+        record.num_computed = covered
+        return covered
+
+    def register_prefix(self, request_id, prompt: Sequence[int], old_computed: int, new_computed: int) -> None:
+        """Register pages of prompt tokens that became complete between two counts of computed
+        tokens (/root/reference/utils/engine.py:383-401)."""
+        if not self.prefix_caching_possible:
+            return
+        record = self.record(request_id)
+        old_complete = min(old_computed, len(prompt)) // self.page_size
+        new_complete = min(new_computed, len(prompt)) // self.page_size
+        for block in range(old_complete, new_complete):
+            tokens = prompt[block * self.page_size:(block + 1) * self.page_size]
+            for group in self.groups:
+                table = record.tables[group.index]
+                parent = "root" if block == 0 else group.pool.page_digest[table[block - 1]]
+                group.pool.register(table[block], self.digest(parent, tokens))
+
+    def check_invariants(self) -> None:
+        for group in self.groups:
+            group.pool.check_invariants()
+            held = {}
+            for record in self.requests.values():
+                for page in record.tables[group.index]:
+                    if page >= 0:
+                        held[page] = held.get(page, 0) + 1
+            for page in range(group.pool.num_pages):
+                assert group.pool.references[page] == held.get(page, 0), (
+                    f"group {group.index} page {page}: {group.pool.references[page]} references, {held.get(page, 0)} holders")
+        slots = [record.state_slot for record in self.requests.values() if record.state_slot >= 0]
+        assert len(slots) == len(set(slots)), "a state slot is held twice"
+        assert not set(slots) & set(self.free_state_slots), "a held state slot is on the free list"
+        if self.state_specs:
+            assert len(slots) + len(self.free_state_slots) == self.num_state_slots, "a state slot was lost"

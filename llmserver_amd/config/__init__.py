@@ -1,0 +1,8 @@
+from .base import ConfigError, ModelConfig, UnsupportedModelError, field, read_config_json
+from .qwen3 import Qwen3Config
+from .registry import (config_from_dict, load_config, register_architecture, registered_architectures,
+                       resolve_architecture, unregister_architecture)
+
+__all__ = ["ConfigError", "ModelConfig", "UnsupportedModelError", "field", "read_config_json", "Qwen3Config",
+           "config_from_dict", "load_config", "register_architecture", "registered_architectures",
+           "resolve_architecture", "unregister_architecture"]

@@ -1,0 +1,332 @@
+// Causal attention over the paged cache for a flat batch: portions of prompts and single decoded
+// tokens go through the same kernel.  Compiled once per (element type, head size): -DLSA_ND=<head
+// size / 16> and -DLSA_BF16=0|1.
+//
+// Work is a list of items made on the host.  An item is one wavefront's job: a tile of 16
+// (token, head-of-the-group) pairs of one request against the keys [k_begin, k_end) of one KV
+// head.  The wavefront walks the keys in steps, keeps a running maximum and sum per pair (online
+// softmax, 32-bit) and accumulates the output in MFMA registers.  If the item covers every key
+// its pairs can see, it writes the output; otherwise it writes its maximum, sum and unnormalised
+// output to a partial slot and `merge` combines the slots by log-sum-exp.
+//
+// MFMA use (64-lane wavefront, lane = 16 * quad + col):
+//   scores:  S^T[key][pair] = K[key][:] . Q[pair][:]      A = K rows (lane: key col, 8 or 4 dims of quad)
+//                                                          B = Q^T    (lane: pair col, same dims)
+//            result lane holds keys 4*quad..4*quad+3 of pair col, so the softmax of a pair is a
+//            reduction inside a lane plus two shuffles, and
+//   output:  O^T[dim][pair] += V^T[dim][key] . P^T[key][pair]   A = V^T rows (lane: dim col, keys of quad)
+//                                                                B = P^T, exactly the registers S^T left.
+// Keys are stored [page][kv_head][slot][dim], values transposed [page][kv_head][dim][slot], so
+// both A operands are contiguous vector loads straight from the pages.
+#include "common.hpp"
+
+#ifndef LSA_ND
+#error "compile with -DLSA_ND=<head_dim / 16>"
+#endif
+#ifndef LSA_BF16
+#error "compile with -DLSA_BF16=0 or 1"
+#endif
+
+using namespace lsa;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+constexpr int ND = LSA_ND;          // 16-wide chunks of the head
+constexpr int D = ND * 16;          // head size
+constexpr float NEG_INF = -__builtin_huge_valf();
+
+struct Item { int row, q0, k_begin, k_end; };
+
+struct Geometry {
+    int n_q, n_kv, group, gheads, tokens_per_tile, gtiles, page_size, window;
+    float scale;
+};
+
+#if LSA_BF16
+typedef bf16_t elem_t;
+constexpr int KEY_STEP = 32;                 // keys per loop step (one 16x16x32 MFMA in the output product)
+constexpr int NS = (D + 31) / 32;            // 32-dim steps of the score product
+#else
+typedef float elem_t;
+constexpr int KEY_STEP = 16;
+constexpr int NS = D / 16;                   // 16-dim steps (four 16x16x4 MFMAs each)
+#endif
+
+__global__ __launch_bounds__(256) void paged_attention_kernel(
+    const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
+    const elem_t* __restrict__ keys, const elem_t* __restrict__ values,
+    const int* __restrict__ table, int table_stride,
+    const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
+    const Item* __restrict__ items, const int* __restrict__ item_slot, int n_items,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, Geometry g) {
+    const int lane = threadIdx.x & 63;
+    const int item_index = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item_index >= n_items) return;
+    const Item item = items[item_index];
+    const int kv_head = blockIdx.y / g.gtiles, gtile = blockIdx.y % g.gtiles;
+    const int col = lane & 15, quad = lane >> 4;
+    const int row = item.row;
+    const int n = row_len[row], first_pos = row_ctx[row] - n, token0 = row_start[row] + item.q0;
+    // The pair this lane's column stands for.
+    const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
+    const bool pair_valid = pair_token < g.tokens_per_tile && item.q0 + pair_token < n && pair_head_in_group < g.group;
+    const int q_pos = pair_valid ? first_pos + item.q0 + pair_token : -1;
+    const int head = kv_head * g.group + pair_head_in_group;
+    const int* row_table = table + (size_t)row * table_stride;
+    const int ps = g.page_size;
+    const size_t kv_head_keys = (size_t)kv_head * ps * D;      // offset of the head inside a key page
+    const size_t kv_head_values = (size_t)kv_head * D * ps;
+    const size_t page_elems = (size_t)g.n_kv * ps * D;
+
+    // Q^T operand, kept in registers for the whole item.
+#if LSA_BF16
+    bf16x8 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int dim = 32 * s + 8 * quad;
+        bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (pair_valid && dim < D)
+            x = *reinterpret_cast<const bf16x8*>(q + (size_t)(token0 + pair_token) * q_token_stride + (size_t)head * D + dim);
+        qf[s] = x;
+    }
+#else
+    f32x4 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        f32x4 x = {0.f, 0.f, 0.f, 0.f};
+        if (pair_valid)
+            x = *reinterpret_cast<const f32x4*>(q + (size_t)(token0 + pair_token) * q_token_stride + (size_t)head * D + 16 * s + 4 * quad);
+        qf[s] = x;
+    }
+#endif
+
+    f32x4 acc[ND];
+#pragma unroll
+    for (int c = 0; c < ND; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float run_max = NEG_INF, run_sum = 0.f;    // run_sum: this lane's share (its keys) of the pair's sum
+
+    const int k_begin = item.k_begin, k_end = item.k_end;
+    for (int kt = (k_begin / KEY_STEP) * KEY_STEP; kt < k_end; kt += KEY_STEP) {
+        const bool edge = kt < k_begin || kt + KEY_STEP > k_end;
+#if LSA_BF16
+        // ---- scores of two 16-key tiles ----
+        f32x4 st[2];
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            const int key = kt + 16 * t2 + col;
+            const bool ok = key >= k_begin && key < k_end;
+            const elem_t* kp = keys;
+            if (ok) kp = keys + (size_t)row_table[key / ps] * page_elems + kv_head_keys + (size_t)(key % ps) * D + 8 * quad;
+            f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                bf16x8 kf = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (ok && 32 * s + 8 * quad < D) kf = *reinterpret_cast<const bf16x8*>(kp + 32 * s);
+                s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], s4, 0, 0, 0);
+            }
+            st[t2] = s4;
+        }
+        // ---- mask, running maximum ----
+        float sv[8];
+        float tile_max = NEG_INF;
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int kpos = kt + 16 * t2 + 4 * quad + r;
+                const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
+                const float v = seen ? st[t2][r] * g.scale : NEG_INF;
+                sv[4 * t2 + r] = v;
+                tile_max = fmaxf(tile_max, v);
+            }
+#else
+        const int key = kt + col;
+        const bool ok = key >= k_begin && key < k_end;
+        const elem_t* kp = keys;
+        if (ok) kp = keys + (size_t)row_table[key / ps] * page_elems + kv_head_keys + (size_t)(key % ps) * D + 4 * quad;
+        f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            f32x4 kf = {0.f, 0.f, 0.f, 0.f};
+            if (ok) kf = *reinterpret_cast<const f32x4*>(kp + 16 * s);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[e], qf[s][e], s4, 0, 0, 0);
+        }
+        float sv[4];
+        float tile_max = NEG_INF;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int kpos = kt + 4 * quad + r;
+            const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
+            const float v = seen ? s4[r] * g.scale : NEG_INF;
+            sv[r] = v;
+            tile_max = fmaxf(tile_max, v);
+        }
+#endif
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+        const float new_max = fmaxf(run_max, tile_max);
+        const float use_max = new_max == NEG_INF ? 0.f : new_max;
+        const float alpha = __expf(run_max - use_max) ;   // run_max = -inf gives 0
+        run_max = new_max;
+        run_sum *= alpha;
+#pragma unroll
+        for (int c = 0; c < ND; ++c) acc[c] *= alpha;
+
+#if LSA_BF16
+        bf16x8 pf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float p = __expf(sv[e] - use_max);
+            run_sum += p;
+            pf[e] = (bf16_t)p;
+        }
+        // ---- output: values of the two 4-key pieces this lane's quad owns ----
+        const elem_t* vp[2];
+        bool vok[2];
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            const int key0 = kt + 16 * t2 + 4 * quad;
+            vok[t2] = key0 + 4 > k_begin && key0 < k_end;
+            vp[t2] = values;
+            if (vok[t2]) vp[t2] = values + (size_t)row_table[key0 / ps] * page_elems + kv_head_values + (size_t)col * ps + key0 % ps;
+        }
+#pragma unroll
+        for (int c = 0; c < ND; ++c) {
+            bf16x8 vf;
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                bf16x4 piece = {0, 0, 0, 0};
+                if (vok[t2]) piece = *reinterpret_cast<const bf16x4*>(vp[t2] + (size_t)(16 * c) * ps);
+                if (edge) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int kpos = kt + 16 * t2 + 4 * quad + r;
+                        if (kpos < k_begin || kpos >= k_end) piece[r] = (bf16_t)0.f;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vf[4 * t2 + r] = piece[r];
+            }
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[c], 0, 0, 0);
+        }
+#else
+        float pv[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            pv[r] = expf(sv[r] - use_max);
+            run_sum += pv[r];
+        }
+        const int key0 = kt + 4 * quad;
+        const bool vok = key0 + 4 > k_begin && key0 < k_end;
+        const elem_t* vp = values;
+        if (vok) vp = values + (size_t)row_table[key0 / ps] * page_elems + kv_head_values + (size_t)col * ps + key0 % ps;
+#pragma unroll
+        for (int c = 0; c < ND; ++c) {
+            f32x4 vf = {0.f, 0.f, 0.f, 0.f};
+            if (vok) vf = *reinterpret_cast<const f32x4*>(vp + (size_t)(16 * c) * ps);
+            if (edge) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (key0 + r < k_begin || key0 + r >= k_end) vf[r] = 0.f;
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[r], pv[r], acc[c], 0, 0, 0);
+        }
+#endif
+    }
+
+    run_sum += __shfl_xor(run_sum, 16, 64);
+    run_sum += __shfl_xor(run_sum, 32, 64);
+    if (!pair_valid) return;
+    const int slot = item_slot[item_index];
+    if (slot < 0) {
+        const float inv = run_sum > 0.f ? 1.f / run_sum : 0.f;
+        elem_t* o = out + ((size_t)(token0 + pair_token) * g.n_q + head) * D + 4 * quad;
+#pragma unroll
+        for (int c = 0; c < ND; ++c) {
+#if LSA_BF16
+            bf16x4 r4;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) r4[r] = (bf16_t)(acc[c][r] * inv);
+            *reinterpret_cast<bf16x4*>(o + 16 * c) = r4;
+#else
+            *reinterpret_cast<f32x4*>(o + 16 * c) = acc[c] * inv;
+#endif
+        }
+    } else {
+        const size_t base = ((size_t)slot * gridDim.y + blockIdx.y) * 16 + col;
+        float* pa = part_acc + base * D + 4 * quad;
+#pragma unroll
+        for (int c = 0; c < ND; ++c) *reinterpret_cast<f32x4*>(pa + 16 * c) = acc[c];
+        if (quad == 0) {
+            part_ml[base * 2] = run_max;
+            part_ml[base * 2 + 1] = run_sum;
+        }
+    }
+}
+
+// Merge the partial slots of a tile: out = sum_s w_s acc_s / sum_s w_s l_s, w_s = exp(m_s - max m).
+struct Merge { int row, q0, first_slot, n_slots; };
+
+__global__ __launch_bounds__(256) void merge_kernel(
+    elem_t* __restrict__ out, const int* __restrict__ row_start, const int* __restrict__ row_len,
+    const Merge* __restrict__ merges, const float* __restrict__ part_acc, const float* __restrict__ part_ml, Geometry g) {
+    __shared__ float weight[64 * 16];      // [slot][pair], at most 64 slots
+    __shared__ float inv_sum[16];
+    const Merge m = merges[blockIdx.x];
+    const int kv_head = blockIdx.y / g.gtiles, gtile = blockIdx.y % g.gtiles;
+    const int n = row_len[m.row], token0 = row_start[m.row] + m.q0;
+    if (threadIdx.x < 16) {
+        const int col = threadIdx.x;
+        float top = NEG_INF;
+        for (int s = 0; s < m.n_slots; ++s)
+            top = fmaxf(top, part_ml[(((size_t)(m.first_slot + s) * gridDim.y + blockIdx.y) * 16 + col) * 2]);
+        float total = 0.f;
+        for (int s = 0; s < m.n_slots; ++s) {
+            const size_t base = (((size_t)(m.first_slot + s) * gridDim.y + blockIdx.y) * 16 + col) * 2;
+            const float w = top == NEG_INF ? 0.f : expf(part_ml[base] - top);
+            weight[s * 16 + col] = w;
+            total += w * part_ml[base + 1];
+        }
+        inv_sum[col] = total > 0.f ? 1.f / total : 0.f;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < 16 * D; e += blockDim.x) {
+        const int col = e / D, dim = e % D;
+        const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
+        if (pair_token >= g.tokens_per_tile || m.q0 + pair_token >= n || pair_head_in_group >= g.group) continue;
+        float total = 0.f;
+        for (int s = 0; s < m.n_slots; ++s) {
+            const float w = weight[s * 16 + col];
+            if (w != 0.f) total += w * part_acc[(((size_t)(m.first_slot + s) * gridDim.y + blockIdx.y) * 16 + col) * D + dim];
+        }
+        const int head = kv_head * g.group + pair_head_in_group;
+        out[((size_t)(token0 + pair_token) * g.n_q + head) * D + dim] = (elem_t)(total * inv_sum[col]);
+    }
+}
+
+LSA_EXPORT int lsa_paged_attention(
+    const void* q, long q_token_stride, void* out, const void* keys, const void* values, const int* table, int table_stride,
+    const int* row_start, const int* row_len, const int* row_ctx, const void* items, const int* item_slot, int n_items,
+    const void* merges, int n_merges, float* part_acc, float* part_ml, float scale, int window, int page_size, int n_q,
+    int n_kv, int gheads, int tokens_per_tile, int gtiles, hipStream_t stream) {
+    if (n_items <= 0) return 0;
+    Geometry g;
+    g.n_q = n_q; g.n_kv = n_kv; g.group = n_q / n_kv; g.gheads = gheads; g.tokens_per_tile = tokens_per_tile;
+    g.gtiles = gtiles; g.page_size = page_size; g.window = window; g.scale = scale;
+    dim3 grid((n_items + 3) / 4, n_kv * gtiles);
+    paged_attention_kernel<<<grid, 256, 0, stream>>>(
+        (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
+        row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g);
+    int err = (int)hipGetLastError();
+    if (err || n_merges <= 0) return err;
+    dim3 mgrid(n_merges, n_kv * gtiles);
+    merge_kernel<<<mgrid, 256, 0, stream>>>((elem_t*)out, row_start, row_len, (const Merge*)merges, part_acc, part_ml, g);
+    LSA_LAUNCH_CHECK();
+}
+
+LSA_EXPORT int lsa_attention_head_dim() { return D; }
+LSA_EXPORT int lsa_attention_is_bf16() { return LSA_BF16; }

@@ -1,0 +1,185 @@
+// Row-wise kernels of the step: embedding lookup, residual sum fused with RMSNorm, SwiGLU,
+// bias add.  One source for bfloat16 and float32 activations; sums, square sums, rsqrt,
+// sigmoid and products are 32-bit inside, results are rounded once when stored.
+#include "common.hpp"
+
+using namespace lsa;
+
+// ------------------------------------------------------------------------------------------
+// Embedding: out[t, :] = table[ids[t], :].  An id outside the table gives a zero row (the
+// host refuses such ids before the launch; the guard keeps a bad id from faulting the GPU).
+template <typename T, bool VEC>
+__global__ void embedding_kernel(const T* __restrict__ table, const int* __restrict__ ids, T* __restrict__ out,
+                                 int width, int vocab) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    const bool ok = id >= 0 && id < vocab;
+    const T* src = table + (size_t)(ok ? id : 0) * width;
+    T* dst = out + (size_t)t * width;
+    if (VEC) {
+        constexpr int V = Elem<T>::kVec;
+        for (int i = threadIdx.x * V; i < width; i += blockDim.x * V) {
+            Vec16<T> x = load_vec16(src + i);
+            if (!ok) {
+#pragma unroll
+                for (int k = 0; k < V; ++k) x.v[k] = (T)0.f;
+            }
+            store_vec16(dst + i, x);
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = ok ? src[i] : (T)0.f;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// s = resid + delta (32-bit sum, rounded to T as the new residual stream);
+// out = s * rsqrt(mean(s^2) + eps) * w, computed from the rounded s.
+// rows == nullptr: every token row t: resid[t] = s, out[t] = norm.
+// rows != nullptr: out[i] = norm of row rows[i]; resid is not written.
+template <typename T, int V>
+__device__ inline void load_sum(const T* __restrict__ x, const T* __restrict__ d, int i, float (&s)[V]) {
+    if (V > 1) {
+        Vec16<T> a = load_vec16(x + i);
+#pragma unroll
+        for (int k = 0; k < V; ++k) s[k] = (float)a.v[k];
+        if (d) {
+            Vec16<T> b = load_vec16(d + i);
+#pragma unroll
+            for (int k = 0; k < V; ++k) s[k] = Elem<T>::round(s[k] + (float)b.v[k]);
+        }
+    } else {
+        s[0] = (float)x[i];
+        if (d) s[0] = Elem<T>::round(s[0] + (float)d[i]);
+    }
+}
+
+template <typename T, int V>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid, const T* __restrict__ delta,
+                                                          const float* __restrict__ weight, float eps,
+                                                          T* __restrict__ out, const int* __restrict__ rows, int width) {
+    __shared__ float scratch[16];
+    const int src_row = rows ? rows[blockIdx.x] : blockIdx.x;
+    T* x = resid + (size_t)src_row * width;
+    const T* d = delta ? delta + (size_t)src_row * width : nullptr;
+    T* y = out + (size_t)blockIdx.x * width;
+    float sq = 0.f;
+    for (int i = threadIdx.x * V; i < width; i += blockDim.x * V) {
+        float s[V];
+        load_sum<T, V>(x, d, i, s);
+#pragma unroll
+        for (int k = 0; k < V; ++k) sq += s[k] * s[k];
+    }
+    const float total = block_sum(sq, scratch);
+    const float rstd = rsqrtf(total / (float)width + eps);
+    for (int i = threadIdx.x * V; i < width; i += blockDim.x * V) {
+        float s[V];
+        load_sum<T, V>(x, d, i, s);
+        if (V > 1) {
+            Vec16<T> o, r;
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                r.v[k] = (T)s[k];
+                o.v[k] = (T)(s[k] * rstd * weight[i + k]);
+            }
+            if (d && !rows) store_vec16(x + i, r);
+            store_vec16(y + i, o);
+        } else {
+            if (d && !rows) x[i] = (T)s[0];
+            y[i] = (T)(s[0] * rstd * weight[i]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// SwiGLU: out[t, i] = silu(gu[t, i]) * gu[t, I + i], silu(g) = g * sigmoid(g).
+template <typename T, int V>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter) {
+    const int t = blockIdx.y;
+    const int i = (blockIdx.x * blockDim.x + threadIdx.x) * V;
+    if (i >= inter) return;
+    const T* g = gate_up + (size_t)t * 2 * inter + i;
+    const T* u = g + inter;
+    T* o = out + (size_t)t * inter + i;
+    if (V > 1) {
+        Vec16<T> a = load_vec16(g), b = load_vec16(u), r;
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            const float gv = (float)a.v[k];
+            r.v[k] = (T)(gv / (1.f + expf(-gv)) * (float)b.v[k]);
+        }
+        store_vec16(o, r);
+    } else {
+        const float gv = (float)g[0];
+        o[0] = (T)(gv / (1.f + expf(-gv)) * (float)u[0]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// y[t, n] += bias[n] (bias float32).
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, int n, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) y[i] = (T)((float)y[i] + bias[i % n]);
+}
+
+// ------------------------------------------------------------------------------------------
+template <typename T>
+static int launch_embedding(const void* table, const int* ids, void* out, int n_tokens, int width, int vocab, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    const bool vec = width % Elem<T>::kVec == 0;
+    if (vec) embedding_kernel<T, true><<<n_tokens, 256, 0, stream>>>((const T*)table, ids, (T*)out, width, vocab);
+    else embedding_kernel<T, false><<<n_tokens, 256, 0, stream>>>((const T*)table, ids, (T*)out, width, vocab);
+    LSA_LAUNCH_CHECK();
+}
+
+template <typename T>
+static int launch_add_rmsnorm(void* resid, const void* delta, const float* weight, float eps, void* out, const int* rows,
+                              int n_out, int width, hipStream_t stream) {
+    if (n_out <= 0) return 0;
+    if (width % Elem<T>::kVec == 0)
+        add_rmsnorm_kernel<T, Elem<T>::kVec><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, weight, eps, (T*)out, rows, width);
+    else
+        add_rmsnorm_kernel<T, 1><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, weight, eps, (T*)out, rows, width);
+    LSA_LAUNCH_CHECK();
+}
+
+template <typename T>
+static int launch_swiglu(const void* gate_up, void* out, int n_tokens, int inter, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (inter % Elem<T>::kVec == 0) {
+        constexpr int V = Elem<T>::kVec;
+        dim3 grid((inter / V + 255) / 256, n_tokens);
+        swiglu_kernel<T, V><<<grid, 256, 0, stream>>>((const T*)gate_up, (T*)out, inter);
+    } else {
+        dim3 grid((inter + 255) / 256, n_tokens);
+        swiglu_kernel<T, 1><<<grid, 256, 0, stream>>>((const T*)gate_up, (T*)out, inter);
+    }
+    LSA_LAUNCH_CHECK();
+}
+
+template <typename T>
+static int launch_add_bias(void* y, const float* bias, int n_tokens, int n, hipStream_t stream) {
+    const size_t total = (size_t)n_tokens * n;
+    if (total == 0) return 0;
+    add_bias_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>((T*)y, bias, n, total);
+    LSA_LAUNCH_CHECK();
+}
+
+// dtype: 0 = float32, 1 = bfloat16
+LSA_EXPORT int lsa_embedding(int dtype, const void* table, const int* ids, void* out, int n_tokens, int width, int vocab, hipStream_t stream) {
+    return dtype ? launch_embedding<bf16_t>(table, ids, out, n_tokens, width, vocab, stream)
+                 : launch_embedding<float>(table, ids, out, n_tokens, width, vocab, stream);
+}
+LSA_EXPORT int lsa_add_rmsnorm(int dtype, void* resid, const void* delta, const float* weight, float eps, void* out,
+                               const int* rows, int n_out, int width, hipStream_t stream) {
+    return dtype ? launch_add_rmsnorm<bf16_t>(resid, delta, weight, eps, out, rows, n_out, width, stream)
+                 : launch_add_rmsnorm<float>(resid, delta, weight, eps, out, rows, n_out, width, stream);
+}
+LSA_EXPORT int lsa_swiglu(int dtype, const void* gate_up, void* out, int n_tokens, int inter, hipStream_t stream) {
+    return dtype ? launch_swiglu<bf16_t>(gate_up, out, n_tokens, inter, stream)
+                 : launch_swiglu<float>(gate_up, out, n_tokens, inter, stream);
+}
+LSA_EXPORT int lsa_add_bias(int dtype, void* y, const float* bias, int n_tokens, int n, hipStream_t stream) {
+    return dtype ? launch_add_bias<bf16_t>(y, bias, n_tokens, n, stream)
+                 : launch_add_bias<float>(y, bias, n_tokens, n, stream);
+}

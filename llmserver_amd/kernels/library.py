@@ -1,0 +1,59 @@
+"""Loads the compiled kernel libraries through ctypes and declares their entry points."""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+from typing import Dict
+
+from . import build
+
+_P = c_void_p
+_SIGNATURES = {
+    "lsa_embedding": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_add_rmsnorm": [c_int, _P, _P, _P, c_float, _P, _P, c_int, c_int, _P],
+    "lsa_swiglu": [c_int, _P, _P, c_int, c_int, _P],
+    "lsa_add_bias": [c_int, _P, _P, c_int, c_int, _P],
+    "lsa_qk_norm_rope_kv_write": [c_int, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int,
+                                  c_int, c_int, _P],
+    "lsa_sample": [_P, _P, _P, _P, c_int, c_int, _P],
+    "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, _P, _P, c_float,
+                            c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+    "lsa_attention_head_dim": [],
+    "lsa_attention_is_bf16": [],
+    "lsa_gemm_skinny": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+}
+
+_loaded: Dict[str, ctypes.CDLL] = {}
+
+
+class KernelLibraryMissing(RuntimeError):
+    """The HIP extension is not there and cannot be built: the engine does not run without it."""
+
+
+def load(name: str) -> ctypes.CDLL:
+    """The named library, compiled first if it is not there yet.  Fails loudly; there is no fallback."""
+    if name in _loaded:
+        return _loaded[name]
+    try:
+        path = build.build([name])[name]
+    except build.KernelBuildError as error:
+        raise KernelLibraryMissing(f"HIP kernel library {name!r} is missing and could not be built: {error}") from error
+    library = ctypes.CDLL(path)
+    for symbol, argtypes in _SIGNATURES.items():
+        if hasattr(library, symbol):
+            function = getattr(library, symbol)
+            function.argtypes = argtypes
+            function.restype = c_int
+    _loaded[name] = library
+    return library
+
+
+def preload(names) -> None:
+    """Compile what is missing in one go (in parallel), then load."""
+    build.build(list(names))
+    for name in names:
+        load(name)
+
+
+def loaded_libraries():
+    return {name: library._name for name, library in _loaded.items()}

@@ -1,0 +1,168 @@
+"""Grouped-query causal attention over a paged cache, with optional per-head q/k RMSNorm,
+rotate-half position encoding and an optional window.
+
+Formulas in execution order (/root/reference/utils/attention.py:114-160, 183-197):
+``q,k,v = x Wq^T, x Wk^T, x Wv^T`` as one stacked product (54-66, 124-126); per head
+``q^ = q * rsqrt(mean_d(q^2) + eps) * w_q`` and the same for k, before the rotation (157-158;
+fused form /root/reference/utils/fused_ops.py:90-134); rotation of q and k by the absolute
+position; rotated k and raw v of every new token go to the cache before attention reads it
+(/root/reference/utils/kv_cache.py:335-349), so a token sees itself; query head ``h`` uses KV head
+``h // G`` (/root/reference/utils/attention.py:77,188); scores ``q.k * scale`` with
+``scale = head_dim^-0.5`` by default (/root/reference/utils/architecture.py:105), causal within
+the request, softmax and accumulation in 32-bit (/root/reference/utils/attention.py:75-96,197);
+output projection (299-300).
+
+The attention kernel works through a list of work items made on the host once a step
+(:func:`build_attention_plan`): an item is 16 rows of (token, head-of-the-group) pairs against
+a contiguous range of keys.  Rows with few tokens and many keys are cut into several items
+whose partial results a second kernel merges by log-sum-exp, the reference's split-KV idea
+(/root/reference/utils/paged_attention.py:78-115).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import numpy as np
+
+from .base import VECTOR, Mixer, PagedKVSpec, ParamSpec, PositionEncoding
+from .linear import Linear
+
+TILE_ROWS = 16          # rows of (token, group head) pairs one wavefront handles (MFMA N dimension)
+KEY_ALIGN = 32          # key ranges of split items start at multiples of this
+MAX_SPLITS = 64
+MIN_KEYS_PER_SPLIT = 64
+TARGET_WAVES = 2048     # wavefronts wanted in flight on 256 CUs
+
+
+def group_tiling(group_size: int):
+    """(heads of a group per tile, tokens per tile, tiles needed to cover the group)."""
+    heads = min(group_size, TILE_ROWS)
+    return heads, TILE_ROWS // heads, -(-group_size // heads)
+
+
+class AttentionPlan:
+    """Host arrays of one step's attention work.
+
+    ``items [n_items, 4] int32``: row, first token of the tile within the row's portion, first
+    key, one past the last key.  ``item_slot [n_items] int32``: index of the partial-result slot,
+    or -1 if the item covers all keys of its rows and writes the output itself.
+    ``merges [n_merges, 4] int32``: row, first token of the tile, first slot, number of slots.
+    """
+
+    def __init__(self, items, item_slot, merges, n_slots):
+        self.items, self.item_slot, self.merges, self.n_slots = items, item_slot, merges, n_slots
+
+
+def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
+                         target_waves: int = TARGET_WAVES) -> AttentionPlan:
+    """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys."""
+    _, tokens_per_tile, group_tiles = group_tiling(group_size)
+    row_len = np.asarray(row_len, dtype=np.int64)
+    row_ctx = np.asarray(row_ctx, dtype=np.int64)
+    tiles_per_row = -(-row_len // tokens_per_tile)
+    waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
+    items, slots, merges = [], [], []
+    n_slots = 0
+    for row in range(len(row_len)):
+        n, ctx = int(row_len[row]), int(row_ctx[row])
+        first_pos = ctx - n
+        for tile in range(int(tiles_per_row[row])):
+            q0 = tile * tokens_per_tile
+            q1 = min(q0 + tokens_per_tile, n)
+            k_end = first_pos + q1                       # last query of the tile sees keys < k_end
+            k_begin = 0 if window is None else max(0, first_pos + q0 - window + 1)
+            n_keys = k_end - k_begin
+            splits = 1
+            if waves_unsplit < target_waves:
+                splits = min(MAX_SPLITS, max(1, target_waves // max(1, waves_unsplit)), max(1, n_keys // MIN_KEYS_PER_SPLIT))
+            if splits <= 1:
+                items.append((row, q0, k_begin, k_end))
+                slots.append(-1)
+                continue
+            start = (k_begin // KEY_ALIGN) * KEY_ALIGN
+            per = -(-(k_end - start) // splits)
+            per = -(-per // KEY_ALIGN) * KEY_ALIGN        # at most `splits` items, each a multiple of KEY_ALIGN keys
+            first_slot = n_slots
+            count = 0
+            while start < k_end:
+                lo, hi = max(start, k_begin), min(start + per, k_end)
+                items.append((row, q0, lo, hi))
+                slots.append(n_slots)
+                n_slots += 1
+                count += 1
+                start += per
+            merges.append((row, q0, first_slot, count))
+    items = np.asarray(items, dtype=np.int32).reshape(-1, 4)
+    merges = np.asarray(merges, dtype=np.int32).reshape(-1, 4)
+    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots)
+
+
+class GQAttention(Mixer):
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
+                 qk_norm_eps: Optional[float] = None, bias: bool = False, out_bias: Optional[bool] = None,
+                 window: Optional[int] = None, scale: Optional[float] = None):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"Number of query heads must be divisible by the number of KV heads: query heads: {n_heads}, KV heads: {n_kv_heads}")
+        self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
+        self.group_size = n_heads // n_kv_heads
+        self.position = position
+        self.qk_norm_eps = qk_norm_eps
+        self.window = window
+        self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
+        self.qkv = Linear(width, ("q_proj", "k_proj", "v_proj"),
+                          (n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * head_dim), bias)
+        self.o = Linear(n_heads * head_dim, ("o_proj",), (width,), bias if out_bias is None else out_bias)
+        self.q_norm_weight = None
+        self.k_norm_weight = None
+
+    def cache_spec(self):
+        return PagedKVSpec(self.n_kv_heads, self.head_dim, self.window)
+
+    def param_specs(self):
+        specs = {**self.qkv.param_specs(), **self.o.param_specs()}
+        if self.qk_norm_eps is not None:
+            specs["q_norm.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
+            specs["k_norm.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
+        return specs
+
+    def assign(self, name, tensor):
+        if name == "q_norm.weight":
+            self.q_norm_weight = tensor
+        elif name == "k_norm.weight":
+            self.k_norm_weight = tensor
+        elif name.startswith("o_proj."):
+            self.o.assign(name, tensor)
+        else:
+            self.qkv.assign(name, tensor)
+
+    def finalize(self):
+        self.qkv.finalize()
+        self.o.finalize()
+
+    def plan_key(self):
+        return ("paged_attention", self.group_size, self.n_kv_heads, self.window)
+
+    def prepare(self, ctx):
+        key = self.plan_key()
+        if ctx.has_plan(key):
+            return
+        plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window)
+        ctx.set_plan(key, {
+            "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "n_items": len(plan.items), "n_merges": len(plan.merges),
+            "n_slots": plan.n_slots,
+        })
+
+    def forward(self, x, ctx, cache):
+        qkv = self.qkv.forward(x, ctx)
+        table = ctx.block_table(cache.group)
+        ctx.ops.qk_norm_rope_kv_write(
+            qkv, cache.keys, cache.values, table, ctx.token_row, ctx.positions,
+            self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
+            self.position.rotary_table(x.device), cache.page_size, self.n_heads, self.n_kv_heads, self.head_dim,
+            cache.writable)
+        out = ctx.empty((x.shape[0], self.n_heads * self.head_dim))
+        ctx.ops.paged_attention(
+            qkv, out, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
+            ctx.get_plan(self.plan_key()), self.scale, self.window, cache.page_size,
+            self.n_heads, self.n_kv_heads, self.head_dim, ctx)
+        return self.o.forward(out, ctx)

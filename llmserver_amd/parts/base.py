@@ -1,0 +1,108 @@
+"""Interfaces of the parts a layer is put together from.
+
+A model is a list of blocks and a list that says in which order they run.  A block arranges
+a mixer (attention here), a feed-forward, norms and a position encoding.  Every part takes its
+sizes and constants as constructor parameters, declares its tensors with :class:`ParamSpec`,
+says what cache it needs with a :class:`CacheSpec`, and runs on a flat batch of tokens described
+by a step context.  No part knows which model it is in.
+
+Shapes used below: ``T`` tokens in the step, ``R`` request rows in the step, ``H`` model width.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, Optional, Tuple
+
+import torch
+
+MATRIX = "matrix"      # follows the compute dtype (bfloat16 for serving, float32 on the 32-bit path)
+VECTOR = "vector"      # small per-channel vectors: always held in float32
+INT_TABLE = "int"      # integer tables: held as int32
+
+
+@dataclasses.dataclass(frozen=True)
+class ParamSpec:
+    """One checkpoint tensor of a part: its shape, how it is stored and how random weights draw it."""
+    shape: Tuple[int, ...]
+    role: str = MATRIX
+    init: str = "normal"          # "normal" | "norm" | "bias" | "zeros"
+    optional: bool = False         # may be absent from the checkpoint
+
+
+@dataclasses.dataclass(frozen=True)
+class PagedKVSpec:
+    """Keys and values of every token, in pages.  ``window`` None keeps all keys; a number keeps
+    only the last ``window`` keys a query can see, so earlier pages can be given back."""
+    n_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclasses.dataclass(frozen=True)
+class StateSpec:
+    """Per-request state of fixed size (one slot per live request)."""
+    shape: Tuple[int, ...]
+    dtype: str = "float32"
+
+
+class Part:
+    """Common base: named tensors in, nothing model-specific."""
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def assign(self, name: str, tensor: torch.Tensor) -> None:
+        raise KeyError(name)
+
+    def finalize(self) -> None:
+        """Called once after all tensors were assigned (fuse, re-lay-out, free the originals)."""
+
+
+class Norm(Part):
+    """Normalisation fused with the residual sum.
+
+    ``add_norm(resid, delta, ctx, rows=None)`` computes ``s = resid + delta`` in 32-bit (``delta``
+    may be None), stores ``s`` back into ``resid`` and returns ``norm(s)``; with ``rows`` (int32
+    device tensor) only those token rows are normalised and returned, ``resid`` is left alone.
+    """
+
+    def add_norm(self, resid, delta, ctx, rows=None):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """How token positions enter a mixer.  ``rotary_table()`` returns the float32 inverse
+    frequencies ``[rotary_dim/2]`` of a rotate-half rotation, or None if nothing is rotated."""
+
+    def rotary_table(self, device) -> Optional[torch.Tensor]:
+        return None
+
+
+class Mixer(Part):
+    """Token mixer: reads and writes its own cache through the view the step gives it."""
+
+    def cache_spec(self):
+        """:class:`PagedKVSpec`, :class:`StateSpec` or None."""
+        return None
+
+    def prepare(self, ctx) -> None:
+        """Stage per-step metadata (host arrays) before the single upload of the step."""
+
+    def forward(self, x, ctx, cache):
+        """``x [T, H]`` normalised input -> ``[T, H]`` update to add to the residual stream."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, ctx):
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of parts.  ``forward(resid, delta, ctx, cache) -> delta'``: ``resid`` is
+    the residual stream (updated in place), ``delta`` the pending update not yet added to it."""
+
+    mixer: Mixer
+
+    def forward(self, resid, delta, ctx, cache):
+        raise NotImplementedError

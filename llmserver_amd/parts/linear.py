@@ -1,0 +1,68 @@
+"""Linear projection ``y = x W^T (+ b)`` with ``W [out, in]`` as checkpoints store it.
+
+The matrix product itself is a library call, as in the reference's engine, which runs every
+projection through the vendor GEMM behind ``nn.Linear`` (/root/reference/utils/attention.py:33-37,
+/root/reference/utils/layers.py:188-191).  Several checkpoint matrices can be stacked along the
+output dimension into one product (/root/reference/utils/attention.py:54-66,
+/root/reference/utils/layers.py:194-203).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Sequence
+
+import torch
+
+from .base import MATRIX, VECTOR, ParamSpec, Part
+
+
+class Linear(Part):
+    """One GEMM over one or several stacked checkpoint matrices.
+
+    ``names``/``out_features`` list the stacked pieces in output order, e.g. ``("q_proj",
+    "k_proj", "v_proj")``.  Tensor names are ``<piece>.weight`` and ``<piece>.bias``.
+    """
+
+    def __init__(self, in_features: int, pieces: Sequence[str], out_features: Sequence[int], bias: bool = False,
+                 out_float32: bool = False):
+        self.in_features = in_features
+        self.pieces = tuple(pieces)
+        self.piece_out = tuple(out_features)
+        self.out_features = sum(out_features)
+        self.has_bias = bias
+        self.out_float32 = out_float32
+        self._w: Dict[str, torch.Tensor] = {}
+        self._b: Dict[str, torch.Tensor] = {}
+        self.weight = None   # [out, in] compute dtype
+        self.bias = None     # [out] float32
+
+    def param_specs(self):
+        specs = {}
+        for piece, n in zip(self.pieces, self.piece_out):
+            specs[f"{piece}.weight"] = ParamSpec((n, self.in_features), MATRIX, "normal")
+            if self.has_bias:
+                specs[f"{piece}.bias"] = ParamSpec((n,), VECTOR, "bias")
+        return specs
+
+    def assign(self, name, tensor):
+        piece, kind = name.rsplit(".", 1)
+        (self._w if kind == "weight" else self._b)[piece] = tensor
+
+    def share_weight(self, tensor: torch.Tensor) -> None:
+        """Use an existing matrix (a tied output head aliases the embedding table, no copy)."""
+        self.weight = tensor
+
+    def finalize(self):
+        if self.weight is None:
+            ws = [self._w[p] for p in self.pieces]
+            self.weight = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0)
+        if self.has_bias and self.bias is None:
+            bs = [self._b[p] for p in self.pieces]
+            self.bias = bs[0] if len(bs) == 1 else torch.cat(bs, dim=0)
+        self._w.clear()
+        self._b.clear()
+
+    def forward(self, x, ctx, out=None):
+        y = ctx.ops.linear(x, self.weight, out=out, out_float32=self.out_float32)
+        if self.bias is not None:
+            ctx.ops.add_bias_(y, self.bias)
+        return y

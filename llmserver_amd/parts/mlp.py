@@ -1,0 +1,36 @@
+"""Gated feed-forward ``down(silu(gate(x)) * up(x))``.
+
+Gate and up are one stacked product, gate first (/root/reference/utils/layers.py:194-218;
+/root/reference/utils/fused_ops.py:59-61, 80-88).  Sigmoid and the product run in 32-bit inside
+the activation kernel.
+"""
+from __future__ import annotations
+
+from .base import FeedForward
+from .linear import Linear
+
+
+class GatedMLP(FeedForward):
+    def __init__(self, width: int, intermediate: int, activation: str = "silu", bias: bool = False):
+        if activation not in ("silu", "swish"):
+            raise ValueError(f"Unsupported activation {activation!r}; supported: ['silu', 'swish']")
+        self.width = width
+        self.intermediate = intermediate
+        self.gate_up = Linear(width, ("gate_proj", "up_proj"), (intermediate, intermediate), bias)
+        self.down = Linear(intermediate, ("down_proj",), (width,), bias)
+
+    def param_specs(self):
+        return {**self.gate_up.param_specs(), **self.down.param_specs()}
+
+    def assign(self, name, tensor):
+        (self.down if name.startswith("down_proj.") else self.gate_up).assign(name, tensor)
+
+    def finalize(self):
+        self.gate_up.finalize()
+        self.down.finalize()
+
+    def forward(self, x, ctx):
+        gate_up = self.gate_up.forward(x, ctx)
+        hidden = ctx.empty((x.shape[0], self.intermediate))
+        ctx.ops.swiglu(gate_up, hidden)
+        return self.down.forward(hidden, ctx)

@@ -1,0 +1,159 @@
+"""A plain, slow implementation of the Qwen3 dense decoder: whole sequences, no cache, one
+function for each part, written from the reference's formulas.  It shares no code with the
+engine (it reads config.json and the safetensors file itself) and is the oracle of the tests.
+Every function cites the lines of the reference it follows.  Arithmetic is float64 by default so
+that the oracle's own rounding is far below the tolerances used against it.
+"""
+from __future__ import annotations
+
+import json
+import math
+import os
+
+import torch
+from safetensors import safe_open
+
+
+def read_folder(folder, dtype=torch.float64):
+    """config.json as a dict and every tensor of model.safetensors, widened to ``dtype``."""
+    with open(os.path.join(folder, "config.json")) as handle:
+        config = json.load(handle)
+    tensors = {}
+    with safe_open(os.path.join(folder, "model.safetensors"), "pt") as handle:
+        for name in handle.keys():
+            tensors[name] = handle.get_tensor(name).to(dtype)
+    return config, tensors
+
+
+def head_dim_of(config):
+    """/root/reference/utils/architecture.py:88"""
+    return config.get("head_dim") or config["hidden_size"] // config["num_attention_heads"]
+
+
+def rope_theta_of(config):
+    """/root/reference/utils/architecture.py:23-30"""
+    parameters = config.get("rope_scaling") or config.get("rope_parameters") or {}
+    theta = config.get("rope_theta")
+    return parameters.get("rope_theta", 10000.0) if theta is None else theta
+
+
+def rms_norm(x, weight, eps):
+    """y = x * rsqrt(mean(x^2, last dim) + eps) * w  (/root/reference/utils/layers.py:133-138)."""
+    variance = x.pow(2).mean(dim=-1, keepdim=True)
+    return weight * (x * torch.rsqrt(variance + eps))
+
+
+def inverse_frequencies(head_dim, theta, dtype=torch.float64):
+    """inv_freq_i = 1 / theta^(2i/d), i = 0..d/2-1  (/root/reference/utils/layers.py:145,158).
+
+    The reference evaluates this in float32; the float32 values are kept so that the oracle's
+    angles are the ones the formula defines at the reference's precision of the table."""
+    indices = torch.arange(0, head_dim, 2, dtype=torch.long)
+    table = 1.0 / (theta ** (indices.to(torch.float32) / head_dim))
+    return table.to(dtype)
+
+
+def rope_cos_sin(positions, head_dim, theta, dtype=torch.float64):
+    """angles = pos * inv_freq, duplicated over both halves  (/root/reference/utils/layers.py:160-164)."""
+    frequencies = positions.to(dtype).unsqueeze(-1) * inverse_frequencies(head_dim, theta, dtype)
+    angles = torch.cat([frequencies, frequencies], dim=-1)
+    return torch.cos(angles), torch.sin(angles)
+
+
+def rotate_half(x):
+    """cat(-x[d/2:], x[:d/2])  (/root/reference/utils/layers.py:166-170)."""
+    half = x.shape[-1] // 2
+    return torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+
+
+def apply_rope(x, cos, sin):
+    """x * cos + rotate_half(x) * sin; x [heads, seq, d], cos/sin [seq, d]  (/root/reference/utils/layers.py:172-177)."""
+    return x * cos.unsqueeze(0) + rotate_half(x) * sin.unsqueeze(0)
+
+
+def causal_attention(q, k, v, scale, window=None):
+    """q [Hq, S, d], k/v [Hkv, S, d] -> [Hq, S, d].
+
+    KV heads repeated per group, scores scaled, causal additive mask, softmax, times V
+    (/root/reference/utils/attention.py:188-198).  ``window`` (not in the reference, which refuses
+    sliding windows at /root/reference/utils/architecture.py:72-76) keeps for query p the keys
+    p-window+1 .. p; None keeps all."""
+    n_q, seq, _ = q.shape
+    group = n_q // k.shape[0]
+    k = torch.repeat_interleave(k, repeats=group, dim=0)
+    v = torch.repeat_interleave(v, repeats=group, dim=0)
+    scores = torch.matmul(q, k.transpose(-1, -2)) * scale
+    place = torch.arange(seq)
+    hidden = place[None, :] > place[:, None]
+    if window is not None:
+        hidden = hidden | (place[None, :] <= place[:, None] - window)
+    scores = scores.masked_fill(hidden.unsqueeze(0), float("-inf"))
+    return torch.matmul(torch.softmax(scores, dim=-1), v)
+
+
+def attention_block(x, tensors, prefix, config, positions, window=None):
+    """Projections, per-head q/k norm before the rotation, rotation, attention, output projection
+    (/root/reference/utils/attention.py:119-128, 155-159, 299-300)."""
+    n_q, n_kv, d = config["num_attention_heads"], config["num_key_value_heads"], head_dim_of(config)
+    seq = x.shape[0]
+
+    def project(name):
+        y = x @ tensors[f"{prefix}.{name}.weight"].T
+        bias = tensors.get(f"{prefix}.{name}.bias")
+        return y if bias is None else y + bias
+
+    q = project("q_proj").view(seq, n_q, d).permute(1, 0, 2)
+    k = project("k_proj").view(seq, n_kv, d).permute(1, 0, 2)
+    v = project("v_proj").view(seq, n_kv, d).permute(1, 0, 2)
+    q = rms_norm(q, tensors[f"{prefix}.q_norm.weight"], config["rms_norm_eps"])
+    k = rms_norm(k, tensors[f"{prefix}.k_norm.weight"], config["rms_norm_eps"])
+    cos, sin = rope_cos_sin(positions, d, rope_theta_of(config), x.dtype)
+    q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+    out = causal_attention(q, k, v, d ** -0.5, window)           # /root/reference/utils/architecture.py:105
+    out = out.permute(1, 0, 2).reshape(seq, n_q * d)
+    y = out @ tensors[f"{prefix}.o_proj.weight"].T
+    bias = tensors.get(f"{prefix}.o_proj.bias")
+    return y if bias is None else y + bias
+
+
+def swiglu_mlp(x, tensors, prefix):
+    """down(silu(gate(x)) * up(x))  (/root/reference/utils/layers.py:210-218)."""
+    gate = x @ tensors[f"{prefix}.gate_proj.weight"].T
+    up = x @ tensors[f"{prefix}.up_proj.weight"].T
+    return (torch.nn.functional.silu(gate) * up) @ tensors[f"{prefix}.down_proj.weight"].T
+
+
+def decoder_layer(h, tensors, index, config, positions, window=None):
+    """h += attn(norm_in(h)); h += mlp(norm_post(h))  (/root/reference/utils/model.py:15-35)."""
+    prefix = f"model.layers.{index}"
+    eps = config["rms_norm_eps"]
+    h = h + attention_block(rms_norm(h, tensors[f"{prefix}.input_layernorm.weight"], eps), tensors,
+                            f"{prefix}.self_attn", config, positions, window)
+    return h + swiglu_mlp(rms_norm(h, tensors[f"{prefix}.post_attention_layernorm.weight"], eps), tensors, f"{prefix}.mlp")
+
+
+def forward(config, tensors, token_ids, windows=None, layer_order=None, first_position=0):
+    """Logits ``[seq, vocab]`` at every position of one whole sequence
+    (/root/reference/utils/model.py:109-158 without cache; tied head rule
+    /root/reference/utils/model_loader.py:56-59).
+
+    ``windows`` (per layer) and ``layer_order`` (which layer runs when) serve the tests' toy
+    arrangements; ``first_position`` shifts all positions."""
+    ids = torch.as_tensor(token_ids, dtype=torch.long)
+    positions = torch.arange(len(ids)) + first_position
+    h = tensors["model.embed_tokens.weight"][ids]
+    order = layer_order if layer_order is not None else range(config["num_hidden_layers"])
+    for index in order:
+        h = decoder_layer(h, tensors, index, config, positions, None if windows is None else windows[index])
+    h = rms_norm(h, tensors["model.norm.weight"], config["rms_norm_eps"])
+    head = tensors["model.embed_tokens.weight"] if config.get("tie_word_embeddings") or "lm_head.weight" not in tensors \
+        else tensors["lm_head.weight"]
+    return h @ head.T
+
+
+def greedy_generate(config, tensors, prompt, new_tokens):
+    """Argmax continuation, recomputing the whole sequence each step (/root/reference/utils/engine.py:295-297)."""
+    tokens = list(prompt)
+    for _ in range(new_tokens):
+        tokens.append(int(torch.argmax(forward(config, tensors, tokens)[-1])))
+    return tokens[len(prompt):]

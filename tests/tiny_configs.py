@@ -1,0 +1,30 @@
+"""The tests' own small configurations of the architecture; they differ in every size and option."""
+from __future__ import annotations
+
+from llmserver_amd.config import Qwen3Config, config_from_dict
+from llmserver_amd.weights import RandomInit
+
+TINY_A = dict(model_type="qwen3", num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
+              head_dim=16, intermediate_size=128, vocab_size=256, rope_theta=10000.0, rms_norm_eps=1e-6,
+              attention_bias=False, tie_word_embeddings=True)
+TINY_A_INIT = RandomInit(seed=11, std=0.02, norm_noise=0.1)
+TINY_A_PAGE = 16
+
+TINY_B = dict(model_type="qwen3", num_hidden_layers=3, hidden_size=96, num_attention_heads=8, num_key_value_heads=2,
+              head_dim=32, intermediate_size=224, vocab_size=384, rope_theta=1e6, rms_norm_eps=1e-5,
+              attention_bias=True, tie_word_embeddings=False)
+TINY_B_INIT = RandomInit(seed=23, std=0.03, norm_noise=0.1, bias_std=0.01)
+TINY_B_PAGE = 8
+
+# A third shape for what A and B do not reach: group of three heads, head size 48, odd vocabulary and width.
+TINY_C = dict(model_type="qwen3", num_hidden_layers=2, hidden_size=72, num_attention_heads=6, num_key_value_heads=2,
+              head_dim=48, intermediate_size=100, vocab_size=301, rope_theta=50000.0, rms_norm_eps=3e-6,
+              attention_bias=False, tie_word_embeddings=False)
+TINY_C_INIT = RandomInit(seed=5, std=0.05, norm_noise=0.2)
+TINY_C_PAGE = 12
+
+CASES = {"A": (TINY_A, TINY_A_INIT, TINY_A_PAGE), "B": (TINY_B, TINY_B_INIT, TINY_B_PAGE), "C": (TINY_C, TINY_C_INIT, TINY_C_PAGE)}
+
+
+def make_config(raw) -> Qwen3Config:
+    return config_from_dict(dict(raw))

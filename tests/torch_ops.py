@@ -1,0 +1,114 @@
+"""Plain torch twins of the HIP kernels, with the same call signatures and the same page layout.
+
+Two uses: each is the reference its kernel is tested against on the GPU, and together they let
+the tests drive the engine's step function, cache and scheduler on a CPU (the product has no CPU
+path of its own; the tests pass this object in place of the kernel namespace).  Arithmetic is
+float32 inside, like the kernels.
+"""
+from __future__ import annotations
+
+import torch
+
+from llmserver_amd.parts.attention import group_tiling  # noqa: F401  (kept for symmetry of imports)
+
+
+class TorchOps:
+    name = "torch"
+
+    def preload(self, head_dims, dtype):
+        pass
+
+    def linear(self, x, weight, out=None, out_float32=False):
+        y = (x.float() @ weight.float().t())
+        y = y if (out_float32 or x.dtype == torch.float32) else y.to(x.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
+    def embedding(self, table, token_ids, out):
+        out.copy_(table[token_ids.long()])
+
+    def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None):
+        if rows is None:
+            total = resid.float()
+            if delta is not None:
+                total = (total + delta.float()).to(resid.dtype)
+                resid.copy_(total)
+                total = total.float()
+        else:
+            index = rows.long()
+            total = resid[index].float()
+            if delta is not None:
+                total = (total + delta[index].float()).to(resid.dtype).float()
+        normed = total * torch.rsqrt(total.pow(2).mean(dim=-1, keepdim=True) + eps) * weight
+        out.copy_(normed.to(out.dtype))
+
+    def swiglu(self, gate_up, out):
+        inter = out.shape[1]
+        gate, up = gate_up[:, :inter].float(), gate_up[:, inter:].float()
+        out.copy_((gate * torch.sigmoid(gate) * up).to(out.dtype))
+
+    def add_bias_(self, y, bias):
+        y.copy_((y.float() + bias).to(y.dtype))
+
+    def qk_norm_rope_kv_write(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, inv_freq,
+                              page_size, n_q, n_kv, head_dim, write_cache=True):
+        n = qkv.shape[0]
+        heads = qkv.view(n, n_q + 2 * n_kv, head_dim)
+        qk = heads[:, :n_q + n_kv].float()
+        if q_weight is not None:
+            weight = torch.cat([q_weight.expand(n_q, -1), k_weight.expand(n_kv, -1)], dim=0)
+            qk = qk * torch.rsqrt(qk.pow(2).mean(dim=-1, keepdim=True) + eps) * weight
+        if inv_freq is not None:
+            angles = positions.float()[:, None] * inv_freq[None, :]
+            cos, sin = torch.cos(angles)[:, None, :], torch.sin(angles)[:, None, :]
+            half = head_dim // 2
+            x1, x2 = qk[..., :half], qk[..., half:]
+            qk = torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
+        heads[:, :n_q] = qk[:, :n_q].to(qkv.dtype)
+        if not write_cache:
+            return
+        pos = positions.long()
+        pages = table.long()[token_row.long(), pos // page_size]
+        slots = pos % page_size
+        keys[pages, :, slots, :] = qk[:, n_q:].to(keys.dtype)
+        values[pages, :, :, slots] = heads[:, n_q + n_kv:].to(values.dtype)
+
+    def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
+                        n_q, n_kv, head_dim, ctx):
+        """Per request row: gather its keys/values through the block table, one softmax over all
+        keys a query may see (no tiles, no splits)."""
+        n = qkv.shape[0]
+        q_all = qkv.view(n, n_q + 2 * n_kv, head_dim)[:, :n_q].float()
+        group = n_q // n_kv
+        for row in range(table.shape[0]):
+            start, length, ctx_len = int(row_start[row]), int(row_len[row]), int(row_ctx[row])
+            first = 0 if not window else max(0, ctx_len - length - window + 1)
+            place = torch.arange(first, ctx_len, device=qkv.device)
+            pages = table[row].long()[place // page_size]
+            k = keys[pages, :, place % page_size, :].float()            # [keys, n_kv, d]
+            v = values[pages, :, :, place % page_size].float()          # [keys, n_kv, d]
+            q = q_all[start:start + length]                               # [len, n_q, d]
+            k = k.repeat_interleave(group, dim=1)
+            v = v.repeat_interleave(group, dim=1)
+            scores = torch.einsum("qhd,khd->hqk", q, k) * scale
+            q_pos = torch.arange(ctx_len - length, ctx_len, device=qkv.device)
+            hidden = place[None, :] > q_pos[:, None]
+            if window:
+                hidden = hidden | (place[None, :] <= q_pos[:, None] - window)
+            scores = scores.masked_fill(hidden[None], float("-inf"))
+            result = torch.einsum("hqk,khd->qhd", torch.softmax(scores, dim=-1), v)
+            out[start:start + length] = result.reshape(length, n_q * head_dim).to(out.dtype)
+
+    def sample(self, logits, temperature, uniform, out):
+        for row in range(logits.shape[0]):
+            temp = float(temperature[row])
+            if not temp > 0.0:
+                out[row] = int(torch.argmax(logits[row]))
+                continue
+            weights = torch.exp((logits[row] - logits[row].max()) / temp)
+            running = torch.cumsum(weights.double(), dim=0)
+            target = float(uniform[row]) * float(running[-1])
+            index = int(torch.searchsorted(running, torch.tensor(target, dtype=torch.float64), right=True))
+            out[row] = min(index, logits.shape[1] - 1)
