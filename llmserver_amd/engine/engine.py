@@ -1,0 +1,312 @@
+"""The engine loop: admission, scheduling, one mixed step, sampling, streaming, finishing.
+
+Constructor options, method names and behaviour follow the reference's ``Engine``
+(/root/reference/utils/engine.py:46-475): ``add_request`` (210-228), ``step`` (437-443),
+``run`` (445-475), ``cancel_request`` (260-277), stop rules (299-314), recompute preemption when
+pages run out (412-435), complete-page prefix caching (193-208, 383-401), bounded history of
+completed requests (230-248).  The difference is the shape of a step: the reference runs a decode
+pass and then padded prefill passes; here the scheduler's plan becomes one flat batch through
+:class:`~llmserver_amd.engine.step.ModelRunner`.
+"""
+from __future__ import annotations
+
+import asyncio
+import json
+import math
+import os
+import time
+import uuid
+from collections import OrderedDict
+from datetime import datetime, timedelta
+from typing import List, Optional
+
+import torch
+
+from ..cache import CacheExhaustedError, CacheManager
+from ..sampling import Sampler, request_uniform
+from .batch import StepEntry
+from .request import (STREAM_END, CompletedRequest, Request, RequestFinishReason, RequestStatus, SamplingParams,
+                      TokenStream)
+from .scheduler import Scheduler
+from .step import ModelRunner
+
+
+def _read_generation_config(model) -> dict:
+    folder = getattr(model, "name", None)
+    if isinstance(folder, str):
+        path = os.path.join(folder, "generation_config.json")
+        if os.path.isfile(path):
+            with open(path) as handle:
+                return json.load(handle)
+    return {}
+
+
+class Engine:
+    def __init__(self, model, tokenizer=None, max_new_tokens=128, max_batch_size=8, max_num_batched_tokens=2048,
+                 max_completed_requests=1000, completed_request_ttl_seconds=3600, prefill_chunk_size=None,
+                 kv_cache_num_blocks=500, kv_cache_block_size=500, stream_text=True, ignore_eos=False,
+                 temperature=0.0, seed=0, enable_prefix_caching=True, ops=None):
+        if max_new_tokens <= 0:
+            raise ValueError(f"max_new_tokens is <= 0: {max_new_tokens}")
+        if max_num_batched_tokens <= 0:
+            raise ValueError(f"max_num_batched_tokens is <= 0: {max_num_batched_tokens}")
+        if max_completed_requests < 0:
+            raise ValueError(f"max_completed_requests cannot be negative: {max_completed_requests}")
+        if completed_request_ttl_seconds < 0:
+            raise ValueError(f"completed_request_ttl_seconds cannot be negative: {completed_request_ttl_seconds}")
+        if temperature < 0:
+            raise ValueError(f"temperature cannot be negative: {temperature}")
+        self.model, self.tokenizer = model, tokenizer
+        self.device, self.dtype = model.device, model.dtype
+        self.max_new_tokens = max_new_tokens
+        self.stream_text = stream_text
+        self.ignore_eos = ignore_eos
+        self.temperature, self.seed = float(temperature), int(seed)
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.max_completed_requests = max_completed_requests
+        self.completed_request_ttl = timedelta(seconds=completed_request_ttl_seconds)
+        self.scheduler = Scheduler(max_batch_size, max_num_batched_tokens, prefill_chunk_size)
+        self.step_profile = {"steps": 0, "decode_steps": 0, "prefill_steps": 0, "schedule_s": 0.0, "step_s": 0.0,
+                             "yield_s": 0.0, "tokens": 0, "prefix_hit_tokens": 0, "preemptions": 0}
+        self.active_requests = {}
+        self.completed_requests = OrderedDict()
+        self.num_blocks, self.block_size = kv_cache_num_blocks, kv_cache_block_size
+        self.kv_cache = CacheManager(model.cache_specs(), kv_cache_block_size, kv_cache_num_blocks,
+                                     num_state_slots=max_batch_size, device=self.device, dtype=self.dtype,
+                                     model_identity=str(getattr(model, "name", "model")))
+        self.enable_prefix_caching = enable_prefix_caching and self.kv_cache.prefix_caching_possible
+        self.runner = ModelRunner(model, self.kv_cache, ops)
+        self.sampler = Sampler(self.runner.ops, self.device)
+        self._requests_added = 0
+        generation = _read_generation_config(model)
+        config = model.config
+
+        def token_id(name):
+            for source in (generation.get(name), getattr(config, name, None), getattr(tokenizer, name, None)):
+                if source is not None:
+                    return source
+            return None
+
+        self.bos_token_id = token_id("bos_token_id")
+        self.pad_token_id = token_id("pad_token_id")
+        eos = token_id("eos_token_id")
+        self.eos_token_ids = set() if eos is None else ({eos} if isinstance(eos, int) else set(eos))
+
+    # -- admission ---------------------------------------------------------------------------
+    def _tokenize(self, prompt: str) -> List[int]:
+        if self.tokenizer is None:
+            raise ValueError("a text prompt needs a tokenizer; pass prompt_token_ids instead")
+        encoded = self.tokenizer(prompt) if callable(self.tokenizer) else self.tokenizer.encode(prompt)
+        if isinstance(encoded, dict) or hasattr(encoded, "keys"):
+            return list(encoded["input_ids"])
+        return list(getattr(encoded, "ids", encoded))
+
+    def add_request(self, prompt=None, prompt_token_ids=None, max_new_tokens=None, temperature=None, seed=None) -> Request:
+        self.prune_completed_requests()
+        if prompt_token_ids is not None:
+            prompt_token_ids = list(prompt_token_ids)
+            if not prompt_token_ids:
+                raise ValueError("prompt_token_ids must not be empty")
+        elif not prompt or prompt.strip() == "":
+            if self.bos_token_id is None:
+                raise ValueError("an empty prompt needs a bos_token_id, and the model folder gives none")
+            prompt_token_ids = [self.bos_token_id]
+        else:
+            prompt_token_ids = self._tokenize(prompt)
+        for token in prompt_token_ids:
+            if not 0 <= token < self.runner.vocab:
+                raise ValueError(f"token id {token} is outside the vocabulary of {self.runner.vocab}")
+        sampling = SamplingParams(self.temperature if temperature is None else float(temperature),
+                                  self.seed + self._requests_added if seed is None else int(seed))
+        self._requests_added += 1
+        request = Request(f"req-{uuid.uuid4()}", prompt, prompt_token_ids, max_new_tokens or self.max_new_tokens,
+                          TokenStream(), sampling)
+        self.active_requests[request.request_id] = request
+        self._open_cache(request)
+        self.scheduler.waiting.append(request)
+        return request
+
+    def _open_cache(self, request: Request) -> None:
+        """Give the request its block tables and state slot and attach cached prefix pages
+        (/root/reference/utils/engine.py:197-208)."""
+        record = self.kv_cache.open(request.request_id)
+        request.block_table = record.tables[0] if record.tables else []
+        if self.enable_prefix_caching:
+            covered = self.kv_cache.share_prefix(request.request_id, request.prompt_token_ids)
+            request.num_computed_tokens += covered
+            self.step_profile["prefix_hit_tokens"] += covered
+
+    # -- history -----------------------------------------------------------------------------
+    def prune_completed_requests(self, now=None):
+        now = now or datetime.now()
+        while self.completed_requests:
+            oldest = next(iter(self.completed_requests.values()))
+            if now - oldest.finished_at < self.completed_request_ttl:
+                break
+            self.completed_requests.popitem(last=False)
+        while len(self.completed_requests) > self.max_completed_requests:
+            self.completed_requests.popitem(last=False)
+
+    def archive_request(self, request):
+        self.active_requests.pop(request.request_id, None)
+        if self.max_completed_requests == 0:
+            return
+        self.completed_requests[request.request_id] = CompletedRequest.from_request(request)
+        self.completed_requests.move_to_end(request.request_id)
+        self.prune_completed_requests()
+
+    def release_request_resources(self, request):
+        if self.kv_cache.has(request.request_id):
+            self.kv_cache.close(request.request_id)
+        request.block_table = []
+
+    def cancel_request(self, request_id) -> bool:
+        self.prune_completed_requests()
+        request = self.active_requests.get(request_id)
+        if request is None or request.status in (RequestStatus.FINISHED, RequestStatus.CANCELLED):
+            return False
+        if request in self.scheduler.waiting:
+            self.scheduler.waiting.remove(request)
+        if request in self.scheduler.running:
+            self.scheduler.running.remove(request)
+        request.cancel()
+        request.output_queue.drain()
+        request.output_queue.put_nowait(STREAM_END)
+        self.release_request_resources(request)
+        self.archive_request(request)
+        return True
+
+    # -- output ------------------------------------------------------------------------------
+    def check_stopping(self, request, token_id):
+        if token_id in self.eos_token_ids and not self.ignore_eos:
+            request.finish(RequestFinishReason.EOS)
+        elif len(request.generated_token_ids) >= request.max_new_tokens:
+            request.finish(RequestFinishReason.LENGTH)
+        else:
+            return
+        request.output_queue.put_nowait(STREAM_END)
+        self.release_request_resources(request)
+        self.archive_request(request)
+
+    def stream_output(self, request):
+        if self.tokenizer is None or not hasattr(self.tokenizer, "decode"):
+            request.output_queue.put_nowait(request.generated_token_ids[-1])
+            return
+        text = self.tokenizer.decode(request.generated_token_ids, skip_special_tokens=True)
+        while text.endswith("�"):        # a character still split across tokens: hold it back
+            text = text[:-1]
+        new_text = text[len(request.emitted_text):]
+        if new_text:
+            request.output_queue.put_nowait(new_text)
+            request.emitted_text = text
+
+    def accept_generated_token(self, request, token_id):
+        request.append_generated_token(token_id)
+        if self.stream_text:
+            self.stream_output(request)
+        self.check_stopping(request, token_id)
+
+    # -- scheduling --------------------------------------------------------------------------
+    def remove_finished_and_cancelled_requests(self):
+        self.scheduler.running[:] = [r for r in self.scheduler.running if r.status not in (RequestStatus.FINISHED, RequestStatus.CANCELLED)]
+
+    def preempt_request(self, request):
+        """Recompute preemption: give everything back, go to the back of the waiting queue
+        (/root/reference/utils/engine.py:412-416)."""
+        self.release_request_resources(request)
+        self.scheduler.running.remove(request)
+        request.preempt_for_compute()
+        self.scheduler.waiting.append(request)
+        self.step_profile["preemptions"] += 1
+
+    def available_blocks(self) -> int:
+        return min(self.kv_cache.available_pages()) if self.kv_cache.groups else 1 << 30
+
+    def schedule_step(self):
+        for request in self.scheduler.waiting:          # a preempted request gets a fresh table (and any cached prefix) back
+            if not self.kv_cache.has(request.request_id):
+                self._open_cache(request)
+        while True:
+            available = self.available_blocks()
+            out = self.scheduler.plan(available, self.block_size)
+            needed = sum(max(0, math.ceil((r.num_computed_tokens + n) / self.block_size) - len(r.block_table))
+                         for r, n in zip(out.prefill_requests, out.prefill_token_counts))
+            needed += sum(max(0, math.ceil((r.num_computed_tokens + 1) / self.block_size) - len(r.block_table))
+                          for r in out.decode_requests)
+            if needed <= available:
+                self.scheduler.commit(out)
+                return out
+            if len(self.scheduler.running) == 1:
+                raise CacheExhaustedError(f"Required blocks {needed} in KV cache exceeds currently free blocks")
+            candidates = [r for r in reversed(self.scheduler.running) if r.block_table]
+            if not candidates:
+                raise CacheExhaustedError(f"Required blocks {needed} in KV cache exceeds currently free blocks")
+            victim = sorted(candidates, key=lambda r: (r.preemption_count, r.waiting_steps))[0]
+            self.preempt_request(victim)
+
+    # -- one step ----------------------------------------------------------------------------
+    def run_scheduled(self, out) -> None:
+        """Turn the plan into one flat batch, run it, sample, and move every request on."""
+        entries, sampled = [], []
+        for request in out.decode_requests:
+            entries.append(StepEntry(request.request_id, [request.generated_token_ids[-1]], [0]))
+            sampled.append(request)
+        prefill = [(r, n) for r, n in zip(out.prefill_requests, out.prefill_token_counts) if r.status == RequestStatus.PREFILL]
+        for request, chunk_len in prefill:
+            start = request.num_computed_tokens
+            tokens = request.prefill_token_ids[start:start + chunk_len]
+            final = start + chunk_len == len(request.prefill_token_ids) and not request.needs_decode_resume
+            entries.append(StepEntry(request.request_id, tokens, [chunk_len - 1] if final else []))
+            if final:
+                sampled.append(request)
+        if not entries:
+            return
+        logits = self.runner.step(entries)
+        temperatures = [r.sampling.temperature for r in sampled]
+        uniforms = [request_uniform(r.sampling.seed, r.num_samples_drawn) if r.sampling.temperature > 0 else 0.0 for r in sampled]
+        token_ids = self.sampler.sample(logits, temperatures, uniforms)
+        self.step_profile["tokens"] += sum(len(e.tokens) for e in entries)
+        for request in out.decode_requests:
+            request.complete_decode()
+        for request, chunk_len in prefill:
+            old = request.num_computed_tokens
+            request.advance_prefill(chunk_len)
+            if self.enable_prefix_caching:
+                self.kv_cache.register_prefix(request.request_id, request.prompt_token_ids, old, request.num_computed_tokens)
+            if request.num_computed_tokens == len(request.prefill_token_ids):
+                request.complete_prefill()
+        for request, token_id in zip(sampled, token_ids):
+            request.num_samples_drawn += 1
+            self.accept_generated_token(request, token_id)
+        self.remove_finished_and_cancelled_requests()
+
+    def step(self) -> bool:
+        out = self.schedule_step()
+        self.run_scheduled(out)
+        self.step_profile["steps"] += 1
+        return bool(self.scheduler.waiting or self.scheduler.running)
+
+    async def run(self):
+        profile, clock = self.step_profile, time.perf_counter
+        while self.scheduler.waiting or self.scheduler.running:
+            t0 = clock()
+            out = self.schedule_step()
+            t1 = clock()
+            self.run_scheduled(out)
+            t2 = clock()
+            await asyncio.sleep(0)          # let other tasks (stream readers) run between steps
+            t3 = clock()
+            profile["steps"] += 1
+            profile["schedule_s"] += t1 - t0
+            profile["step_s"] += t2 - t1
+            profile["yield_s"] += t3 - t2
+            profile["decode_steps"] += bool(out.decode_requests)
+            profile["prefill_steps"] += bool(out.prefill_requests)
+
+    def generate(self, prompts_token_ids, max_new_tokens=None, temperature=None, seed=None) -> List[List[int]]:
+        """Add the prompts, run to the end, return the generated token ids in the prompts' order."""
+        requests = [self.add_request(None, prompt_token_ids=ids, max_new_tokens=max_new_tokens, temperature=temperature,
+                                     seed=None if seed is None else seed + i) for i, ids in enumerate(prompts_token_ids)]
+        while self.step():
+            pass
+        return [list(r.generated_token_ids) for r in requests]
