@@ -223,10 +223,10 @@ class Engine:
         return min(self.kv_cache.available_pages()) if self.kv_cache.groups else 1 << 30
 
     def schedule_step(self):
-        for request in self.scheduler.waiting:          # a preempted request gets a fresh table (and any cached prefix) back
-            if not self.kv_cache.has(request.request_id):
-                self._open_cache(request)
         while True:
+            for request in self.scheduler.waiting:      # a preempted request gets a fresh table (and any cached prefix) back
+                if not self.kv_cache.has(request.request_id):
+                    self._open_cache(request)
             available = self.available_blocks()
             out = self.scheduler.plan(available, self.block_size)
             needed = sum(max(0, math.ceil((r.num_computed_tokens + n) / self.block_size) - len(r.block_table))

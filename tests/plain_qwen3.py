@@ -91,9 +91,13 @@ def causal_attention(q, k, v, scale, window=None):
     return torch.matmul(torch.softmax(scores, dim=-1), v)
 
 
-def attention_block(x, tensors, prefix, config, positions, window=None):
+def attention_block(x, tensors, prefix, config, positions, window=None, kv_store=None, kv_from=None):
     """Projections, per-head q/k norm before the rotation, rotation, attention, output projection
-    (/root/reference/utils/attention.py:119-128, 155-159, 299-300)."""
+    (/root/reference/utils/attention.py:119-128, 155-159, 299-300).
+
+    ``kv_store`` (a dict) receives this layer's rotated keys and values under ``prefix``;
+    ``kv_from`` names a prefix whose stored keys and values are used instead of this layer's own
+    (the tests' toy arrangement in which one layer reads another layer's cache)."""
     n_q, n_kv, d = config["num_attention_heads"], config["num_key_value_heads"], head_dim_of(config)
     seq = x.shape[0]
 
@@ -109,6 +113,11 @@ def attention_block(x, tensors, prefix, config, positions, window=None):
     k = rms_norm(k, tensors[f"{prefix}.k_norm.weight"], config["rms_norm_eps"])
     cos, sin = rope_cos_sin(positions, d, rope_theta_of(config), x.dtype)
     q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+    if kv_store is not None:
+        if kv_from is not None:
+            k, v = kv_store[kv_from]
+        else:
+            kv_store[prefix] = (k, v)
     out = causal_attention(q, k, v, d ** -0.5, window)           # /root/reference/utils/architecture.py:105
     out = out.permute(1, 0, 2).reshape(seq, n_q * d)
     y = out @ tensors[f"{prefix}.o_proj.weight"].T

@@ -1,0 +1,85 @@
+"""Generation through the Python entry point and the engine on the GPU."""
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import model_folder, plain_model, random_tokens
+from tiny_configs import CASES
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("case", ["A", "C"])
+def test_greedy_generation_matches_the_plain_implementation(case):
+    """Workload of tiny configuration A: prompts of 5, 17 and 33 tokens, 8 greedy tokens each."""
+    from llmserver_amd import generate
+    print(f"greedy generation case {case}", flush=True)
+    config, tensors = plain_model(case)
+    prompts = [random_tokens(config["vocab_size"], n, 40 + i) for i, n in enumerate((5, 17, 33))]
+    expected = [plain.greedy_generate(config, tensors, prompt, 8) for prompt in prompts]
+    got = generate(model_folder(case), prompts, max_new_tokens=8, dtype="float32", block_size=CASES[case][2])
+    assert got == expected
+    got_bf16 = generate(model_folder(case), prompts, max_new_tokens=8, dtype="bfloat16", block_size=CASES[case][2])
+    agree = sum(a == b for g, e in zip(got_bf16, expected) for a, b in zip(g, e))
+    assert agree >= 20, (got_bf16, expected)             # bfloat16 may leave the greedy path where two logits nearly tie
+
+
+def test_small_budget_and_few_pages_give_the_same_tokens():
+    """Chunked prefill beside decodes under a token budget of 32, and a pool so small that requests
+    are preempted and recomputed, must not change greedy output (float32)."""
+    from llmserver_amd import Engine, load_model
+    print("generation under a small budget", flush=True)
+    case = "B"
+    config, tensors = plain_model(case)
+    prompts = [random_tokens(config["vocab_size"], n, 60 + i) for i, n in enumerate((1, 40, 64, 100))]
+    expected = [plain.greedy_generate(config, tensors, prompt, 12) for prompt in prompts]
+    model = load_model(model_folder(case), "cuda", "float32")
+    roomy = Engine(model, None, max_new_tokens=12, max_batch_size=4, max_num_batched_tokens=32, kv_cache_num_blocks=64,
+                   kv_cache_block_size=8, ignore_eos=True)
+    assert roomy.generate(prompts) == expected
+    tight = Engine(model, None, max_new_tokens=12, max_batch_size=4, max_num_batched_tokens=32, kv_cache_num_blocks=27,
+                   kv_cache_block_size=8, ignore_eos=True)
+    assert tight.generate(prompts) == expected
+    assert tight.step_profile["preemptions"] > 0
+    tight.kv_cache.check_invariants()
+    assert min(tight.kv_cache.available_pages()) == 27
+
+
+def test_temperature_sampling_is_seeded_per_request():
+    """Workload of tiny configuration B: temperature 0.8 with a fixed seed; a request's tokens do not
+    depend on what shares its batch or on the token budget."""
+    from llmserver_amd import Engine, load_model
+    print("temperature sampling", flush=True)
+    case = "B"
+    vocab = CASES[case][0]["vocab_size"]
+    prompts = [random_tokens(vocab, n, 80 + i) for i, n in enumerate((1, 40, 64, 100))]
+    model = load_model(model_folder(case), "cuda", "float32")
+
+    def run(budget, batch, which):
+        engine = Engine(model, None, max_new_tokens=12, max_batch_size=batch, max_num_batched_tokens=budget,
+                        kv_cache_num_blocks=64, kv_cache_block_size=8, ignore_eos=True, temperature=0.8)
+        requests = [engine.add_request(None, prompts[i], seed=1000 + i) for i in which]
+        while engine.step():
+            pass
+        return {i: r.generated_token_ids for i, r in zip(which, requests)}
+
+    together = run(32, 4, [0, 1, 2, 3])
+    alone = {}
+    for i in range(4):
+        alone.update(run(256, 1, [i]))
+    assert together == alone
+    assert len({tuple(v) for v in together.values()}) == 4
+    other_seed = Engine(model, None, max_new_tokens=12, max_batch_size=1, max_num_batched_tokens=256, kv_cache_num_blocks=64,
+                        kv_cache_block_size=8, ignore_eos=True, temperature=0.8)
+    r = other_seed.add_request(None, prompts[3], seed=5)
+    while other_seed.step():
+        pass
+    assert r.generated_token_ids != together[3]
+
+
+def test_engine_refuses_to_run_without_its_kernels(monkeypatch):
+    """No CPU path: asking for the kernels where no GPU is visible raises instead of falling back."""
+    from llmserver_amd.kernels import KernelLibraryMissing, ops
+    monkeypatch.setattr(torch.cuda, "is_available", lambda: False)
+    with pytest.raises(KernelLibraryMissing):
+        ops.HipOps()

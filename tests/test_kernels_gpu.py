@@ -1,0 +1,256 @@
+"""Each HIP kernel alone against its plain torch twin, at other sizes than the engine's tests use:
+head sizes in steps of 16, groups that are no power of two, widths and vocabularies that are no
+power of two, page sizes from 4 to 500.  Inputs are built so that faults show: a far key that must
+win, a window's edge, pages in scrambled order, a page used again."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from llmserver_amd.parts.attention import build_attention_plan, group_tiling
+from torch_ops import TorchOps
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = {torch.float32: dict(atol=2e-5, rtol=1e-5), torch.bfloat16: dict(atol=2e-2, rtol=2e-2)}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from llmserver_amd.kernels import default_ops
+    return default_ops()
+
+
+class Ctx:
+    def empty(self, shape, dtype=None):
+        return torch.empty(shape, device=DEV, dtype=dtype)
+
+
+def close(a, b, dtype):
+    torch.testing.assert_close(a.float(), b.float(), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [8, 100, 1000, 4104, 9001])
+def test_add_rmsnorm(ops, dtype, width):
+    print(f"add_rmsnorm {dtype} width {width}", flush=True)
+    torch.manual_seed(width)
+    x = (3 * torch.randn(11, width, device=DEV)).to(dtype)
+    delta = torch.randn(11, width, device=DEV).to(dtype)
+    weight = 1 + 0.2 * torch.randn(width, device=DEV)
+    for d in (delta, None):
+        got_x, ref_x = x.clone(), x.clone()
+        got, ref = torch.empty_like(x), torch.empty_like(x)
+        ops.add_rmsnorm(got_x, d, weight, 1e-5, got)
+        TorchOps().add_rmsnorm(ref_x, d, weight, 1e-5, ref)
+        assert torch.equal(got_x, ref_x)                          # the residual sum is rounded once, identically
+        close(got, ref, dtype)
+    rows = torch.tensor([10, 0, 3, 3], device=DEV, dtype=torch.int32)
+    got_x = x.clone()
+    got, ref = (torch.empty(4, width, device=DEV, dtype=dtype) for _ in range(2))
+    ops.add_rmsnorm(got_x, delta, weight, 1e-5, got, rows)
+    TorchOps().add_rmsnorm(x.clone(), delta, weight, 1e-5, ref, rows)
+    assert torch.equal(got_x, x)                                  # selected rows only: the stream is left alone
+    close(got, ref, dtype)
+
+
+def test_rmsnorm_sums_in_32_bit(ops):
+    """Ten thousand bfloat16 ones: a 16-bit running sum would stall at 256."""
+    x = torch.ones(1, 10000, device=DEV, dtype=torch.bfloat16)
+    out = torch.empty_like(x)
+    ops.add_rmsnorm(x, None, torch.ones(10000, device=DEV), 0.0, out)
+    assert torch.equal(out, x)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("inter", [4, 100, 6152, 13001])
+def test_swiglu_embedding_bias(ops, dtype, inter):
+    print(f"swiglu/embedding/bias {dtype} {inter}", flush=True)
+    torch.manual_seed(inter)
+    gate_up = (4 * torch.randn(7, 2 * inter, device=DEV)).to(dtype)
+    got, ref = (torch.empty(7, inter, device=DEV, dtype=dtype) for _ in range(2))
+    ops.swiglu(gate_up, got)
+    TorchOps().swiglu(gate_up, ref)
+    close(got, ref, dtype)
+    table = torch.randn(301, inter, device=DEV).to(dtype)
+    ids = torch.tensor([300, 0, 17, 17, 299], device=DEV, dtype=torch.int32)
+    out = torch.empty(5, inter, device=DEV, dtype=dtype)
+    ops.embedding(table, ids, out)
+    assert torch.equal(out, table[ids.long()])
+    y = torch.randn(7, inter, device=DEV).to(dtype)
+    bias = torch.randn(inter, device=DEV)
+    ref = (y.float() + bias).to(dtype)
+    ops.add_bias_(y, bias)
+    assert torch.equal(y, ref)
+
+
+def make_cache(n_pages, n_kv, page, d, dtype):
+    keys = torch.zeros(n_pages, n_kv, page, d, device=DEV, dtype=dtype)
+    values = torch.zeros(n_pages, n_kv, d, page, device=DEV, dtype=dtype)
+    return keys, values
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (6, 2, 48, 12), (8, 8, 64, 4), (5, 1, 80, 8), (32, 8, 128, 16), (2, 1, 256, 500)])
+def test_qk_norm_rope_kv_write(ops, dtype, n_q, n_kv, d, page):
+    print(f"qk_norm_rope_kv_write {dtype} {n_q}/{n_kv} d{d} page{page}", flush=True)
+    torch.manual_seed(d + n_q)
+    lens, starts = [5, 1, 23], [0, 700, 37]                        # a fresh prompt, a decoded token far out, a later portion
+    rows = len(lens)
+    n_pages = 200 if page < 500 else 8
+    width = max(-(-(s + n) // page) for s, n in zip(starts, lens))
+    table = torch.full((rows, width), -1, dtype=torch.int32)
+    perm = torch.randperm(n_pages)
+    used = 0
+    for r, (s, n) in enumerate(zip(starts, lens)):
+        blocks = -(-(s + n) // page)
+        table[r, :blocks] = perm[used:used + blocks].int()
+        used += blocks
+    positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).int()
+    token_row = torch.cat([torch.full((n,), r) for r, n in enumerate(lens)]).int()
+    tokens = len(positions)
+    qkv = torch.randn(tokens, (n_q + 2 * n_kv) * d, device=DEV).to(dtype)
+    qw, kw = 1 + 0.2 * torch.randn(d, device=DEV), 1 + 0.2 * torch.randn(d, device=DEV)
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, d, 2).float() / d))).to(DEV)
+    table, positions, token_row = table.to(DEV), positions.to(DEV), token_row.to(DEV)
+    for norm, rope, write in ((True, True, True), (False, True, True), (True, False, True), (True, True, False)):
+        got_qkv, ref_qkv = qkv.clone(), qkv.clone()
+        got_k, got_v = make_cache(n_pages, n_kv, page, d, dtype)
+        ref_k, ref_v = make_cache(n_pages, n_kv, page, d, dtype)
+        args = (table, token_row, positions, qw if norm else None, kw if norm else None, 1e-6, inv_freq if rope else None, page, n_q, n_kv, d, write)
+        ops.qk_norm_rope_kv_write(got_qkv, got_k, got_v, *args)
+        TorchOps().qk_norm_rope_kv_write(ref_qkv, ref_k, ref_v, *args)
+        close(got_qkv[:, :n_q * d], ref_qkv[:, :n_q * d], dtype)
+        close(got_k, ref_k, dtype)
+        assert torch.equal(got_v, ref_v)
+        if not write:
+            assert not got_k.any() and not got_v.any()
+
+
+def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, needle=True, seed=0, target_waves=None):
+    """Random q/k/v through both implementations.  Pages are handed out in scrambled order from a
+    pool that first held other data (as if used before).  With ``needle``, one far key per request
+    is made to dominate its first query's softmax."""
+    torch.manual_seed(seed)
+    rows = len(lens)
+    n_pages = sum(-(-c // page) for c in ctxs) + 3
+    keys = (5 * torch.randn(n_pages, n_kv, page, d, device=DEV)).to(dtype)      # stale data of earlier users
+    values = (5 * torch.randn(n_pages, n_kv, d, page, device=DEV)).to(dtype)
+    perm = torch.randperm(n_pages)
+    width = max(-(-c // page) for c in ctxs)
+    table = torch.full((rows, width), -1, dtype=torch.int32)
+    used = 0
+    tokens = sum(lens)
+    qkv = torch.randn(tokens, (n_q + 2 * n_kv) * d, device=DEV).to(dtype)
+    row_start = np.cumsum([0] + list(lens[:-1])).astype(np.int32)
+    for r, c in enumerate(ctxs):
+        blocks = -(-c // page)
+        first = 0 if window is None else max(0, c - lens[r] - window + 1) // page
+        table[r, :blocks] = perm[used:used + blocks].int()
+        used += blocks
+        k = torch.randn(c, n_kv, d, device=DEV)
+        v = torch.randn(c, n_kv, d, device=DEV)
+        if needle and c > 40:
+            far = 3 if window is None else max(0, c - lens[r] - window + 1)       # the oldest key the first query may see
+            q0 = qkv[row_start[r], :d].float()
+            k[far, 0] = 6.0 * q0 / q0.norm() * math.sqrt(d) / max(1.0, float(q0.norm()) / math.sqrt(d))
+            v[far, 0] = 10.0
+        place = torch.arange(c)
+        pages = table[r].long()[place // page].to(DEV)
+        keys[pages, :, (place % page).to(DEV), :] = k.to(dtype)
+        values[pages, :, :, (place % page).to(DEV)] = v.to(dtype)
+        table[r, :first] = -1                                                     # pages a window has passed are gone
+    plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, **({} if target_waves is None else {"target_waves": target_waves}))
+    staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
+              "merges": torch.from_numpy(plan.merges).to(DEV), "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots}
+    t = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
+    got = torch.zeros(tokens, n_q * d, device=DEV, dtype=dtype)
+    ref = torch.zeros_like(got)
+    table = table.to(DEV)
+    scale = d ** -0.5
+    ops.paged_attention(qkv, got, keys, values, table, t(row_start), t(lens), t(ctxs), staged, scale, window, page, n_q, n_kv, d, Ctx())
+    TorchOps().paged_attention(qkv, ref, keys, values, table.clamp(min=0), t(row_start), t(lens), t(ctxs), None, scale, window, page, n_q, n_kv, d, None)
+    torch.cuda.synchronize()
+    assert torch.isfinite(got.float()).all()
+    close(got, ref, dtype)
+    return plan, ref
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 2, 48, 12), (3, 3, 64, 4), (32, 8, 128, 16),
+                                                (5, 1, 80, 20), (20, 1, 16, 16), (16, 1, 112, 64), (2, 1, 256, 500), (7, 7, 96, 32)])
+def test_attention_mixed_batch(ops, dtype, n_q, n_kv, d, page):
+    """Decoded tokens at contexts straddling pages and key steps beside portions of prompts with and without a prefix."""
+    print(f"attention mixed {dtype} {n_q}/{n_kv} d{d} page{page}", flush=True)
+    lens = [1, 1, 1, 17, 40, 2, 1]
+    ctxs = [1, 33, 300, 17, 140, 65, 1025]
+    plan, _ = attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, seed=n_q * d)
+    assert plan.n_slots > 0                                     # long contexts of single tokens were split
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_long_context_splits_and_needle(ops, dtype):
+    print(f"attention long {dtype}", flush=True)
+    plan, ref = attention_case(ops, dtype, 8, 2, 128, 16, [1, 3], [2049, 1500], seed=3)
+    assert len(plan.merges) == 2 and plan.n_slots >= 16
+    assert float(ref[0, :128].float().mean()) > 5.0             # the far key won: its value (10) dominates the first head
+    attention_case(ops, dtype, 8, 2, 128, 16, [1, 3], [2049, 1500], seed=3, target_waves=1)      # same, unsplit
+    attention_case(ops, dtype, 4, 4, 64, 16, [600], [600], seed=4, target_waves=10 ** 6)         # a whole prompt, split to the limit
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 7, 16, 33, 100])
+def test_attention_window_edge(ops, dtype, window):
+    """The oldest key inside the window carries the needle; the one before it must not be read (its page is gone)."""
+    print(f"attention window {window} {dtype}", flush=True)
+    attention_case(ops, dtype, 4, 2, 32, 8, [1, 1, 25, 60, 2], [50, 300, 125, 60, 200], window=window, seed=window)
+    attention_case(ops, dtype, 4, 2, 32, 8, [1, 9], [700, 400], window=window, seed=window, target_waves=10 ** 6)
+
+
+def test_attention_refuses_sizes_it_cannot_take(ops):
+    from llmserver_amd.kernels import build
+    with pytest.raises(ValueError, match="head sizes"):
+        build.attention_module(True, 24)
+    with pytest.raises(ValueError, match="head sizes"):
+        build.attention_module(True, 272)
+    qkv = torch.zeros(1, 4 * 16, device=DEV)
+    out = torch.zeros(1, 2 * 16, device=DEV)
+    keys, values = torch.zeros(2, 1, 6, 16, device=DEV), torch.zeros(2, 1, 16, 6, device=DEV)
+    one = torch.ones(1, dtype=torch.int32, device=DEV)
+    plan = {"items": torch.zeros(1, 4, dtype=torch.int32, device=DEV), "item_slot": -one, "merges": torch.zeros(0, 4, dtype=torch.int32, device=DEV),
+            "n_items": 1, "n_merges": 0, "n_slots": 0}
+    with pytest.raises(ValueError, match="multiple of 4"):
+        ops.paged_attention(qkv, out, keys, values, torch.zeros(1, 1, dtype=torch.int32, device=DEV), 0 * one, one, one, plan, 1.0, None, 6, 2, 1, 16, Ctx())
+    with pytest.raises(TypeError):
+        ops.swiglu(torch.zeros(1, 4, device=DEV, dtype=torch.float16), torch.zeros(1, 2, device=DEV, dtype=torch.float16))
+    with pytest.raises(ValueError, match="GPU"):
+        ops.swiglu(torch.zeros(1, 4), torch.zeros(1, 2))
+
+
+@pytest.mark.parametrize("vocab", [7, 301, 1024, 151936])
+def test_sampling(ops, vocab):
+    print(f"sampling vocab {vocab}", flush=True)
+    torch.manual_seed(vocab)
+    rows = 9
+    logits = (3 * torch.randn(rows, vocab, device=DEV)).float()
+    logits[0, vocab // 2] = logits[0, vocab - 1] = 50.0                         # a tie: the first maximum wins
+    temperature = torch.tensor([0.0, 0.0, 0.8, 0.8, 1.0, 2.5, 0.3, 0.8, 0.8], device=DEV)
+    uniform = torch.tensor([0.5, 0.1, 0.0, 0.999999, 0.5, 0.25, 0.75, 0.5, 0.123], device=DEV)
+    out = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+    ops.sample(logits, temperature, uniform, out)
+    got = out.tolist()
+    assert got[0] == vocab // 2 and got[1] == int(torch.argmax(logits[1]))
+    for row in range(2, rows):
+        weights = torch.exp((logits[row].double() - logits[row].double().max()) / float(temperature[row]))
+        cdf = torch.cumsum(weights, 0) / weights.sum()
+        u, index = float(uniform[row]), got[row]
+        low = float(cdf[index - 1]) if index else 0.0
+        assert 0 <= index < vocab and low - 1e-4 <= u <= float(cdf[index]) + 1e-4, (row, index, low, u, float(cdf[index]))
+    # frequencies follow the distribution
+    few = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]], device=DEV).repeat(4000, 1)
+    draws = torch.empty(4000, dtype=torch.int32, device=DEV)
+    ops.sample(few, torch.full((4000,), 0.7, device=DEV), torch.rand(4000, device=DEV), draws)
+    freq = torch.bincount(draws.long().cpu(), minlength=5).double() / 4000
+    expected = torch.softmax(few[0].double().cpu() / 0.7, 0)
+    assert float((freq - expected).abs().max()) < 0.03

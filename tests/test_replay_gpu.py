@@ -1,0 +1,104 @@
+"""bin/trace_run on the GPU, as a user runs it: the same requests whole, with the last 32 tokens
+decoded one by one, in portions of changing size, and mixed with other requests so that pages are
+used again; in float32 and in bfloat16; every position against the plain implementation."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import traces
+from helpers import model_folder, plain_logits, random_tokens
+from tiny_configs import CASES
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = {"float32": dict(atol=3e-5, rtol=1e-4), "bfloat16": None}
+
+
+def bf16_atol(expected):
+    """bfloat16 keeps 8 bits: a few roundings of that size through two or three layers."""
+    return 0.02 * max(1.0, float(np.abs(expected).max()))
+
+
+def build_trace(case):
+    vocab = CASES[case][0]["vocab_size"]
+    lengths = {"a": 70, "b": 33, "c": 100}
+    mixed_lengths = (5, 17, 33, 70, 100, 41, 64, 1, 90, 130, 20, 77)
+    meta, steps = {}, []
+
+    def add(prefix, requests_meta, maker):
+        requests = {f"{prefix}{rid}": random_tokens(vocab, n, seed) for rid, (n, seed) in requests_meta.items()}
+        meta.update({f"{prefix}{rid}": v for rid, v in requests_meta.items()})
+        part = maker(requests)
+        for step in part:
+            step["step"] = len(steps)
+            steps.append(step)
+        return part
+
+    base = {rid: (n, 100 + i) for i, (rid, n) in enumerate(lengths.items())}
+    add("w-", base, traces.whole)
+    add("t-", base, lambda r: traces.tail_decoded(r, 32))
+    add("p-", base, traces.changing_portions)
+    mixed = add("m-", {f"q{i}": (n, 200 + i) for i, n in enumerate(mixed_lengths)}, lambda r: traces.mixed(r, seed=7, budget_tokens=256))
+    assert max(len(s["entries"]) for s in mixed) >= 3
+    return steps, meta
+
+
+def run_trace(case, dtype, steps, tmp_path, max_tokens, page_size):
+    out = tmp_path / f"out-{case}-{dtype}"
+    command = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_folder(case), "--dtype", dtype,
+               "--out", str(out), "--max-tokens", str(max_tokens), "--page-size", str(page_size)]
+    done = subprocess.run(command, input=traces.to_lines(steps), capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    assert done.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+    return traces.collect(steps, str(out), CASES[case][0]["vocab_size"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case, page_size", [("A", 16), ("B", 8), ("C", 4)])
+def test_all_schedules_match_the_plain_implementation(case, page_size, dtype, tmp_path):
+    print(f"replay case {case} {dtype} page {page_size}", flush=True)
+    steps, meta = build_trace(case)
+    max_tokens = traces.peak_tokens(steps)
+    assert max_tokens <= 256
+    results = run_trace(case, dtype, steps, tmp_path, max_tokens, page_size)
+    assert len(results) == sum(n for n, _ in meta.values())
+    worst = 0.0
+    for (rid, position), logits in results.items():
+        n, seed = meta[rid]
+        expected = plain_logits(case, n, seed)[position].numpy()
+        if dtype == "float32":
+            np.testing.assert_allclose(logits, expected, err_msg=f"{rid} position {position}", **TOLERANCE["float32"])
+        else:
+            error = float(np.abs(logits - expected).max())
+            worst = max(worst, error)
+            assert error <= bf16_atol(expected), f"{rid} position {position}: {error}"
+    # the same request cut differently agrees with itself at least as well as with the oracle
+    for rid in ("a", "b", "c"):
+        n, _ = meta[f"w-{rid}"]
+        for position in range(n):
+            for other in ("t-", "p-"):
+                a, b = results[(f"w-{rid}", position)], results[(f"{other}{rid}", position)]
+                limit = 1e-4 if dtype == "float32" else bf16_atol(a)
+                assert float(np.abs(a - b).max()) <= limit, (rid, other, position)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(dtype, tmp_path):
+    """A one-token prompt decoded for 300 tokens, crossing many pages; and the very first positions."""
+    case = "B"
+    vocab = CASES[case][0]["vocab_size"]
+    tokens = random_tokens(vocab, 301, 31)
+    steps = traces.tail_decoded({"long": tokens}, tail=300)
+    assert len(steps) == 301 and all(len(s["entries"][0]["tokens"]) == 1 for s in steps)
+    results = run_trace(case, dtype, steps, tmp_path, 320, 8)
+    expected = plain_logits(case, 301, 31).numpy()
+    for position in range(301):
+        got = results[("long", position)]
+        if dtype == "float32":
+            np.testing.assert_allclose(got, expected[position], err_msg=f"position {position}", **TOLERANCE["float32"])
+        else:
+            assert float(np.abs(got - expected[position]).max()) <= bf16_atol(expected[position]), position

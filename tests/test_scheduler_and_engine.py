@@ -1,0 +1,317 @@
+"""The scheduler's decisions and the engine's loop on the host (CPU).  The model's forward is
+replaced by a script that returns one-hot logits, the reference's own way of testing its engine
+(/root/reference/tests/test_engine.py:11-55); cache, step builder and sampler are the real ones
+(with the torch twins of the kernels).  Decision vectors marked "reference" are the outcomes the
+reference's tests hold for the same situations."""
+import asyncio
+
+import pytest
+import torch
+
+from llmserver_amd.cache import CacheExhaustedError
+from llmserver_amd.engine import (STREAM_END, Engine, Request, RequestFinishReason, RequestStateError, RequestStatus,
+                                  Scheduler, load_model)
+from helpers import model_folder
+from torch_ops import TorchOps
+
+
+def request(name, prompt=None):
+    return Request(name, "Hello", prompt or [9707], 20)
+
+
+def decoding(name, prompt=None):
+    r = request(name, prompt)
+    r.start_prefill()
+    r.advance_prefill(len(r.prompt_token_ids))
+    r.complete_prefill()
+    return r
+
+
+# ---------------------------------------------------------------- request state machine
+def test_request_walks_through_its_states():
+    r = request("a", [1, 2, 3])
+    with pytest.raises(RequestStateError):
+        r.advance_prefill(1)
+    r.start_prefill()
+    with pytest.raises(ValueError):
+        r.advance_prefill(4)
+    r.advance_prefill(2)
+    with pytest.raises(RequestStateError):
+        r.complete_prefill()
+    r.advance_prefill(1)
+    r.complete_prefill()
+    r.append_generated_token(7)
+    r.complete_decode()
+    assert (r.status, r.num_computed_tokens) == (RequestStatus.DECODING, 4)
+    r.finish("length")
+    assert r.finish_reason == RequestFinishReason.LENGTH
+    with pytest.raises(RequestStateError):
+        r.finish("eos")
+
+
+def test_preempted_decoder_prefills_prompt_plus_all_but_the_last_generated_token():
+    r = decoding("a", [20])
+    r.append_generated_token(60)
+    r.append_generated_token(51)
+    r.preempt_for_compute()
+    assert (r.status, r.num_computed_tokens, r.preemption_count, r.needs_decode_resume) == (RequestStatus.WAITING, 0, 1, True)
+    assert r.prefill_token_ids == [20, 60]                        # reference: tests/test_engine.py:507
+    r.start_prefill()
+    r.advance_prefill(2)
+    r.complete_prefill()
+    assert not r.needs_decode_resume and r.generated_token_ids == [60, 51]
+
+
+# ---------------------------------------------------------------- scheduler decisions
+def plan_commit(scheduler, free=100, page=2):
+    out = scheduler.plan(free, page)
+    scheduler.commit(out)
+    return out
+
+
+def test_budget_is_shared_by_decodes_and_portions():
+    s = Scheduler(max_batch_size=3, max_num_batched_tokens=5)
+    d, first, second = decoding("d"), request("first", [10, 11, 12]), request("second", [20, 21])
+    s.running.append(d)
+    s.waiting.extend([first, second])
+    out = plan_commit(s)
+    assert out.decode_requests == [d] and out.prefill_requests == [first, second]
+    assert out.prefill_token_counts == [3, 1] and out.num_scheduled_tokens == 5          # reference [3, 1]
+    assert s.running == [d, first, second] and not s.waiting
+
+
+def test_prompt_longer_than_the_budget_is_cut_and_computed_tokens_are_not_counted():
+    s = Scheduler(max_batch_size=1, max_num_batched_tokens=3)
+    r = request("long", [10, 11, 12, 13])
+    s.waiting.append(r)
+    assert plan_commit(s).prefill_token_counts == [3]
+    r.advance_prefill(3)
+    assert plan_commit(s).prefill_token_counts == [1]                                      # reference [3] then [1]
+    s = Scheduler(max_batch_size=2, max_num_batched_tokens=4)
+    partial = request("partial", [10, 11, 12, 13, 14])
+    partial.num_computed_tokens = 2                                                        # a cached prefix
+    s.running.append(decoding("d"))
+    s.waiting.append(partial)
+    assert plan_commit(s).prefill_token_counts == [3]
+
+
+def test_chunk_size_caps_each_portion_and_running_prefills_keep_their_slot():
+    s = Scheduler(max_batch_size=2, max_num_batched_tokens=4, prefill_chunk_size=2)
+    a, b = request("a", [1, 2, 3, 4, 5]), request("b", [6, 7, 8, 9, 10])
+    s.waiting.extend([a, b])
+    assert plan_commit(s).prefill_token_counts == [2, 2]
+    a.advance_prefill(2)
+    b.advance_prefill(2)
+    out = plan_commit(s)
+    assert out.prefill_requests == [a, b] and out.prefill_token_counts == [2, 2] and s.running == [a, b]
+
+
+def test_plan_changes_nothing_and_waiting_steps_count_committed_steps():
+    s = Scheduler(max_batch_size=1, max_num_batched_tokens=1)
+    rs = [request(f"r{i}") for i in range(3)]
+    s.waiting.extend(rs)
+    out = s.plan(10, 2)
+    assert list(s.waiting) == rs and not s.running and [r.waiting_steps for r in rs] == [0, 0, 0]
+    s.commit(out)
+    assert [r.waiting_steps for r in rs] == [0, 1, 1]
+    plan_commit(s, 10)
+    s.running.remove(rs[0])
+    plan_commit(s, 10)
+    assert [r.waiting_steps for r in rs] == [0, 2, 3] and s.running == [rs[1]]            # reference [0, 2, 3]
+
+
+def test_admission_keeps_one_spare_page_per_running_request():
+    for free, admitted in ((2, 0), (3, 1)):                                               # reference: headroom cases
+        s = Scheduler(max_batch_size=2, max_num_batched_tokens=2)
+        d = decoding("d", [10, 11])
+        d.block_table = [0]
+        w = request("w", [20])
+        s.running.append(d)
+        s.waiting.append(w)
+        out = s.plan(free, 2)
+        assert out.decode_requests == [d] and out.num_admitted_requests == admitted
+    s = Scheduler(max_batch_size=1, max_num_batched_tokens=5)
+    s.waiting.append(request("long", [1, 2, 3, 4, 5]))
+    assert s.plan(1, 2).prefill_token_counts == [2]                                        # shrunk to the free page
+
+
+def test_nothing_fits_raises_and_bad_limits_are_refused():
+    s = Scheduler(max_batch_size=1, max_num_batched_tokens=1)
+    s.waiting.append(request("w"))
+    with pytest.raises(CacheExhaustedError):
+        s.plan(0, 2)
+    assert s.plan(1, 2).num_admitted_requests == 1
+    empty = Scheduler(max_batch_size=1, max_num_batched_tokens=1).plan(1, 2)
+    assert empty.num_scheduled_tokens == 0
+    for args in ((0, 2), (2, 0), (3, 2)):
+        with pytest.raises(ValueError):
+            Scheduler(*args)
+    with pytest.raises(ValueError):
+        Scheduler(1, 2, prefill_chunk_size=0)
+
+
+# ---------------------------------------------------------------- the engine with a scripted model
+class Script:
+    """Replaces the model's forward: one-hot logits from a list of token ids per call; records the calls."""
+
+    def __init__(self, model, token_ids_by_call):
+        self.tokens, self.calls, self.vocab = list(token_ids_by_call), [], model.head.out_features
+        model.forward = self
+
+    def __call__(self, ctx, caches):
+        self.calls.append({"requests": list(ctx.request_ids), "tokens": [ctx.h_token_ids[s:s + n].tolist() for s, n in zip(ctx.h_row_start, ctx.h_row_len)],
+                           "start": [int(c - n) for c, n in zip(ctx.h_row_ctx, ctx.h_row_len)], "n_out": ctx.n_out})
+        ids = self.tokens.pop(0) if self.tokens else [0] * ctx.n_out
+        assert len(ids) == ctx.n_out, (ids, ctx.n_out)
+        logits = torch.zeros(ctx.n_out, self.vocab)
+        for row, token in enumerate(ids):
+            logits[row, token] = 1.0
+        return logits
+
+
+def scripted_engine(script, **options):
+    model = load_model(model_folder("A"), "cpu", torch.float32)
+    defaults = dict(max_new_tokens=3, max_batch_size=2, max_num_batched_tokens=2, kv_cache_num_blocks=2, kv_cache_block_size=2,
+                    ignore_eos=True, ops=TorchOps())
+    defaults.update(options)
+    engine = Engine(model, None, **defaults)
+    return engine, Script(model, script)
+
+
+def test_recompute_preemption_resumes_without_duplicate_output():
+    """Two one-token prompts, two pages of two tokens: the third step needs a third page.
+    The reference's trace for this situation is tests/test_engine.py:494-523."""
+    engine, script = scripted_engine([[50, 60], [51, 51], [51], [], [51]])
+    first, second = engine.add_request(None, [10]), engine.add_request(None, [20])
+    assert engine.step() and engine.step()
+    assert second.generated_token_ids == [60, 51] and min(engine.kv_cache.available_pages()) == 0
+    assert second.output_queue.drain() == [60, 51]
+    assert engine.step()                                # the later request is the victim; the first decodes and finishes
+    assert first.status == RequestStatus.FINISHED and first.generated_token_ids == [50, 51, 51]
+    assert second.status == RequestStatus.WAITING and second.prefill_token_ids == [20, 60] and second.block_table == []
+    assert engine.step()                                # re-prefill of prompt + generated[:-1]; its last row is not sampled
+    assert second.status == RequestStatus.DECODING and second.num_computed_tokens == 2
+    assert second.generated_token_ids == [60, 51] and second.output_queue.empty()
+    assert script.calls[3]["tokens"] == [[20, 60]] and script.calls[3]["n_out"] == 0
+    assert not engine.step()
+    assert second.generated_token_ids == [60, 51, 51] and second.status == RequestStatus.FINISHED
+    assert script.calls[4]["tokens"] == [[51]] and script.calls[4]["start"] == [2]
+    assert [c["requests"] for c in script.calls] == [[first.request_id, second.request_id]] * 2 + [[first.request_id]] + [[second.request_id]] * 2
+    assert engine.step_profile["preemptions"] == 1
+    engine.kv_cache.check_invariants()
+    assert min(engine.kv_cache.available_pages()) == 2
+
+
+@pytest.mark.parametrize("first, second, victim", [((0, 0), (0, 0), 1), ((0, 0), (1, 0), 0), ((1, 1), (1, 3), 0), ((1, 3), (1, 1), 1)])
+def test_victim_is_least_preempted_then_least_waited_then_latest_admitted(first, second, victim):
+    """reference: tests/test_engine.py:525-545"""
+    engine, _ = scripted_engine([[50, 60], [51, 51]])
+    requests = [engine.add_request(None, [10]), engine.add_request(None, [20])]
+    engine.step()
+    engine.step()
+    for r, (count, steps) in zip(requests, (first, second)):
+        r.preemption_count, r.waiting_steps = count, steps
+    out = engine.schedule_step()
+    assert out.decode_requests == [requests[1 - victim]] and list(engine.scheduler.waiting) == [requests[victim]]
+    assert requests[victim].preemption_count == (first, second)[victim][0] + 1 and requests[victim].block_table == []
+
+
+def test_a_single_request_that_cannot_grow_raises():
+    engine, _ = scripted_engine([[50], [51], [52], [53], [54]], max_new_tokens=8, max_batch_size=1, max_num_batched_tokens=4)
+    engine.add_request(None, [10, 11])
+    engine.step()
+    engine.step()
+    with pytest.raises(CacheExhaustedError):
+        for _ in range(4):
+            engine.step()
+
+
+@pytest.mark.parametrize("length, complete", [(3, 0), (4, 1), (6, 1), (8, 2)])
+def test_only_complete_pages_of_prompt_tokens_become_shareable(length, complete):
+    """reference: tests/test_engine.py:186-194"""
+    engine, _ = scripted_engine([[50]], max_batch_size=1, max_num_batched_tokens=8, kv_cache_num_blocks=4, kv_cache_block_size=4)
+    r = engine.add_request(None, list(range(10, 10 + length)))
+    engine.step()
+    assert engine.kv_cache.groups[0].pool.cacheable == set(r.block_table[:complete])
+
+
+@pytest.mark.parametrize("length, shared", [(4, 0), (8, 1), (10, 2)])
+def test_second_request_reuses_the_longest_cached_prefix(length, shared):
+    """reference: tests/test_engine.py:230-250"""
+    prompt = list(range(10, 10 + length))
+    engine, script = scripted_engine([[50], [51, 60]], max_num_batched_tokens=12, kv_cache_num_blocks=6, kv_cache_block_size=4)
+    first = engine.add_request(None, prompt)
+    engine.step()
+    second = engine.add_request(None, prompt)
+    assert second.block_table == first.block_table[:shared] and second.num_computed_tokens == shared * 4
+    assert all(engine.kv_cache.groups[0].pool.references[p] == 2 for p in second.block_table)
+    engine.step()                       # one mixed step: the first request's decode token beside the second's portion
+    call = script.calls[-1]
+    assert call["requests"] == [first.request_id, second.request_id]
+    index = call["requests"].index(second.request_id)
+    assert call["tokens"][index] == prompt[shared * 4:] and call["start"][index] == shared * 4
+    assert second.generated_token_ids == [60]
+    assert engine.step_profile["prefix_hit_tokens"] == shared * 4
+
+
+def test_stop_rules_stream_and_history():
+    engine, _ = scripted_engine([[7], [9], [9]], max_batch_size=1, max_num_batched_tokens=4, kv_cache_num_blocks=4, ignore_eos=False)
+    engine.eos_token_ids = {9}
+    r = engine.add_request(None, [1, 2, 3])
+    assert engine.step() and not engine.step()
+    assert r.generated_token_ids == [7, 9] and r.finish_reason == RequestFinishReason.EOS
+    assert r.output_queue.drain() == [7, 9, STREAM_END]
+    assert r.request_id in engine.completed_requests and r.request_id not in engine.active_requests
+    assert min(engine.kv_cache.available_pages()) == 4
+    with pytest.raises(ValueError):
+        engine.add_request(None, [])
+    with pytest.raises(ValueError):
+        engine.add_request(None, [10 ** 6])
+    with pytest.raises(ValueError):
+        engine.add_request("text without a tokenizer")
+
+
+def test_cancel_frees_pages_and_ends_the_stream():
+    engine, _ = scripted_engine([[50, 60]], kv_cache_num_blocks=4)
+    a, b = engine.add_request(None, [10]), engine.add_request(None, [20])
+    engine.step()
+    assert engine.cancel_request(b.request_id) and not engine.cancel_request(b.request_id)
+    assert b.status == RequestStatus.CANCELLED and b.output_queue.drain() == [STREAM_END]
+    assert engine.scheduler.running == [a]
+    engine.kv_cache.check_invariants()
+
+
+def test_run_yields_between_steps():
+    engine, _ = scripted_engine([[50, 60], [51, 61], [52, 62]], kv_cache_num_blocks=8)
+    a, b = engine.add_request(None, [10]), engine.add_request(None, [20])
+    ticks = []
+
+    async def watcher():
+        while engine.scheduler.waiting or engine.scheduler.running:
+            ticks.append(len(a.generated_token_ids))
+            await asyncio.sleep(0)
+
+    async def both():
+        await asyncio.gather(engine.run(), watcher())
+
+    asyncio.run(both())
+    assert a.generated_token_ids == [50, 51, 52] and b.generated_token_ids == [60, 61, 62]
+    assert ticks == [1, 2] and engine.step_profile["steps"] == 3      # the watcher ran after the first and second step
+
+
+def test_real_model_under_a_small_budget_and_few_pages_generates_the_same_tokens():
+    """Chunked prefill beside decodes under a token budget of 32, and a pool so small that requests
+    are preempted and recomputed, must not change greedy output (CPU, torch twins of the kernels)."""
+    import plain_qwen3 as plain
+    from helpers import plain_model, random_tokens
+    config, tensors = plain_model("B")
+    prompts = [random_tokens(config["vocab_size"], n, 60 + i) for i, n in enumerate((1, 40, 64, 100))]
+    expected = [plain.greedy_generate(config, tensors, prompt, 12) for prompt in prompts]
+    model = load_model(model_folder("B"), "cpu", torch.float32)
+    for pages in (64, 27):
+        engine = Engine(model, None, max_new_tokens=12, max_batch_size=4, max_num_batched_tokens=32, kv_cache_num_blocks=pages,
+                        kv_cache_block_size=8, ignore_eos=True, ops=TorchOps())
+        assert engine.generate(prompts) == expected
+        engine.kv_cache.check_invariants()
+        assert min(engine.kv_cache.available_pages()) == pages
+    assert engine.step_profile["preemptions"] > 0

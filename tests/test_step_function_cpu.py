@@ -1,0 +1,81 @@
+"""The step function, the cache and the replay driver on the CPU (with the torch twins of the
+kernels): every way of cutting and batching gives the plain implementation's logits."""
+import io
+
+import numpy as np
+import pytest
+import torch
+
+import traces
+from helpers import model_folder, plain_logits, random_tokens
+from llmserver_amd.engine.replay import make_runner, replay
+from tiny_configs import CASES
+from torch_ops import TorchOps
+
+
+def requests_for(case, lengths, seed0=100):
+    vocab = CASES[case][0]["vocab_size"]
+    return {f"q{i}": random_tokens(vocab, n, seed0 + i) for i, n in enumerate(lengths)}, {f"q{i}": (n, seed0 + i) for i, n in enumerate(lengths)}
+
+
+def run(case, steps, max_tokens, tmp_path, page_size=None):
+    page = page_size or CASES[case][2]
+    runner = make_runner(model_folder(case), "float32", max_tokens, page, device="cpu", ops=TorchOps())
+    report = io.StringIO()
+    replay(runner, traces.to_lines(steps).splitlines(), str(tmp_path), report)
+    assert report.getvalue().split() == [w for s in steps for w in ("done", str(s["step"]))]
+    runner.cache.check_invariants()
+    assert not runner.cache.requests and min(runner.cache.available_pages()) == runner.cache.groups[0].pool.num_pages
+    return traces.collect(steps, str(tmp_path), CASES[case][0]["vocab_size"]), runner
+
+
+def check(case, results, meta, atol=3e-5):
+    for (rid, position), logits in results.items():
+        n, seed = meta[rid]
+        expected = plain_logits(case, n, seed)[position].numpy()
+        np.testing.assert_allclose(logits, expected, atol=atol, rtol=1e-4, err_msg=f"{rid} position {position}")
+    assert len(results) == sum(n for n, _ in meta.values())
+
+
+@pytest.mark.parametrize("case", ["A", "B", "C"])
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+def test_every_schedule_matches_the_plain_implementation(case, schedule, tmp_path):
+    lengths = (5, 17, 33, 70, 100, 41, 64, 1, 90, 130, 20, 77) if schedule == "mixed" else (70, 33, 100)
+    requests, meta = requests_for(case, lengths)
+    if schedule == "whole":
+        steps = traces.whole(requests)
+    elif schedule == "tail":
+        steps = traces.tail_decoded(requests, 32)
+    elif schedule == "portions":
+        steps = traces.changing_portions(requests)
+    else:
+        steps = traces.mixed(requests, seed=7, budget_tokens=256)
+        assert max(len(s["entries"]) for s in steps) >= 3
+        assert any(len(e["tokens"]) == 1 for s in steps for e in s["entries"]) and any(len(e["tokens"]) > 8 for s in steps for e in s["entries"])
+    budget = traces.peak_tokens(steps)
+    results, runner = run(case, steps, budget, tmp_path)
+    if schedule == "mixed":
+        assert sum(lengths) > 2 * budget            # more tokens ran through than the pool holds: pages were used again
+    check(case, results, meta)
+
+
+def test_a_step_refuses_what_does_not_fit(tmp_path):
+    runner = make_runner(model_folder("A"), "float32", 64, 16, device="cpu", ops=TorchOps())
+    from llmserver_amd.cache import CacheExhaustedError
+    from llmserver_amd.engine import StepEntry
+    runner.cache.open("a")
+    with pytest.raises(ValueError, match="vocabulary"):
+        runner.step([StepEntry("a", [5, 999], [0])])
+    with pytest.raises(ValueError, match="wanted place"):
+        runner.step([StepEntry("a", [5, 6], [2])])
+    with pytest.raises(ValueError, match="twice"):
+        runner.step([StepEntry("a", [5], []), StepEntry("a", [6], [])])
+    with pytest.raises(ValueError, match="no tokens"):
+        runner.step([StepEntry("a", [], [])])
+    with pytest.raises(KeyError):
+        runner.step([StepEntry("nobody", [5], [])])
+    with pytest.raises(CacheExhaustedError):
+        runner.step([StepEntry("a", [1] * 65, [])])
+    assert runner.cache.record("a").num_computed == 0 and runner.cache.available_pages() == [4]
+    out = runner.step([StepEntry("a", [1, 2, 3], [])])
+    assert out.shape == (0, 256) and runner.cache.record("a").num_computed == 3

@@ -1,0 +1,191 @@
+"""Generality of the parts, shown with toys that live in this file only: a mixer with state of its
+own, layers with different windows, a layer run twice, a layer that reads another layer's cache.
+Each toy is registered as an architecture, written as a random model folder, loaded and stepped
+through the framework's own step function in different cuts, without a change to the framework.
+The CPU variants use the torch twins of the kernels, the GPU variants the HIP kernels."""
+import dataclasses
+import tempfile
+from typing import ClassVar
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import random_tokens
+from llmserver_amd.cache import CacheManager
+from llmserver_amd.config import ModelConfig, field, register_architecture
+from llmserver_amd.engine import ModelRunner, StepEntry, load_model
+from llmserver_amd.models.decoder import DecoderModel, LayerCall
+from llmserver_amd.parts import (MATRIX, GatedMLP, GQAttention, Linear, Mixer, ParamSpec, PreNormBlock, RMSNorm,
+                                 RotaryPosition, StateSpec, TokenEmbedding)
+from llmserver_amd.weights import RandomInit, write_random_model
+from torch_ops import TorchOps
+
+
+# ----------------------------------------------------------------------------- a mixer with state
+class RunningMeanMixer(Mixer):
+    """out_t = W . mean(x_0 .. x_t).  Its state is the running sum, one vector per request."""
+
+    def __init__(self, width):
+        self.width = width
+        self.weight = None
+
+    def cache_spec(self):
+        return StateSpec((self.width,), "float32")
+
+    def param_specs(self):
+        return {"mix.weight": ParamSpec((self.width, self.width), MATRIX, "normal")}
+
+    def assign(self, name, tensor):
+        self.weight = tensor
+
+    def forward(self, x, ctx, cache):
+        out = torch.empty_like(x)
+        for row, (start, n, end) in enumerate(zip(ctx.h_row_start, ctx.h_row_len, ctx.h_row_ctx)):
+            slot = int(ctx.h_state_slots[row])
+            sums = cache.state[slot] + torch.cumsum(x[start:start + n].float(), dim=0)
+            cache.state[slot] = sums[-1]
+            counts = torch.arange(end - n + 1, end + 1, device=x.device, dtype=torch.float32)[:, None]
+            out[start:start + n] = ((sums / counts) @ self.weight.float().t()).to(x.dtype)
+        return out
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyConfig(ModelConfig):
+    MODEL_TYPE: ClassVar[str] = "toy_parts"
+    vocab_size: int = field("vocab_size", int)
+    hidden_size: int = field("hidden_size", int)
+    intermediate_size: int = field("intermediate_size", int)
+    num_attention_heads: int = field("num_attention_heads", int)
+    num_key_value_heads: int = field("num_key_value_heads", int)
+    head_dim: int = field("head_dim", int)
+    rms_norm_eps: float = field("rms_norm_eps", float)
+    rope_theta: float = field("rope_theta", float)
+    layer_kinds: object = field("layer_kinds", object)       # per block: "mean", or an attention window (0 = all keys)
+    layer_order: object = field("layer_order", object)       # per call: [block, cache, writes]
+    tie_word_embeddings: bool = field("tie_word_embeddings", bool, False)
+
+    @property
+    def num_hidden_layers(self):
+        return len(self.layer_kinds)
+
+
+def build_toy(config: ToyConfig) -> DecoderModel:
+    position = RotaryPosition(config.head_dim, config.rope_theta)
+    blocks = []
+    for kind in config.layer_kinds:
+        if kind == "mean":
+            mixer = RunningMeanMixer(config.hidden_size)
+        else:
+            mixer = GQAttention(config.hidden_size, config.num_attention_heads, config.num_key_value_heads, config.head_dim,
+                                position, qk_norm_eps=config.rms_norm_eps, window=kind or None)
+        blocks.append(PreNormBlock(RMSNorm(config.hidden_size, config.rms_norm_eps), mixer,
+                                   RMSNorm(config.hidden_size, config.rms_norm_eps), GatedMLP(config.hidden_size, config.intermediate_size)))
+    order = [LayerCall(b, c, bool(w)) for b, c, w in config.layer_order]
+    head = Linear(config.hidden_size, ("lm_head",), (config.vocab_size,), out_float32=True)
+    return DecoderModel(config, TokenEmbedding(config.vocab_size, config.hidden_size), blocks,
+                        RMSNorm(config.hidden_size, config.rms_norm_eps), head, config.tie_word_embeddings, order)
+
+
+register_architecture("toy_parts", ToyConfig, build_toy, replace=True)
+
+BASE = dict(model_type="toy_parts", vocab_size=97, hidden_size=48, intermediate_size=80, num_attention_heads=4,
+            num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-5, rope_theta=1e4)
+TOYS = {
+    # attention, running mean, attention: a model whose layers have different mixers
+    "state": dict(BASE, layer_kinds=[0, "mean", 0], layer_order=[[0, 0, 1], [1, 1, 1], [2, 2, 1]]),
+    # windows of 9 and 20 keys beside layers that keep all keys: three cache groups
+    "windows": dict(BASE, layer_kinds=[0, 9, 20, 0, 9], layer_order=[[i, i, 1] for i in range(5)]),
+    # block 1 runs twice (shared weights, a cache for each run); the last call reads the cache block 0 wrote
+    "order": dict(BASE, layer_kinds=[0, 0, 0], layer_order=[[0, 0, 1], [1, 1, 1], [1, 2, 1], [2, 0, 0]]),
+}
+
+
+def plain_toy(raw, tensors, tokens):
+    """The toy models over a whole sequence, from the plain implementation's functions."""
+    config = dict(raw, num_hidden_layers=len(raw["layer_kinds"]))
+    ids = torch.as_tensor(tokens)
+    positions = torch.arange(len(tokens))
+    h = tensors["model.embed_tokens.weight"][ids]
+    eps = raw["rms_norm_eps"]
+    stored, cache_owner = {}, {}
+    for block, cache, writes in raw["layer_order"]:
+        prefix = f"model.layers.{block}"
+        kind = raw["layer_kinds"][block]
+        normed = plain.rms_norm(h, tensors[f"{prefix}.input_layernorm.weight"], eps)
+        if kind == "mean":
+            counts = torch.arange(1, len(tokens) + 1, dtype=h.dtype)[:, None]
+            mixed = (torch.cumsum(normed, 0) / counts) @ tensors[f"{prefix}.self_attn.mix.weight"].T
+        else:
+            slot = f"cache{cache}"
+            local = {}
+            mixed = plain.attention_block(normed, tensors, f"{prefix}.self_attn", config, positions, kind or None,
+                                          kv_store=local if writes else stored, kv_from=None if writes else slot)
+            if writes:
+                stored[slot] = local[f"{prefix}.self_attn"]
+        h = h + mixed
+        h = h + plain.swiglu_mlp(plain.rms_norm(h, tensors[f"{prefix}.post_attention_layernorm.weight"], eps), tensors, f"{prefix}.mlp")
+    return plain.rms_norm(h, tensors["model.norm.weight"], eps) @ tensors["lm_head.weight"].T
+
+
+def run_toy(name, device, dtype, ops, tol):
+    raw = TOYS[name]
+    from llmserver_amd.config import config_from_dict
+    folder = tempfile.mkdtemp(prefix=f"llmserver_amd_toy_{name}_")
+    write_random_model(config_from_dict(dict(raw)), folder, RandomInit(seed=9, std=0.08, norm_noise=0.1))
+    model = load_model(folder, device, dtype)
+    _, tensors = plain.read_folder(folder)
+    page = 4
+    cache = CacheManager(model.cache_specs(), page, 36, num_state_slots=2, device=device, dtype=model.dtype)
+    if name == "windows":
+        assert sorted(str(g.spec.window) for g in cache.groups) == ["20", "9", "None"]
+    if name == "state":
+        assert cache.state_specs and not cache.prefix_caching_possible
+    runner = ModelRunner(model, cache, ops)
+    sequences = {"x": random_tokens(97, 75, 1), "y": random_tokens(97, 52, 2)}
+    expected = {rid: plain_toy(raw, tensors, tokens) for rid, tokens in sequences.items()}
+    cuts = {"x": [0, 30, 31, 33, 60, 61, 62, 75], "y": [0, 2, 27, 28, 29, 50, 51, 52]}
+    got = {rid: [] for rid in sequences}
+    for rid in sequences:
+        cache.open(rid)
+    for turn in range(7):                      # both requests in every step: portions beside single tokens
+        entries = []
+        for rid, tokens in sequences.items():
+            a, b = cuts[rid][turn], cuts[rid][turn + 1]
+            entries.append(StepEntry(rid, tokens[a:b], list(range(b - a))))
+        logits = runner.step(entries).double().cpu()
+        row = 0
+        for entry in entries:
+            got[entry.request_id].append(logits[row:row + len(entry.tokens)])
+            row += len(entry.tokens)
+        cache.check_invariants()
+    if name == "windows":
+        tables = cache.record("x").tables
+        window9 = next(g.index for g in cache.groups if g.spec.window == 9)
+        assert tables[window9][:15] == [-1] * 15 and all(p >= 0 for p in tables[window9][17:])   # pages the window passed are gone
+    for rid in sequences:
+        error = float((torch.cat(got[rid]) - expected[rid]).abs().max())
+        assert error < tol, (name, rid, error)
+        cache.close(rid)
+    cache.check_invariants()
+    assert all(g.pool.num_available == g.pool.num_pages for g in cache.groups)
+    # the same request again, whole, through pages that were used before
+    cache.open("again")
+    whole = runner.step([StepEntry("again", sequences["x"], list(range(75)))]).double().cpu()
+    assert float((whole - expected["x"]).abs().max()) < tol
+    cache.close("again")
+
+
+@pytest.mark.parametrize("name", sorted(TOYS))
+def test_toy_on_cpu(name):
+    run_toy(name, "cpu", "float32", TorchOps(), 5e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype, tol", [("float32", 5e-5), ("bfloat16", 6e-2)])
+@pytest.mark.parametrize("name", sorted(TOYS))
+def test_toy_on_gpu(name, dtype, tol):
+    print(f"toy {name} {dtype}", flush=True)
+    from llmserver_amd.kernels import default_ops
+    run_toy(name, "cuda", dtype, default_ops(), tol)
