@@ -37,10 +37,14 @@ constexpr int ND = LSA_ND;          // 16-wide chunks of the head
 constexpr int D = ND * 16;          // head size
 constexpr float NEG_INF = -__builtin_huge_valf();
 
+// Two wavefronts per SIMD while the double-buffered operands of a step fit into 256 registers.
+#define LSA_MIN_WAVES (LSA_ND <= 8 ? 2 : 1)
+
 struct Item { int row, q0, k_begin, k_end; };
 
 struct Geometry {
     int n_q, n_kv, group, gheads, tokens_per_tile, gtiles, page_size, window;
+    unsigned page_magic;      // ceil(2^32 / page_size): key / page_size == mulhi(key, page_magic) for key < 2^32 / page_size
     float scale;
 };
 
@@ -54,7 +58,7 @@ constexpr int KEY_STEP = 16;
 constexpr int NS = D / 16;                   // 16-dim steps (four 16x16x4 MFMAs each)
 #endif
 
-__global__ __launch_bounds__(256) void paged_attention_kernel(
+__global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
     const elem_t* __restrict__ keys, const elem_t* __restrict__ values,
     const int* __restrict__ table, int table_stride,
@@ -108,73 +112,142 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
     float run_max = NEG_INF, run_sum = 0.f;    // run_sum: this lane's share (its keys) of the pair's sum
 
     const int k_begin = item.k_begin, k_end = item.k_end;
-    for (int kt = (k_begin / KEY_STEP) * KEY_STEP; kt < k_end; kt += KEY_STEP) {
-        const bool edge = kt < k_begin || kt + KEY_STEP > k_end;
+
+    // One step of KEY_STEP keys: the K rows and V^T pieces this lane feeds to the MFMAs.  Steps are
+    // loaded one ahead of the step being computed, so the loads of the next step are in flight
+    // while the softmax and the products of this one run.
+    struct Step {
 #if LSA_BF16
-        // ---- scores of two 16-key tiles ----
-        f32x4 st[2];
+        bf16x8 k[2][NS];
+        bf16x4 v[ND][2];
+#else
+        f32x4 k[NS];
+        f32x4 v[ND];
+#endif
+    };
+
+    // Page ids come from the block table 64 logical blocks at a time: lane l of `pages_cur` holds
+    // the page of block 64 * chunk + l, and a lane fetches the entry it needs with a shuffle.  The
+    // next 64 are requested when a chunk is entered, long before they are needed, so that no load
+    // of keys or values ever waits for a table entry.
+    int chunk = -1, pages_cur = 0, pages_next = 0;
+    auto table_chunk = [&](int c) { return row_table[min(64 * c + lane, table_stride - 1)]; };
+    auto enter_chunk = [&](int kt) {            // kt is uniform over the wavefront
+        const int c = (int)__umulhi((unsigned)kt, g.page_magic) >> 6;
+        if (c != chunk) {
+            pages_cur = (chunk >= 0 && c == chunk + 1) ? pages_next : table_chunk(c);
+            chunk = c;
+            pages_next = table_chunk(c + 1);
+        }
+    };
+    // Element offset of key `key` inside the pool: page * page_elems (+ what the caller adds).
+    auto locate = [&](int key, int& slot) {
+        const int block = (int)__umulhi((unsigned)key, g.page_magic);
+        slot = key - block * ps;
+        return (size_t)__shfl(pages_cur, block - 64 * chunk, 64) * page_elems;
+    };
+
+    // Loads of a step are unconditional: a lane whose key lies outside the item's range reads a
+    // key of the step that lies inside it (any valid address will do); scores of such keys are
+    // masked and their values are zeroed before use.
+    auto load_step = [&](Step& f, int kt) {
+        enter_chunk(kt);
+        const int lo = max(k_begin, kt), hi = min(k_end, kt + KEY_STEP) - 1;      // valid keys of this step
+#if LSA_BF16
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
-            const int key = kt + 16 * t2 + col;
-            const bool ok = key >= k_begin && key < k_end;
-            const elem_t* kp = keys;
-            if (ok) kp = keys + (size_t)row_table[key / ps] * page_elems + kv_head_keys + (size_t)(key % ps) * D + 8 * quad;
-            f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+            int slot;
+            const int key = min(max(kt + 16 * t2 + col, lo), hi);
+            const size_t page = locate(key, slot);
+            const elem_t* kp = keys + page + kv_head_keys + (size_t)slot * D + 8 * quad;
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
-                bf16x8 kf = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (ok && 32 * s + 8 * quad < D) kf = *reinterpret_cast<const bf16x8*>(kp + 32 * s);
-                s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], s4, 0, 0, 0);
+                if (32 * s + 32 <= D) {
+                    f.k[t2][s] = *reinterpret_cast<const bf16x8*>(kp + 32 * s);
+                } else {                                   // head size not a multiple of 32: upper half of the last step is zero
+                    bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + 32 * s - (quad >= 2 ? 16 : 0));
+                    if (quad >= 2) kf = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+                    f.k[t2][s] = kf;
+                }
             }
-            st[t2] = s4;
         }
-        // ---- mask, running maximum ----
-        float sv[8];
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            int slot;
+            const int key0 = min(max(kt + 16 * t2 + 4 * quad, lo & ~3), hi & ~3);
+            const size_t page = locate(key0, slot);
+            const elem_t* vp = values + page + kv_head_values + (size_t)col * ps + slot;
+#pragma unroll
+            for (int c = 0; c < ND; ++c) f.v[c][t2] = *reinterpret_cast<const bf16x4*>(vp + (size_t)(16 * c) * ps);
+        }
+#else
+        int slot;
+        const int key = min(max(kt + col, lo), hi);
+        const size_t page = locate(key, slot);
+        const elem_t* kp = keys + page + kv_head_keys + (size_t)slot * D + 4 * quad;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) f.k[s] = *reinterpret_cast<const f32x4*>(kp + 16 * s);
+        const int key0 = min(max(kt + 4 * quad, lo & ~3), hi & ~3);
+        const size_t vpage = locate(key0, slot);
+        const elem_t* vp = values + vpage + kv_head_values + (size_t)col * ps + slot;
+#pragma unroll
+        for (int c = 0; c < ND; ++c) f.v[c] = *reinterpret_cast<const f32x4*>(vp + (size_t)(16 * c) * ps);
+#endif
+    };
+
+    auto compute_step = [&](Step& f, int kt) {
+        const bool edge = kt < k_begin || kt + KEY_STEP > k_end;
+#if LSA_BF16
+        constexpr int NV = 8;
+        float sv[NV];
         float tile_max = NEG_INF;
 #pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2)
+        for (int t2 = 0; t2 < 2; ++t2) {
+            f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < NS; ++s) s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[t2][s], qf[s], s4, 0, 0, 0);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int kpos = kt + 16 * t2 + 4 * quad + r;
                 const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
-                const float v = seen ? st[t2][r] * g.scale : NEG_INF;
+                const float v = seen ? s4[r] * g.scale : NEG_INF;
                 sv[4 * t2 + r] = v;
                 tile_max = fmaxf(tile_max, v);
             }
-#else
-        const int key = kt + col;
-        const bool ok = key >= k_begin && key < k_end;
-        const elem_t* kp = keys;
-        if (ok) kp = keys + (size_t)row_table[key / ps] * page_elems + kv_head_keys + (size_t)(key % ps) * D + 4 * quad;
-        f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            f32x4 kf = {0.f, 0.f, 0.f, 0.f};
-            if (ok) kf = *reinterpret_cast<const f32x4*>(kp + 16 * s);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[e], qf[s][e], s4, 0, 0, 0);
         }
-        float sv[4];
+#else
+        constexpr int NV = 4;
+        float sv[NV];
         float tile_max = NEG_INF;
+        {
+            f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int kpos = kt + 4 * quad + r;
-            const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
-            const float v = seen ? s4[r] * g.scale : NEG_INF;
-            sv[r] = v;
-            tile_max = fmaxf(tile_max, v);
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(f.k[s][e], qf[s][e], s4, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int kpos = kt + 4 * quad + r;
+                const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
+                const float v = seen ? s4[r] * g.scale : NEG_INF;
+                sv[r] = v;
+                tile_max = fmaxf(tile_max, v);
+            }
         }
 #endif
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
         const float new_max = fmaxf(run_max, tile_max);
         const float use_max = new_max == NEG_INF ? 0.f : new_max;
-        const float alpha = __expf(run_max - use_max) ;   // run_max = -inf gives 0
+#if LSA_BF16
+        const float alpha = __expf(run_max - use_max);   // run_max = -inf gives 0
+#else
+        const float alpha = expf(run_max - use_max);
+#endif
         run_max = new_max;
         run_sum *= alpha;
 #pragma unroll
         for (int c = 0; c < ND; ++c) acc[c] *= alpha;
-
 #if LSA_BF16
         bf16x8 pf;
 #pragma unroll
@@ -183,24 +256,13 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
             run_sum += p;
             pf[e] = (bf16_t)p;
         }
-        // ---- output: values of the two 4-key pieces this lane's quad owns ----
-        const elem_t* vp[2];
-        bool vok[2];
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-            const int key0 = kt + 16 * t2 + 4 * quad;
-            vok[t2] = key0 + 4 > k_begin && key0 < k_end;
-            vp[t2] = values;
-            if (vok[t2]) vp[t2] = values + (size_t)row_table[key0 / ps] * page_elems + kv_head_values + (size_t)col * ps + key0 % ps;
-        }
 #pragma unroll
         for (int c = 0; c < ND; ++c) {
             bf16x8 vf;
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
-                bf16x4 piece = {0, 0, 0, 0};
-                if (vok[t2]) piece = *reinterpret_cast<const bf16x4*>(vp[t2] + (size_t)(16 * c) * ps);
-                if (edge) {
+                bf16x4 piece = f.v[c][t2];
+                if (edge) {                      // keys outside the item's range may hold anything: keep them out of the sum
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int kpos = kt + 16 * t2 + 4 * quad + r;
@@ -219,23 +281,42 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
             pv[r] = expf(sv[r] - use_max);
             run_sum += pv[r];
         }
-        const int key0 = kt + 4 * quad;
-        const bool vok = key0 + 4 > k_begin && key0 < k_end;
-        const elem_t* vp = values;
-        if (vok) vp = values + (size_t)row_table[key0 / ps] * page_elems + kv_head_values + (size_t)col * ps + key0 % ps;
 #pragma unroll
         for (int c = 0; c < ND; ++c) {
-            f32x4 vf = {0.f, 0.f, 0.f, 0.f};
-            if (vok) vf = *reinterpret_cast<const f32x4*>(vp + (size_t)(16 * c) * ps);
+            f32x4 vf = f.v[c];
             if (edge) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if (key0 + r < k_begin || key0 + r >= k_end) vf[r] = 0.f;
+                    if (kt + 4 * quad + r < k_begin || kt + 4 * quad + r >= k_end) vf[r] = 0.f;
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[r], pv[r], acc[c], 0, 0, 0);
         }
 #endif
+    };
+
+    if (k_begin < k_end) {
+        Step a, b;
+        int kt = (k_begin / KEY_STEP) * KEY_STEP;
+        int steps = (k_end - kt + KEY_STEP - 1) / KEY_STEP;
+        load_step(a, kt);
+        // Steady state without a branch between the loads of one step and the products of the
+        // step before it, so that the wait for operands leaves the newer loads in flight.
+        while (steps >= 3) {
+            load_step(b, kt + KEY_STEP);
+            compute_step(a, kt);
+            load_step(a, kt + 2 * KEY_STEP);
+            compute_step(b, kt + KEY_STEP);
+            kt += 2 * KEY_STEP;
+            steps -= 2;
+        }
+        if (steps == 2) {
+            load_step(b, kt + KEY_STEP);
+            compute_step(a, kt);
+            compute_step(b, kt + KEY_STEP);
+        } else {
+            compute_step(a, kt);
+        }
     }
 
     run_sum += __shfl_xor(run_sum, 16, 64);
@@ -271,40 +352,47 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
 // Merge the partial slots of a tile: out = sum_s w_s acc_s / sum_s w_s l_s, w_s = exp(m_s - max m).
 struct Merge { int row, q0, first_slot, n_slots; };
 
-__global__ __launch_bounds__(256) void merge_kernel(
+__global__ __launch_bounds__(128) void merge_kernel(
     elem_t* __restrict__ out, const int* __restrict__ row_start, const int* __restrict__ row_len,
     const Merge* __restrict__ merges, const float* __restrict__ part_acc, const float* __restrict__ part_ml, Geometry g) {
-    __shared__ float weight[64 * 16];      // [slot][pair], at most 64 slots
-    __shared__ float inv_sum[16];
+    // One block per (tile, KV head, pair).  First the slots' weights (a thread per slot), then
+    // the weighted sum (a thread per output dimension, slots unrolled so their loads overlap).
+    __shared__ float weight[64];
+    __shared__ float inv_total;
     const Merge m = merges[blockIdx.x];
+    const int col = blockIdx.z;
     const int kv_head = blockIdx.y / g.gtiles, gtile = blockIdx.y % g.gtiles;
-    const int n = row_len[m.row], token0 = row_start[m.row] + m.q0;
-    if (threadIdx.x < 16) {
-        const int col = threadIdx.x;
-        float top = NEG_INF;
-        for (int s = 0; s < m.n_slots; ++s)
-            top = fmaxf(top, part_ml[(((size_t)(m.first_slot + s) * gridDim.y + blockIdx.y) * 16 + col) * 2]);
-        float total = 0.f;
-        for (int s = 0; s < m.n_slots; ++s) {
-            const size_t base = (((size_t)(m.first_slot + s) * gridDim.y + blockIdx.y) * 16 + col) * 2;
-            const float w = top == NEG_INF ? 0.f : expf(part_ml[base] - top);
-            weight[s * 16 + col] = w;
-            total += w * part_ml[base + 1];
+    const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
+    if (pair_token >= g.tokens_per_tile || m.q0 + pair_token >= row_len[m.row] || pair_head_in_group >= g.group) return;
+    const size_t stride = (size_t)gridDim.y * 16;                       // pairs per slot
+    const size_t base = ((size_t)m.first_slot * gridDim.y + blockIdx.y) * 16 + col;
+    if (threadIdx.x < 64) {
+        const int s = threadIdx.x;
+        float mx = NEG_INF, sum = 0.f;
+        if (s < m.n_slots) {
+            mx = part_ml[(base + s * stride) * 2];
+            sum = part_ml[(base + s * stride) * 2 + 1];
         }
-        inv_sum[col] = total > 0.f ? 1.f / total : 0.f;
+        const float top = wave_max(mx);
+        const float w = mx == NEG_INF ? 0.f : expf(mx - top);
+        weight[s] = w;
+        const float total = wave_sum(w * sum);
+        if (s == 0) inv_total = total > 0.f ? 1.f / total : 0.f;
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < 16 * D; e += blockDim.x) {
-        const int col = e / D, dim = e % D;
-        const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
-        if (pair_token >= g.tokens_per_tile || m.q0 + pair_token >= n || pair_head_in_group >= g.group) continue;
+    const int head = kv_head * g.group + pair_head_in_group;
+    elem_t* o = out + ((size_t)(row_start[m.row] + m.q0 + pair_token) * g.n_q + head) * D;
+    const float* acc = part_acc + base * D;
+    for (int dim = threadIdx.x; dim < D; dim += blockDim.x) {
         float total = 0.f;
-        for (int s = 0; s < m.n_slots; ++s) {
-            const float w = weight[s * 16 + col];
-            if (w != 0.f) total += w * part_acc[(((size_t)(m.first_slot + s) * gridDim.y + blockIdx.y) * 16 + col) * D + dim];
+        int s = 0;
+        for (; s + 4 <= m.n_slots; s += 4) {
+            const float a0 = acc[(size_t)(s + 0) * stride * D + dim], a1 = acc[(size_t)(s + 1) * stride * D + dim];
+            const float a2 = acc[(size_t)(s + 2) * stride * D + dim], a3 = acc[(size_t)(s + 3) * stride * D + dim];
+            total += weight[s] * a0 + weight[s + 1] * a1 + weight[s + 2] * a2 + weight[s + 3] * a3;
         }
-        const int head = kv_head * g.group + pair_head_in_group;
-        out[((size_t)(token0 + pair_token) * g.n_q + head) * D + dim] = (elem_t)(total * inv_sum[col]);
+        for (; s < m.n_slots; ++s) total += weight[s] * acc[(size_t)s * stride * D + dim];
+        o[dim] = (elem_t)(total * inv_total);
     }
 }
 
@@ -317,14 +405,15 @@ LSA_EXPORT int lsa_paged_attention(
     Geometry g;
     g.n_q = n_q; g.n_kv = n_kv; g.group = n_q / n_kv; g.gheads = gheads; g.tokens_per_tile = tokens_per_tile;
     g.gtiles = gtiles; g.page_size = page_size; g.window = window; g.scale = scale;
+    g.page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     dim3 grid((n_items + 3) / 4, n_kv * gtiles);
     paged_attention_kernel<<<grid, 256, 0, stream>>>(
         (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
         row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g);
     int err = (int)hipGetLastError();
     if (err || n_merges <= 0) return err;
-    dim3 mgrid(n_merges, n_kv * gtiles);
-    merge_kernel<<<mgrid, 256, 0, stream>>>((elem_t*)out, row_start, row_len, (const Merge*)merges, part_acc, part_ml, g);
+    dim3 mgrid(n_merges, n_kv * gtiles, 16);
+    merge_kernel<<<mgrid, 128, 0, stream>>>((elem_t*)out, row_start, row_len, (const Merge*)merges, part_acc, part_ml, g);
     LSA_LAUNCH_CHECK();
 }
 

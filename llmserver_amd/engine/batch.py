@@ -32,6 +32,7 @@ class Staging:
         self.device = torch.device(device)
         self.capacity = 0
         self.used = 0
+        self._copied = None       # event after the last upload: the host buffer is free again once it has passed
         self._grow(capacity)
 
     def _grow(self, capacity: int):
@@ -41,9 +42,14 @@ class Staging:
         self.dev = torch.empty(capacity, dtype=torch.int32, device=self.device) if on_gpu else self.host
         self.capacity = capacity
 
-    def reset(self, needed: int = 0):
+    def reset(self, needed: int = 0, may_grow: bool = True):
+        if self._copied is not None:
+            self._copied.synchronize()
+            self._copied = None
         self.used = 0
         if needed > self.capacity:
+            if not may_grow:
+                raise RuntimeError("staging buffer of a captured step is too small")
             self._grow(max(needed, 2 * self.capacity))
 
     def stage(self, array: np.ndarray) -> torch.Tensor:
@@ -60,6 +66,8 @@ class Staging:
     def upload(self):
         if self.dev is not self.host and self.used:
             self.dev[:self.used].copy_(self.host[:self.used], non_blocking=True)
+            self._copied = torch.cuda.Event()
+            self._copied.record()
 
 
 class StepContext:
@@ -69,6 +77,7 @@ class StepContext:
         self.ops, self.device, self.dtype, self.staging = ops, torch.device(device), dtype, staging
         self._plans: Dict[object, dict] = {}
         self._tables: Dict[int, torch.Tensor] = {}
+        self.static_max_keys: Optional[int] = None      # set when the step's array shapes must be fixed (graph capture)
 
     # -- building ------------------------------------------------------------------------
     def fill(self, token_ids, positions, token_row, row_start, row_len, row_ctx, logit_idx, tables: List[np.ndarray],
@@ -94,7 +103,8 @@ class StepContext:
         if self.h_state_slots is not None:
             arrays.append(self.h_state_slots)
         needed = sum(a.size + 4 for a in arrays) + sum(plan[name].size + 4 for plan, name in plan_arrays)
-        self.staging.reset(needed)
+        self.staging.reset(needed, may_grow=self.static_max_keys is None)
+        self.layout = tuple(a.shape for a in arrays) + tuple(plan[name].shape for plan, name in plan_arrays)
         stage = self.staging.stage
         self.token_ids, self.positions, self.token_row = stage(self.h_token_ids), stage(self.h_positions), stage(self.h_token_row)
         self.row_start, self.row_len, self.row_ctx = stage(self.h_row_start), stage(self.h_row_len), stage(self.h_row_ctx)

@@ -5,10 +5,18 @@ portions of prompts beside single decoded tokens, cut anywhere.  The reference r
 forward per engine step, padded prefill batches and a decode batch
 (/root/reference/utils/engine.py:437-443, /root/reference/utils/model.py:76-158); here there is
 one pass, and one code path serves generation, the benchmark and trace replay.
+
+A step that brings one token per request is launch-bound, so it is captured once into a HIP
+graph per (rows, block-table width, wanted rows) and replayed afterwards: the kernels read
+everything that changes from the staged arrays, whose addresses and shapes stay the same.  The
+reference replays its decode pass from a CUDA graph in the same way
+(/root/reference/utils/cuda_graph.py:51-99).
 """
 from __future__ import annotations
 
-from typing import List, Sequence
+import warnings
+from collections import OrderedDict
+from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -16,9 +24,17 @@ import torch
 from ..cache.manager import CacheManager
 from .batch import Staging, StepContext, StepEntry
 
+TABLE_WIDTH_STEP = 64      # captured steps serve block tables up to the next multiple of this many pages
+MAX_GRAPHS = 12
+
+
+class _CapturedStep:
+    def __init__(self, graph, logits, layout, staging):
+        self.graph, self.logits, self.layout, self.staging = graph, logits, layout, staging
+
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager, ops=None):
+    def __init__(self, model, cache: CacheManager, ops=None, use_graphs: Optional[bool] = None):
         if ops is None:
             from ..kernels import default_ops
             ops = default_ops()
@@ -27,8 +43,15 @@ class ModelRunner:
         self._staging = [Staging(self.device), Staging(self.device)]
         self._flip = 0
         self.vocab = model.head.out_features
+        graph_safe = all(block.mixer.graph_safe for block in model.blocks) and not cache.state_specs
+        if use_graphs is None:
+            use_graphs = self.device.type == "cuda" and getattr(ops, "name", "") == "hip"
+        self.use_graphs = bool(use_graphs and graph_safe)
+        self._graphs: "OrderedDict[tuple, _CapturedStep]" = OrderedDict()
+        self.graph_replays = 0
 
-    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+    def build_context(self, entries: Sequence[StepEntry], staging: Optional[Staging] = None,
+                      table_width: Optional[int] = None) -> StepContext:
         """Check the entries against the cache, allocate their pages, lay out the flat batch."""
         if not entries:
             raise ValueError("a step needs at least one entry")
@@ -60,16 +83,13 @@ class ModelRunner:
             token_ids.extend(tokens)
             positions.extend(range(start, start + len(tokens)))
             token_row.extend([row] * len(tokens))
-        taken = []
-        try:
-            for entry, ctx_len in zip(entries, row_ctx):
-                self.cache.ensure(entry.request_id, ctx_len)
-                taken.append(entry.request_id)
-        except Exception:
-            raise
+        for entry, ctx_len in zip(entries, row_ctx):
+            self.cache.ensure(entry.request_id, ctx_len)
         tables = []
         for group in self.cache.groups:
             width = max(1, max(len(self.cache.record(rid).tables[group.index]) for rid in request_ids))
+            if table_width is not None:
+                width = table_width
             table = np.full((len(entries), width), -1, dtype=np.int32)
             for row, rid in enumerate(request_ids):
                 pages = self.cache.record(rid).tables[group.index]
@@ -78,18 +98,69 @@ class ModelRunner:
         slots = None
         if self.cache.state_specs:
             slots = np.asarray([self.cache.record(rid).state_slot for rid in request_ids], dtype=np.int32)
-        self._flip ^= 1
-        ctx = StepContext(self.ops, self.device, self.dtype, self._staging[self._flip])
+        if staging is None:
+            self._flip ^= 1
+            staging = self._staging[self._flip]
+        ctx = StepContext(self.ops, self.device, self.dtype, staging)
         ctx.fill(token_ids, positions, token_row, row_start, row_len, row_ctx, logit_idx, tables, slots, request_ids)
         return ctx
 
+    # -- captured single-token steps ---------------------------------------------------------
+    def _graph_key(self, entries: Sequence[StepEntry]):
+        if not self.use_graphs or any(len(entry.tokens) != 1 for entry in entries):
+            return None
+        blocks = 1
+        for entry in entries:
+            record = self.cache.requests.get(entry.request_id)
+            if record is None:
+                return None
+            blocks = max(blocks, -(-(record.num_computed + 1) // self.cache.page_size))
+        width = -(-blocks // TABLE_WIDTH_STEP) * TABLE_WIDTH_STEP
+        return (len(entries), width, sum(len(entry.want) for entry in entries))
+
+    def _step_captured(self, entries, key) -> torch.Tensor:
+        captured = self._graphs.get(key)
+        staging = captured.staging if captured is not None else Staging(self.device, capacity=4096)
+        ctx = self.build_context(entries, staging=staging, table_width=key[1])
+        ctx.static_max_keys = key[1] * self.cache.page_size
+        self.model.prepare(ctx)
+        if captured is None:
+            ctx.static_max_keys = None           # the first upload may size the staging buffer
+            ctx.upload()
+            ctx.static_max_keys = key[1] * self.cache.page_size
+            logits = self.model.forward(ctx, self.cache)              # this step's result, run eagerly
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_logits = self.model.forward(ctx, self.cache)   # recorded, not run
+            self._graphs[key] = _CapturedStep(graph, static_logits, ctx.layout, staging)
+            while len(self._graphs) > MAX_GRAPHS:
+                self._graphs.popitem(last=False)
+            return logits
+        self._graphs.move_to_end(key)
+        ctx.upload()
+        if ctx.layout != captured.layout:
+            warnings.warn("a captured step met arrays of another shape; running it eagerly")
+            return self.model.forward(ctx, self.cache)
+        captured.graph.replay()
+        self.graph_replays += 1
+        return captured.logits
+
     @torch.inference_mode()
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Run one step; returns float32 logits ``[wanted, vocab]`` in the order of the entries and their ``want``."""
-        ctx = self.build_context(entries)
-        self.model.prepare(ctx)
-        ctx.upload()
-        logits = self.model.forward(ctx, self.cache)
-        for rid, ctx_len in zip(ctx.request_ids, ctx.h_row_ctx):
-            self.cache.advance(rid, int(ctx_len))
+        """Run one step; returns float32 logits ``[wanted, vocab]`` in the order of the entries and their ``want``.
+
+        The tensor a captured step returns is overwritten by the next step of the same shape."""
+        key = self._graph_key(entries)
+        if key is not None:
+            logits = self._step_captured(entries, key)
+            ctx_rows = [(entry.request_id, self.cache.record(entry.request_id).num_computed + 1) for entry in entries]
+        else:
+            ctx = self.build_context(entries)
+            self.model.prepare(ctx)
+            ctx.upload()
+            logits = self.model.forward(ctx, self.cache)
+            ctx_rows = list(zip(ctx.request_ids, (int(c) for c in ctx.h_row_ctx)))
+        for rid, ctx_len in ctx_rows:
+            self.cache.advance(rid, ctx_len)
         return logits

@@ -25,7 +25,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HEAD_DIMS = tuple(range(16, 257, 16))
-BASE_MODULES = ("elementwise", "rope_kv", "sampling")
+BASE_MODULES = ("elementwise", "rope_kv", "sampling", "gemm")
 
 
 class KernelBuildError(RuntimeError):

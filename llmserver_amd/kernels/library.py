@@ -20,7 +20,7 @@ _SIGNATURES = {
                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_attention_head_dim": [],
     "lsa_attention_is_bf16": [],
-    "lsa_gemm_skinny": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+    "lsa_gemm_skinny": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

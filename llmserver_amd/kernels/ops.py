@@ -15,6 +15,7 @@ from ..parts.attention import group_tiling
 from . import build, library
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+SKINNY_GEMM_ROWS = 8        # up to this many rows the hand-written weight-streaming product beats the library (measured)
 
 
 def _code(tensor: torch.Tensor) -> int:
@@ -63,7 +64,9 @@ class HipOps:
         self._elementwise = library.load("elementwise")
         self._rope_kv = library.load("rope_kv")
         self._sampling = library.load("sampling")
+        self._gemm = library.load("gemm")
         self._attention = {}
+        self.skinny_rows = SKINNY_GEMM_ROWS
 
     @staticmethod
     def required_modules(head_dims, dtype):
@@ -80,6 +83,17 @@ class HipOps:
         """``x [T, in] @ weight[out, in]^T``; float32 result if asked (the output head)."""
         if x.shape[1] != weight.shape[1]:
             raise ValueError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
+        rows, width = x.shape
+        if x.dtype == torch.bfloat16 and 0 < rows <= self.skinny_rows and width % 8 == 0:
+            # Few rows: the product is a stream over the weights; the hand-written kernel reads them once at HBM rate.
+            _check(x, "x", torch.bfloat16)
+            _check(weight, "weight", torch.bfloat16)
+            if out is None or out_float32:
+                out = torch.empty((rows, weight.shape[0]), device=x.device, dtype=torch.float32 if out_float32 else torch.bfloat16)
+            _check(out, "out", None, (rows, weight.shape[0]))
+            _launched(self._gemm.lsa_gemm_skinny(1 if out_float32 else 0, _ptr(x), _ptr(weight), _ptr(out), rows,
+                                                 weight.shape[0], width, _stream()), "gemm_skinny")
+            return out
         if out_float32 and x.dtype != torch.float32:
             return torch.mm(x, weight.t(), out_dtype=torch.float32)
         return torch.mm(x, weight.t(), out=out) if out is not None else torch.mm(x, weight.t())

@@ -30,8 +30,8 @@ from .linear import Linear
 TILE_ROWS = 16          # rows of (token, group head) pairs one wavefront handles (MFMA N dimension)
 KEY_ALIGN = 32          # key ranges of split items start at multiples of this
 MAX_SPLITS = 64
-MIN_KEYS_PER_SPLIT = 64
-TARGET_WAVES = 2048     # wavefronts wanted in flight on 256 CUs
+MIN_KEYS_PER_SPLIT = 256
+TARGET_WAVES = 1024     # wavefronts wanted in flight on 256 CUs (measured: more and shorter items cost more in the merge than they gain)
 
 
 def group_tiling(group_size: int):
@@ -53,9 +53,21 @@ class AttentionPlan:
         self.items, self.item_slot, self.merges, self.n_slots = items, item_slot, merges, n_slots
 
 
+def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: int, target_waves: int = TARGET_WAVES) -> int:
+    """Splits per row when the plan's shape must not depend on the rows' contexts (a captured
+    graph of a decode step): enough to fill the chip, never pieces shorter than MIN_KEYS_PER_SPLIT
+    at the longest context the graph serves."""
+    _, _, group_tiles = group_tiling(group_size)
+    waves = max(1, n_rows * n_kv_heads * group_tiles)
+    return max(1, min(MAX_SPLITS, target_waves // waves, max_keys // MIN_KEYS_PER_SPLIT))
+
+
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
-                         target_waves: int = TARGET_WAVES) -> AttentionPlan:
-    """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys."""
+                         target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None) -> AttentionPlan:
+    """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
+
+    With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
+    arrays have the same shape whatever the contexts are."""
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
@@ -73,7 +85,9 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
             k_begin = 0 if window is None else max(0, first_pos + q0 - window + 1)
             n_keys = k_end - k_begin
             splits = 1
-            if waves_unsplit < target_waves:
+            if fixed_splits is not None:
+                splits = fixed_splits
+            elif waves_unsplit < target_waves:
                 splits = min(MAX_SPLITS, max(1, target_waves // max(1, waves_unsplit)), max(1, n_keys // MIN_KEYS_PER_SPLIT))
             if splits <= 1:
                 items.append((row, q0, k_begin, k_end))
@@ -84,9 +98,9 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
             per = -(-per // KEY_ALIGN) * KEY_ALIGN        # at most `splits` items, each a multiple of KEY_ALIGN keys
             first_slot = n_slots
             count = 0
-            while start < k_end:
+            while start < k_end or (fixed_splits is not None and count < splits):
                 lo, hi = max(start, k_begin), min(start + per, k_end)
-                items.append((row, q0, lo, hi))
+                items.append((row, q0, lo, max(lo, hi)) if lo < k_end else (row, q0, k_end, k_end))
                 slots.append(n_slots)
                 n_slots += 1
                 count += 1
@@ -98,6 +112,8 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
 
 
 class GQAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  qk_norm_eps: Optional[float] = None, bias: bool = False, out_bias: Optional[bool] = None,
                  window: Optional[int] = None, scale: Optional[float] = None):
@@ -146,7 +162,11 @@ class GQAttention(Mixer):
         key = self.plan_key()
         if ctx.has_plan(key):
             return
-        plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window)
+        fixed = None
+        if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
+            fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys)
+        plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
+                                    fixed_splits=fixed)
         ctx.set_plan(key, {
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "n_items": len(plan.items), "n_merges": len(plan.merges),
             "n_slots": plan.n_slots,

@@ -81,6 +81,11 @@ class PositionEncoding(Part):
 class Mixer(Part):
     """Token mixer: reads and writes its own cache through the view the step gives it."""
 
+    # True if ``forward`` only launches work whose shapes and addresses follow from the step's
+    # staged arrays (no host-side loops over rows, no host reads): such a step can be captured
+    # into a graph once and replayed.
+    graph_safe = False
+
     def cache_spec(self):
         """:class:`PagedKVSpec`, :class:`StateSpec` or None."""
         return None

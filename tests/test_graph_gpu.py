@@ -1,0 +1,45 @@
+"""Captured single-token steps against the same steps run eagerly: every replay is checked, with
+eager work (portions of other prompts) and synchronisations between the replays."""
+import pytest
+import torch
+
+from helpers import model_folder, random_tokens
+from tiny_configs import CASES
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", ["A", "B"])
+def test_replayed_steps_equal_eager_steps(case, dtype):
+    from llmserver_amd.cache import CacheManager
+    from llmserver_amd.engine import ModelRunner, StepEntry, load_model
+    print(f"graph replay {case} {dtype}", flush=True)
+    raw, _, page = CASES[case]
+    model = load_model(model_folder(case), "cuda", dtype)
+    runners = []
+    for use_graphs in (True, False):
+        cache = CacheManager(model.cache_specs(), page, 200, device="cuda", dtype=model.dtype)
+        runners.append(ModelRunner(model, cache, use_graphs=use_graphs))
+    prompts = {"a": random_tokens(raw["vocab_size"], 37, 1), "b": random_tokens(raw["vocab_size"], 5, 2), "c": random_tokens(raw["vocab_size"], 64, 3)}
+    feed = {rid: random_tokens(raw["vocab_size"], 80, 10 + i) for i, rid in enumerate(prompts)}
+    for runner in runners:
+        for rid, tokens in prompts.items():
+            runner.cache.open(rid)
+            runner.step([StepEntry(rid, tokens, [])])
+    worst = 0.0
+    for turn in range(70):
+        live = ["a", "b", "c"] if turn % 9 else ["a", "c"]             # another number of rows now and then: another graph
+        entries = [StepEntry(rid, [feed[rid][turn]], [0]) for rid in live]
+        outs = [runner.step(entries).clone() for runner in runners]
+        torch.cuda.synchronize()
+        worst = max(worst, float((outs[0] - outs[1]).abs().max()))
+        if turn % 7 == 3:                                              # eager work between the replays
+            for runner in runners:
+                runner.cache.open("tmp")
+                runner.step([StepEntry("tmp", random_tokens(raw["vocab_size"], 23, turn), [22])])
+                runner.cache.close("tmp")
+    assert runners[0].graph_replays >= 60 and runners[1].graph_replays == 0
+    assert worst <= (1e-5 if dtype == "float32" else 2e-2), worst
+    for runner in runners:
+        runner.cache.check_invariants()
