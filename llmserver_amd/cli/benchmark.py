@@ -1,0 +1,152 @@
+"""Benchmark of the engine on token-id prompts, in the manner of the reference's
+``benchmark_cuda.py`` (/root/reference/benchmark_cuda.py:1-13, 475-496): option names and
+meanings follow it where it has them.
+
+    python benchmark.py --model DIR --prompt-tokens 128,1024 --batch-sizes 1,8,32 --output-tokens 128
+    python benchmark.py --random-config qwen3-8b --prompt-tokens 2048 --batch-sizes 1,8,64 --output-tokens 2048
+
+For each (prompt length, batch size):
+  * ttft_s  = time to generate 1 token for the whole batch (prefill latency)
+  * total_s = time to generate ``--output-tokens`` tokens for the whole batch
+  * decode tok/s = batch * (output_tokens - 1) / (total_s - ttft_s)
+EOS is ignored, decoding is greedy unless ``--temperature`` is given, and every (prompt length,
+batch size, repeat) gets its own seeded random token ids, so prefix caching cannot help
+(/root/reference/benchmark_cuda.py:13, 32-38).  ``--random-config`` draws seeded random weights
+on the device instead of reading a folder.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import statistics
+import sys
+import time
+
+RANDOM_CONFIGS = {
+    "tiny-a": dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                   intermediate_size=128, vocab_size=256, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True),
+    "tiny-b": dict(num_hidden_layers=3, hidden_size=96, num_attention_heads=8, num_key_value_heads=2, head_dim=32,
+                   intermediate_size=224, vocab_size=384, rope_theta=1e6, rms_norm_eps=1e-5, attention_bias=True),
+    "qwen3-1.7b": dict(num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
+                       intermediate_size=6144, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=True),
+    "qwen3-8b": dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                     intermediate_size=12288, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
+    "qwen3-32b": dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+                      intermediate_size=25600, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
+}
+
+
+def parse_ints(text):
+    return [int(item) for item in text.split(",") if item.strip()]
+
+
+def build_prompts(vocab, prompt_tokens, count, tag, seed):
+    """Seeded uniform random token ids, different for every tag (they stand in for tokenised text)."""
+    import hashlib
+
+    import torch
+    generator = torch.Generator().manual_seed(int.from_bytes(hashlib.sha256(f"{tag}:{seed}".encode()).digest()[:4], "little"))
+    return [torch.randint(0, vocab, (prompt_tokens,), generator=generator).tolist() for _ in range(count)]
+
+
+def run_once(engine, prompts, new_tokens):
+    import torch
+    engine.max_new_tokens = new_tokens
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    requests = [engine.add_request(None, prompt_token_ids=prompt, max_new_tokens=new_tokens) for prompt in prompts]
+    while engine.step():
+        pass
+    torch.cuda.synchronize()
+    return time.perf_counter() - start, [list(r.generated_token_ids) for r in requests]
+
+
+def main(argv=None) -> int:
+    parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    parser.add_argument("--model", default=None, help="model folder (config.json + safetensors)")
+    parser.add_argument("--random-config", default=None, choices=sorted(RANDOM_CONFIGS), help="seeded random weights of a named size instead of --model")
+    parser.add_argument("--prompt-tokens", default="128,1024")
+    parser.add_argument("--batch-sizes", default="1,8,32")
+    parser.add_argument("--output-tokens", type=int, default=128)
+    parser.add_argument("--repeats", type=int, default=3)
+    parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
+    parser.add_argument("--device", default="cuda")
+    parser.add_argument("--block-size", type=int, default=16)
+    parser.add_argument("--max-num-batched-tokens", type=int, default=16384)
+    parser.add_argument("--prefill-chunk-size", type=int, default=None)
+    parser.add_argument("--temperature", type=float, default=0.0)
+    parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--profile", action="store_true", help="print the engine's per-phase step counters")
+    parser.add_argument("--json", default=None, help="write the results to this file")
+    args = parser.parse_args(argv)
+    if (args.model is None) == (args.random_config is None):
+        parser.error("pass exactly one of --model and --random-config")
+
+    import torch
+
+    from ..config import config_from_dict
+    from ..engine import Engine, load_model
+    from ..engine.loading import parse_dtype
+    from ..cache import CacheManager
+    from ..weights import RandomInit, random_model_on_device
+
+    started = time.perf_counter()
+    if args.model:
+        model = load_model(args.model, args.device, args.dtype)
+    else:
+        config = config_from_dict(dict(RANDOM_CONFIGS[args.random_config], model_type="qwen3"))
+        model = random_model_on_device(config, args.device, parse_dtype(args.dtype), RandomInit(seed=args.seed, std=0.02))
+        model.name = args.random_config
+    torch.cuda.synchronize()
+    print(f"loaded {model.name} in {time.perf_counter() - started:.1f} s", flush=True)
+    vocab = model.config.vocab_size
+    prompt_lengths, batches = parse_ints(args.prompt_tokens), parse_ints(args.batch_sizes)
+    max_batch, max_length = max(batches), max(prompt_lengths) + args.output_tokens
+    bytes_per_block = CacheManager.bytes_per_token(model.cache_specs(), model.dtype) * args.block_size
+    wanted = max_batch * math.ceil(max_length / args.block_size) + 8          # /root/reference/benchmark_cuda.py:107-111
+    wanted = min(wanted, int(torch.cuda.mem_get_info()[0] * 0.8 // max(1, bytes_per_block)))
+    engine = Engine(model, None, max_new_tokens=1, max_batch_size=max_batch,
+                    max_num_batched_tokens=max(args.max_num_batched_tokens, max_batch), prefill_chunk_size=args.prefill_chunk_size,
+                    kv_cache_num_blocks=wanted, kv_cache_block_size=args.block_size, stream_text=False, max_completed_requests=0,
+                    ignore_eos=True, temperature=args.temperature, seed=args.seed, enable_prefix_caching=True)
+    results = []
+    for prompt_length in prompt_lengths:
+        for batch in batches:
+            entry = {"prompt_tokens": prompt_length, "batch": batch, "output_tokens": args.output_tokens}
+            try:
+                if batch * (prompt_length + args.output_tokens) > wanted * args.block_size:
+                    raise MemoryError("KV cache too small for this configuration")
+                run_once(engine, build_prompts(vocab, prompt_length, batch, f"warm-{prompt_length}-{batch}", args.seed), 2)
+                ttft, total, tokens = [], [], None
+                for repeat in range(args.repeats):
+                    seconds, _ = run_once(engine, build_prompts(vocab, prompt_length, batch, f"t1-{prompt_length}-{batch}-{repeat}", args.seed), 1)
+                    ttft.append(seconds)
+                for repeat in range(args.repeats):
+                    seconds, generated = run_once(engine, build_prompts(vocab, prompt_length, batch, f"tn-{prompt_length}-{batch}-{repeat}", args.seed), args.output_tokens)
+                    total.append(seconds)
+                    tokens = tokens or generated
+                ttft_s, total_s = statistics.median(ttft), statistics.median(total)
+                decode_s = max(total_s - ttft_s, 1e-9)
+                entry.update(ttft_s=ttft_s, total_s=total_s, decode_tok_s=batch * (args.output_tokens - 1) / decode_s,
+                             e2e_tok_s=batch * args.output_tokens / total_s, prefill_tok_s=batch * prompt_length / ttft_s,
+                             ms_per_token=1000 * decode_s / max(args.output_tokens - 1, 1), tokens=tokens,
+                             peak_alloc_gb=round(torch.cuda.max_memory_allocated() / 2 ** 30, 2))
+                print(f"prompt {prompt_length:6d}  batch {batch:3d}:  ttft {ttft_s * 1000:9.2f} ms   decode {entry['decode_tok_s']:10.1f} tok/s   "
+                      f"prefill {entry['prefill_tok_s']:10.1f} tok/s   end-to-end {entry['e2e_tok_s']:10.1f} tok/s", flush=True)
+            except Exception as error:            # record per-configuration failures (e.g. out of memory) and go on
+                entry["error"] = f"{type(error).__name__}: {error}"
+                print(f"prompt {prompt_length:6d}  batch {batch:3d}:  {entry['error']}", flush=True)
+            results.append(entry)
+    if args.profile:
+        print("step profile:", json.dumps(engine.step_profile), flush=True)
+    report = {"model": model.name, "dtype": args.dtype, "block_size": args.block_size, "kv_blocks": wanted, "gpu": torch.cuda.get_device_name(0),
+              "torch": torch.__version__, "results": results, "step_profile": engine.step_profile}
+    if args.json:
+        with open(args.json, "w") as handle:
+            json.dump(report, handle)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

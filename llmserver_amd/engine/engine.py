@@ -281,9 +281,16 @@ class Engine:
         self.remove_finished_and_cancelled_requests()
 
     def step(self) -> bool:
+        clock, profile = time.perf_counter, self.step_profile
+        t0 = clock()
         out = self.schedule_step()
+        t1 = clock()
         self.run_scheduled(out)
-        self.step_profile["steps"] += 1
+        profile["steps"] += 1
+        profile["schedule_s"] += t1 - t0
+        profile["step_s"] += clock() - t1
+        profile["decode_steps"] += bool(out.decode_requests)
+        profile["prefill_steps"] += bool(out.prefill_requests)
         return bool(self.scheduler.waiting or self.scheduler.running)
 
     async def run(self):
