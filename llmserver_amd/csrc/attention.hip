@@ -349,6 +349,271 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     }
 }
 
+#if LSA_BF16
+// ------------------------------------------------------------------------------------------------
+// Portions of prompts: four wavefronts of a workgroup take four consecutive tiles of 16 pairs of
+// one request.  They see (almost) the same keys, so each step's 32 keys and values are fetched
+// from the pages once per workgroup into LDS (double-buffered: the global loads of step i+1 are
+// issued before the products of step i and stored to the other buffer afterwards, one barrier a
+// step) and every wavefront reads its MFMA operands from there.  Rows in LDS are padded so that
+// the operand reads of a wavefront spread over the banks.  No key ranges are split here: such
+// rows have many tiles.  `tiles[i]` = {row, first token of the workgroup's 4 tiles, k_begin, k_end}.
+constexpr int K_ROW = D * 2 + 16;                 // bytes of a key row in LDS
+constexpr int V_ROW = 32 * 2 + 8;                 // bytes of a value row (one head dimension, 32 keys)
+constexpr int K_TILE_BYTES = 32 * K_ROW, V_TILE_BYTES = D * V_ROW;
+constexpr int K_PIECES = 32 * (D / 8), V_PIECES = D * 8;       // 16-byte pieces of keys, 8-byte pieces of values
+constexpr int KPT = (K_PIECES + 255) / 256, VPT = (V_PIECES + 255) / 256;
+// Three wavefronts per SIMD hide the latency of a step's dependent chain (LDS read, MFMA, softmax, MFMA).
+#define LSA_TILE_MIN_WAVES (LSA_ND <= 8 ? 3 : 1)
+
+__global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES) void paged_attention_tile_kernel(
+    const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
+    const elem_t* __restrict__ keys, const elem_t* __restrict__ values,
+    const int* __restrict__ table, int table_stride,
+    const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
+    const Item* __restrict__ tiles, Geometry g) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2][K_TILE_BYTES + V_TILE_BYTES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const Item tile = tiles[blockIdx.x];
+    const int kv_head = blockIdx.y / g.gtiles, gtile = blockIdx.y % g.gtiles;
+    const int col = lane & 15, quad = lane >> 4;
+    const int row = tile.row;
+    const int n = row_len[row], first_pos = row_ctx[row] - n;
+    const int q0 = tile.q0 + wave * g.tokens_per_tile;          // first token of this wavefront's tile
+    const int token0 = row_start[row] + q0;
+    const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
+    const bool pair_valid = pair_token < g.tokens_per_tile && q0 + pair_token < n && pair_head_in_group < g.group;
+    const int q_pos = pair_valid ? first_pos + q0 + pair_token : -1;
+    const int head = kv_head * g.group + pair_head_in_group;
+    const int* row_table = table + (size_t)row * table_stride;
+    const int ps = g.page_size;
+    const size_t kv_head_keys = (size_t)kv_head * ps * D, kv_head_values = (size_t)kv_head * D * ps;
+    const size_t page_elems = (size_t)g.n_kv * ps * D;
+    // Keys this wavefront's pairs can see at all: [wave_lo, wave_hi).
+    const int wave_tokens = max(0, min(g.tokens_per_tile, n - q0));
+    const int wave_hi = wave_tokens > 0 ? first_pos + q0 + wave_tokens : 0;
+    const int wave_lo = g.window > 0 ? max(0, first_pos + q0 - g.window + 1) : 0;
+    const int q_pos_min = first_pos + q0;                       // smallest position among the wavefront's valid pairs
+    const float scale_log2 = g.scale * 1.44269504088896340736f;
+
+    bf16x8 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int dim = 32 * s + 8 * quad;
+        bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (pair_valid && dim < D)
+            x = *reinterpret_cast<const bf16x8*>(q + (size_t)(token0 + pair_token) * q_token_stride + (size_t)head * D + dim);
+        qf[s] = x;
+    }
+    f32x4 acc[ND];
+#pragma unroll
+    for (int c = 0; c < ND; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float run_max = NEG_INF, run_sum = 0.f;
+
+    const int k_begin = tile.k_begin, k_end = tile.k_end;
+    int chunk = -1, pages_cur = 0, pages_next = 0;
+    auto table_chunk = [&](int c) { return row_table[min(64 * c + lane, table_stride - 1)]; };
+    auto enter_chunk = [&](int kt) {
+        const int c = (int)__umulhi((unsigned)kt, g.page_magic) >> 6;
+        if (c != chunk) {
+            pages_cur = (chunk >= 0 && c == chunk + 1) ? pages_next : table_chunk(c);
+            chunk = c;
+            pages_next = table_chunk(c + 1);
+        }
+    };
+    auto locate = [&](int key, int& slot) {
+        const int block = (int)__umulhi((unsigned)key, g.page_magic);
+        slot = key - block * ps;
+        return (size_t)__shfl(pages_cur, block - 64 * chunk, 64) * page_elems;
+    };
+
+    struct Staged {
+        bf16x8 k[KPT];
+        bf16x4 v[VPT];
+    };
+    // Where each of this thread's pieces lies inside a step: constant over the steps.
+    int k_off[KPT], v_off[VPT];
+    bool k_second[KPT], v_second[VPT];             // piece belongs to keys 16..31 of the step
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const int p = min(tid + 256 * j, K_PIECES - 1), key = p / (D / 8);
+        k_second[j] = key >= 16;
+        k_off[j] = (key & 15) * D + 8 * (p % (D / 8));
+    }
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int p = min(tid + 256 * j, V_PIECES - 1), piece = p & 7;
+        v_second[j] = piece >= 4;
+        v_off[j] = (p >> 3) * ps + 4 * (piece & 3);
+    }
+    const bool pages_of_16 = (ps & 15) == 0;        // then each half of a step (16 keys) lies inside one page
+    auto issue_loads = [&](Staged& r, int kt) {
+        enter_chunk(kt);
+        if (pages_of_16 && kt >= k_begin && kt + 32 <= k_end) {
+            // Interior step: two page lookups for the whole wavefront (scalar), then one add per piece.
+            const int block_a = (int)__umulhi((unsigned)kt, g.page_magic), block_b = (int)__umulhi((unsigned)(kt + 16), g.page_magic);
+            const int slot_a = kt - block_a * ps, slot_b = kt + 16 - block_b * ps;
+            const size_t page_a = (size_t)__builtin_amdgcn_readlane(pages_cur, block_a - 64 * chunk) * page_elems;
+            const size_t page_b = (size_t)__builtin_amdgcn_readlane(pages_cur, block_b - 64 * chunk) * page_elems;
+            const elem_t* ka = keys + page_a + kv_head_keys + (size_t)slot_a * D;
+            const elem_t* kb = keys + page_b + kv_head_keys + (size_t)slot_b * D;
+            const elem_t* va = values + page_a + kv_head_values + slot_a;
+            const elem_t* vb = values + page_b + kv_head_values + slot_b;
+#pragma unroll
+            for (int j = 0; j < KPT; ++j) r.k[j] = *reinterpret_cast<const bf16x8*>((k_second[j] ? kb : ka) + k_off[j]);
+#pragma unroll
+            for (int j = 0; j < VPT; ++j) r.v[j] = *reinterpret_cast<const bf16x4*>((v_second[j] ? vb : va) + v_off[j]);
+            return;
+        }
+        const int lo = max(k_begin, kt), hi = min(k_end, kt + 32) - 1;
+#pragma unroll
+        for (int j = 0; j < KPT; ++j) {
+            const int p = min(tid + 256 * j, K_PIECES - 1);
+            int slot;
+            const int key = min(max(kt + p / (D / 8), lo), hi);
+            const size_t page = locate(key, slot);
+            r.k[j] = *reinterpret_cast<const bf16x8*>(keys + page + kv_head_keys + (size_t)slot * D + 8 * (p % (D / 8)));
+        }
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            const int p = min(tid + 256 * j, V_PIECES - 1);
+            int slot;
+            const int key0 = min(max(kt + 4 * (p & 7), lo & ~3), hi & ~3);
+            const size_t page = locate(key0, slot);
+            r.v[j] = *reinterpret_cast<const bf16x4*>(values + page + kv_head_values + (size_t)(p >> 3) * ps + slot);
+        }
+    };
+    auto store_lds = [&](int buf, Staged& r, int kt) {
+        unsigned char* kl = lds[buf];
+        unsigned char* vl = lds[buf] + K_TILE_BYTES;
+#pragma unroll
+        for (int j = 0; j < KPT; ++j) {
+            const int p = tid + 256 * j;
+            if (p < K_PIECES) *reinterpret_cast<bf16x8*>(kl + (p / (D / 8)) * K_ROW + 16 * (p % (D / 8))) = r.k[j];
+        }
+        const bool edge = kt < k_begin || kt + 32 > k_end;
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            const int p = tid + 256 * j;
+            bf16x4 piece = r.v[j];
+            if (edge) {                           // keys outside the range may hold anything: keep them out of the sums
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int kpos = kt + 4 * (p & 7) + r;
+                    if (kpos < k_begin || kpos >= k_end) piece[r] = (bf16_t)0.f;
+                }
+            }
+            if (p < V_PIECES) *reinterpret_cast<bf16x4*>(vl + (p >> 3) * V_ROW + 8 * (p & 7)) = piece;
+        }
+    };
+    auto compute = [&](int buf, int kt) {
+        if (kt >= wave_hi || kt + 32 <= wave_lo) return;          // nothing for this wavefront's pairs in this step
+        const unsigned char* kl = lds[buf];
+        const unsigned char* vl = lds[buf] + K_TILE_BYTES;
+        // Steps every valid pair sees completely need no mask.
+        const bool full = kt >= k_begin && kt + 32 <= k_end && kt + 31 <= q_pos_min && wave_tokens == g.tokens_per_tile &&
+                          (g.window <= 0 || kt > first_pos + q0 + wave_tokens - 1 - g.window);
+        float sv[8];
+        float tile_max = NEG_INF;
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                bf16x8 kf = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (32 * s + 32 <= D || quad < 2) kf = *reinterpret_cast<const bf16x8*>(kl + (16 * t2 + col) * K_ROW + 64 * s + 16 * quad);
+                s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], s4, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = s4[r] * scale_log2;          // scores in units of ln 2: exp2 below is one instruction
+                if (!full) {
+                    const int kpos = kt + 16 * t2 + 4 * quad + r;
+                    const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
+                    v = seen ? v : NEG_INF;
+                } else if (!pair_valid) {
+                    v = NEG_INF;
+                }
+                sv[4 * t2 + r] = v;
+                tile_max = fmaxf(tile_max, v);
+            }
+        }
+        // The running maximum of a pair only moves when some key of this step beats it, which
+        // soon becomes rare: then the exchange between the lanes of a pair and the rescaling of
+        // the accumulators are skipped (the result is the same, the maximum being unchanged).
+        if (__any(tile_max > run_max)) {
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+            const float new_max = fmaxf(run_max, tile_max);
+            const float alpha = __builtin_amdgcn_exp2f(run_max - (new_max == NEG_INF ? 0.f : new_max));
+            run_max = new_max;
+            run_sum *= alpha;
+#pragma unroll
+            for (int c = 0; c < ND; ++c) acc[c] *= alpha;
+        }
+        const float use_max = run_max == NEG_INF ? 0.f : run_max;
+        bf16x8 pf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float p = __builtin_amdgcn_exp2f(sv[e] - use_max);
+            run_sum += p;
+            pf[e] = (bf16_t)p;
+        }
+#pragma unroll
+        for (int c = 0; c < ND; ++c) {
+            const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vl + (16 * c + col) * V_ROW + 8 * quad);
+            const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vl + (16 * c + col) * V_ROW + 32 + 8 * quad);
+            bf16x8 vf;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                vf[r] = lo4[r];
+                vf[4 + r] = hi4[r];
+            }
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[c], 0, 0, 0);
+        }
+    };
+
+    if (k_begin < k_end) {
+        // Loads run two steps ahead of the products: while step i is multiplied out of one LDS
+        // buffer, step i+1 sits in registers on its way to the other buffer and step i+2 is being
+        // fetched.  Loads are issued unconditionally (past the end they fetch the last step again),
+        // so that nothing between a load and its use makes the wait stricter than it has to be.
+        Staged r0, r1;
+        int kt = (k_begin / 32) * 32;
+        const int last = ((k_end - 1) / 32) * 32;
+        issue_loads(r0, kt);
+        issue_loads(r1, min(kt + 32, last));
+        store_lds(0, r0, kt);
+        __syncthreads();
+        while (true) {
+            issue_loads(r0, min(kt + 64, last));
+            compute(0, kt);
+            if (kt + 32 > last) break;
+            store_lds(1, r1, kt + 32);
+            __syncthreads();
+            issue_loads(r1, min(kt + 96, last));
+            compute(1, kt + 32);
+            if (kt + 64 > last) break;
+            store_lds(0, r0, kt + 64);
+            __syncthreads();
+            kt += 64;
+        }
+    }
+    run_sum += __shfl_xor(run_sum, 16, 64);
+    run_sum += __shfl_xor(run_sum, 32, 64);
+    if (!pair_valid) return;
+    const float inv = run_sum > 0.f ? 1.f / run_sum : 0.f;
+    elem_t* o = out + ((size_t)(token0 + pair_token) * g.n_q + head) * D + 4 * quad;
+#pragma unroll
+    for (int c = 0; c < ND; ++c) {
+        bf16x4 r4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) r4[r] = (bf16_t)(acc[c][r] * inv);
+        *reinterpret_cast<bf16x4*>(o + 16 * c) = r4;
+    }
+}
+#endif  // LSA_BF16
+
 // Merge the partial slots of a tile: out = sum_s w_s acc_s / sum_s w_s l_s, w_s = exp(m_s - max m).
 struct Merge { int row, q0, first_slot, n_slots; };
 
@@ -399,13 +664,26 @@ __global__ __launch_bounds__(128) void merge_kernel(
 LSA_EXPORT int lsa_paged_attention(
     const void* q, long q_token_stride, void* out, const void* keys, const void* values, const int* table, int table_stride,
     const int* row_start, const int* row_len, const int* row_ctx, const void* items, const int* item_slot, int n_items,
-    const void* merges, int n_merges, float* part_acc, float* part_ml, float scale, int window, int page_size, int n_q,
-    int n_kv, int gheads, int tokens_per_tile, int gtiles, hipStream_t stream) {
-    if (n_items <= 0) return 0;
+    const void* merges, int n_merges, float* part_acc, float* part_ml, const void* tiles, int n_tiles, float scale, int window,
+    int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles, hipStream_t stream) {
+    if (n_items <= 0 && n_tiles <= 0) return 0;
     Geometry g;
     g.n_q = n_q; g.n_kv = n_kv; g.group = n_q / n_kv; g.gheads = gheads; g.tokens_per_tile = tokens_per_tile;
     g.gtiles = gtiles; g.page_size = page_size; g.window = window; g.scale = scale;
     g.page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
+    if (n_tiles > 0) {
+#if LSA_BF16
+        dim3 tgrid(n_tiles, n_kv * gtiles);
+        paged_attention_tile_kernel<<<tgrid, 256, 0, stream>>>(
+            (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
+            row_start, row_len, row_ctx, (const Item*)tiles, g);
+        const int terr = (int)hipGetLastError();
+        if (terr) return terr;
+#else
+        return -1;                    // the workgroup-tile kernel exists for bfloat16 only
+#endif
+    }
+    if (n_items <= 0) return 0;
     dim3 grid((n_items + 3) / 4, n_kv * gtiles);
     paged_attention_kernel<<<grid, 256, 0, stream>>>(
         (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,

@@ -194,6 +194,12 @@ class HipOps:
         _check(plan["items"], "plan items", torch.int32, (n_items, 4))
         _check(plan["item_slot"], "plan item_slot", torch.int32, (n_items,))
         _check(plan["merges"], "plan merges", torch.int32, (n_merges, 4))
+        n_tiles = plan.get("n_tiles", 0)
+        tiles = plan.get("tiles") if n_tiles else None
+        if n_tiles:
+            _check(tiles, "plan tiles", torch.int32, (n_tiles, 4))
+            if qkv.dtype != torch.bfloat16:
+                raise TypeError("the workgroup-tile attention kernel exists for bfloat16 only")
         gheads, tokens_per_tile, gtiles = group_tiling(n_q // n_kv)
         part_acc = part_ml = None
         if n_slots:
@@ -203,8 +209,8 @@ class HipOps:
         _launched(lib.lsa_paged_attention(
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(row_start),
             _ptr(row_len), _ptr(row_ctx), _ptr(plan["items"]), _ptr(plan["item_slot"]), n_items, _ptr(plan["merges"]),
-            n_merges, _ptr(part_acc), _ptr(part_ml), float(scale), int(window) if window else 0, page_size, n_q, n_kv,
-            gheads, tokens_per_tile, gtiles, _stream()), "paged_attention")
+            n_merges, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), n_tiles, float(scale), int(window) if window else 0,
+            page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, _stream()), "paged_attention")
 
     def sample(self, logits, temperature, uniform, out):
         n, vocab = logits.shape

@@ -47,10 +47,13 @@ class AttentionPlan:
     key, one past the last key.  ``item_slot [n_items] int32``: index of the partial-result slot,
     or -1 if the item covers all keys of its rows and writes the output itself.
     ``merges [n_merges, 4] int32``: row, first token of the tile, first slot, number of slots.
+    ``tiles [n_tiles, 4] int32``: row, first token, first key, one past the last key of four
+    consecutive tiles that one workgroup handles together, sharing the keys it loads.
     """
 
-    def __init__(self, items, item_slot, merges, n_slots):
+    def __init__(self, items, item_slot, merges, n_slots, tiles=None):
         self.items, self.item_slot, self.merges, self.n_slots = items, item_slot, merges, n_slots
+        self.tiles = tiles if tiles is not None else np.zeros((0, 4), dtype=np.int32)
 
 
 def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: int, target_waves: int = TARGET_WAVES) -> int:
@@ -62,22 +65,34 @@ def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: i
     return max(1, min(MAX_SPLITS, target_waves // waves, max_keys // MIN_KEYS_PER_SPLIT))
 
 
+WORKGROUP_TILES = 4     # tiles a workgroup of the prompt-portion kernel handles together
+MIN_TILES_FOR_WORKGROUPS = 16
+
+
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
-                         target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None) -> AttentionPlan:
+                         target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
+                         workgroup_tiles: bool = False) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
-    arrays have the same shape whatever the contexts are."""
+    arrays have the same shape whatever the contexts are.  With ``workgroup_tiles`` rows with many
+    tiles (portions of prompts) go to the kernel in which four tiles share the keys they load."""
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
     tiles_per_row = -(-row_len // tokens_per_tile)
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
-    items, slots, merges = [], [], []
+    items, slots, merges, tiles = [], [], [], []
     n_slots = 0
     for row in range(len(row_len)):
         n, ctx = int(row_len[row]), int(row_ctx[row])
         first_pos = ctx - n
+        if workgroup_tiles and fixed_splits is None and tiles_per_row[row] >= MIN_TILES_FOR_WORKGROUPS:
+            span = WORKGROUP_TILES * tokens_per_tile
+            for q0 in range(0, n, span):
+                k_begin = 0 if window is None else max(0, first_pos + q0 - window + 1)
+                tiles.append((row, q0, k_begin, first_pos + min(q0 + span, n)))
+            continue
         for tile in range(int(tiles_per_row[row])):
             q0 = tile * tokens_per_tile
             q1 = min(q0 + tokens_per_tile, n)
@@ -108,7 +123,9 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
             merges.append((row, q0, first_slot, count))
     items = np.asarray(items, dtype=np.int32).reshape(-1, 4)
     merges = np.asarray(merges, dtype=np.int32).reshape(-1, 4)
-    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots)
+    tiles.sort(key=lambda tile: tile[2] - tile[3])       # most keys first: the long tiles must not start last
+    tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 4)
+    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, tiles)
 
 
 class GQAttention(Mixer):
@@ -165,10 +182,12 @@ class GQAttention(Mixer):
         fixed = None
         if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
             fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys)
+        import torch
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
-                                    fixed_splits=fixed)
+                                    fixed_splits=fixed, workgroup_tiles=ctx.dtype == torch.bfloat16)
         ctx.set_plan(key, {
-            "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "n_items": len(plan.items), "n_merges": len(plan.merges),
+            "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
+            "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),
             "n_slots": plan.n_slots,
         })
 

@@ -128,7 +128,7 @@ def test_qk_norm_rope_kv_write(ops, dtype, n_q, n_kv, d, page):
             assert not got_k.any() and not got_v.any()
 
 
-def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, needle=True, seed=0, target_waves=None):
+def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, needle=True, seed=0, target_waves=None, workgroup_tiles=None):
     """Random q/k/v through both implementations.  Pages are handed out in scrambled order from a
     pool that first held other data (as if used before).  With ``needle``, one far key per request
     is made to dominate its first query's softmax."""
@@ -161,9 +161,13 @@ def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, need
         keys[pages, :, (place % page).to(DEV), :] = k.to(dtype)
         values[pages, :, :, (place % page).to(DEV)] = v.to(dtype)
         table[r, :first] = -1                                                     # pages a window has passed are gone
-    plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, **({} if target_waves is None else {"target_waves": target_waves}))
+    if workgroup_tiles is None:
+        workgroup_tiles = dtype == torch.bfloat16
+    plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, workgroup_tiles=workgroup_tiles,
+                                **({} if target_waves is None else {"target_waves": target_waves}))
     staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
-              "merges": torch.from_numpy(plan.merges).to(DEV), "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots}
+              "merges": torch.from_numpy(plan.merges).to(DEV), "tiles": torch.from_numpy(plan.tiles).to(DEV), "n_tiles": len(plan.tiles),
+              "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots}
     t = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
     got = torch.zeros(tokens, n_q * d, device=DEV, dtype=dtype)
     ref = torch.zeros_like(got)
@@ -208,6 +212,20 @@ def test_attention_window_edge(ops, dtype, window):
     attention_case(ops, dtype, 4, 2, 32, 8, [1, 9], [700, 400], window=window, seed=window, target_waves=10 ** 6)
 
 
+@pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 2, 48, 12), (32, 8, 128, 16), (5, 1, 80, 20), (20, 1, 16, 4),
+                                                (2, 1, 256, 500), (16, 16, 64, 64)])
+@pytest.mark.parametrize("window", [None, 40])
+def test_attention_prompt_portions_in_workgroup_tiles(ops, n_q, n_kv, d, page, window):
+    """Long portions of prompts, with and without a prefix, beside decoded tokens: the portions go
+    through the kernel whose four wavefronts share the keys they load (bfloat16)."""
+    print(f"attention workgroup tiles {n_q}/{n_kv} d{d} page{page} window {window}", flush=True)
+    lens = [333, 1, 200, 97, 1]
+    ctxs = [333, 90, 777, 130, 400]
+    plan, _ = attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d)
+    assert len(plan.tiles) > 0 and len(plan.items) > 0
+    attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d, workgroup_tiles=False)
+
+
 def test_attention_refuses_sizes_it_cannot_take(ops):
     from llmserver_amd.kernels import build
     with pytest.raises(ValueError, match="head sizes"):
@@ -219,7 +237,7 @@ def test_attention_refuses_sizes_it_cannot_take(ops):
     keys, values = torch.zeros(2, 1, 6, 16, device=DEV), torch.zeros(2, 1, 16, 6, device=DEV)
     one = torch.ones(1, dtype=torch.int32, device=DEV)
     plan = {"items": torch.zeros(1, 4, dtype=torch.int32, device=DEV), "item_slot": -one, "merges": torch.zeros(0, 4, dtype=torch.int32, device=DEV),
-            "n_items": 1, "n_merges": 0, "n_slots": 0}
+            "n_items": 1, "n_merges": 0, "n_slots": 0, "n_tiles": 0}
     with pytest.raises(ValueError, match="multiple of 4"):
         ops.paged_attention(qkv, out, keys, values, torch.zeros(1, 1, dtype=torch.int32, device=DEV), 0 * one, one, one, plan, 1.0, None, 6, 2, 1, 16, Ctx())
     with pytest.raises(TypeError):
