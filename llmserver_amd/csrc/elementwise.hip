@@ -57,13 +57,27 @@ template <typename T, int V>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid, const T* __restrict__ delta,
                                                           const float* __restrict__ weight, float eps,
                                                           T* __restrict__ out, const int* __restrict__ rows, int width) {
+    // The first CACHE vectors of a thread stay in registers between the two passes (a row of up
+    // to 256 * V * CACHE elements is read from memory once); what lies beyond is read again.
+    constexpr int CACHE = 4;
     __shared__ float scratch[16];
     const int src_row = rows ? rows[blockIdx.x] : blockIdx.x;
     T* x = resid + (size_t)src_row * width;
     const T* d = delta ? delta + (size_t)src_row * width : nullptr;
     T* y = out + (size_t)blockIdx.x * width;
+    const int stride = blockDim.x * V;
+    float kept[CACHE][V];
     float sq = 0.f;
-    for (int i = threadIdx.x * V; i < width; i += blockDim.x * V) {
+#pragma unroll
+    for (int c = 0; c < CACHE; ++c) {
+        const int i = threadIdx.x * V + c * stride;
+        if (i < width) {
+            load_sum<T, V>(x, d, i, kept[c]);
+#pragma unroll
+            for (int k = 0; k < V; ++k) sq += kept[c][k] * kept[c][k];
+        }
+    }
+    for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
         float s[V];
         load_sum<T, V>(x, d, i, s);
 #pragma unroll
@@ -71,9 +85,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
     }
     const float total = block_sum(sq, scratch);
     const float rstd = rsqrtf(total / (float)width + eps);
-    for (int i = threadIdx.x * V; i < width; i += blockDim.x * V) {
-        float s[V];
-        load_sum<T, V>(x, d, i, s);
+    auto emit = [&](int i, const float (&s)[V]) {
         if (V > 1) {
             Vec16<T> o, r;
 #pragma unroll
@@ -87,6 +99,16 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
             if (d && !rows) x[i] = (T)s[0];
             y[i] = (T)(s[0] * rstd * weight[i]);
         }
+    };
+#pragma unroll
+    for (int c = 0; c < CACHE; ++c) {
+        const int i = threadIdx.x * V + c * stride;
+        if (i < width) emit(i, kept[c]);
+    }
+    for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
+        float s[V];
+        load_sum<T, V>(x, d, i, s);
+        emit(i, s);
     }
 }
 

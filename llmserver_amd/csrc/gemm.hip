@@ -17,37 +17,76 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int GEMM_WAVES = 8;
 
-template <int MT, typename OutT>
+// What the kernel does to its activations before the product (fused so that few-row steps need
+// fewer launches):
+//   PLAIN   X is bfloat16 [M, K].
+//   NORM    X = rmsnorm(resid + delta) * norm_weight, not yet computed: the kernel forms
+//           s = round(resid + delta) (32-bit sum, the new residual stream, written to resid_out by
+//           the first workgroup), multiplies round(s * norm_weight) into the product and scales the
+//           result by rsqrt(mean(s^2) + eps), which it gets from the same pass over s.
+//   SWIGLU  X = silu(gate) * up with gate_up [M, 2K] (gate first), computed in 32-bit.
+enum { PLAIN = 0, NORM = 1, SWIGLU = 2 };
+
+struct Prologue {
+    const bf16_t* second;        // NORM: delta (may be null); SWIGLU: unused (up follows gate in the row)
+    const float* norm_weight;    // NORM: [K]
+    bf16_t* resid_out;           // NORM: [M, K], written if second != null
+    float eps;
+};
+
+template <int MT, typename OutT, int PRO>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                                      OutT* __restrict__ y, int M, int N, int K) {
-    constexpr int CH = MT <= 2 ? 8 : 4;          // 32-wide k steps loaded together (one chunk)
+                                                                      OutT* __restrict__ y, int M, int N, int K, Prologue pro) {
+    constexpr int CH = (PRO != PLAIN || MT > 2) ? 4 : 8;          // 32-wide k steps loaded together (one chunk)
     __shared__ float partial[GEMM_WAVES][MT][256];
+    __shared__ float squares[GEMM_WAVES][MT][16];
+    extern __shared__ float norm_weight_lds[];                     // NORM: the norm weights, [K]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, quad = lane >> 4;
     const int n0 = blockIdx.x * 16;
     const int k_per_wave = ((K + GEMM_WAVES - 1) / GEMM_WAVES + 31) / 32 * 32;
     const int k_begin = min(K, wave * k_per_wave), k_end = min(K, k_begin + k_per_wave);
+    const int x_stride = PRO == SWIGLU ? 2 * K : K;
     const bf16_t* wp = w + (size_t)min(n0 + col, N - 1) * K + 8 * quad;
     const bf16_t* xp[MT];
+    const bf16_t* x2p[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) xp[t] = x + (size_t)min(16 * t + col, M - 1) * K + 8 * quad;
+    for (int t = 0; t < MT; ++t) {
+        const size_t row = (size_t)min(16 * t + col, M - 1);
+        xp[t] = x + row * x_stride + 8 * quad;
+        x2p[t] = PRO == SWIGLU ? xp[t] + K : (PRO == NORM && pro.second ? pro.second + row * K + 8 * quad : xp[t]);
+    }
+    if (PRO == NORM) {
+        for (int i = threadIdx.x * 4; i < K; i += GEMM_WAVES * 64 * 4)
+            *reinterpret_cast<f32x4*>(norm_weight_lds + i) = *reinterpret_cast<const f32x4*>(pro.norm_weight + i);
+        __syncthreads();
+    }
     f32x4 acc[MT];
+    float sumsq[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < MT; ++t) {
+        acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        sumsq[t] = 0.f;
+    }
 
     // A chunk: the operands of CH consecutive k steps.  Chunks are loaded one ahead of the chunk
     // being multiplied, X first (it comes from cache) so that it never queues behind the weights.
     struct Chunk {
         bf16x8 a[CH];
         bf16x8 b[CH][MT];
+        bf16x8 b2[PRO == PLAIN ? 1 : CH][PRO == PLAIN ? 1 : MT];
     };
     const int k_safe = K - 8;                      // a lane past the end reads the row's last 8 values and is zeroed
+    const bool has_second = PRO == SWIGLU || (PRO == NORM && pro.second != nullptr);
     auto load_chunk = [&](Chunk& c, int k0) {
 #pragma unroll
         for (int u = 0; u < CH; ++u) {
             const int k = min(k0 + 32 * u + 8 * quad, k_safe) - 8 * quad;
 #pragma unroll
-            for (int t = 0; t < MT; ++t) c.b[u][t] = *reinterpret_cast<const bf16x8*>(xp[t] + k);
+            for (int t = 0; t < MT; ++t) {
+                c.b[u][t] = *reinterpret_cast<const bf16x8*>(xp[t] + k);
+                if (PRO != PLAIN) c.b2[u][t] = *reinterpret_cast<const bf16x8*>(x2p[t] + k);
+            }
         }
 #pragma unroll
         for (int u = 0; u < CH; ++u) {
@@ -58,10 +97,40 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
     auto multiply_chunk = [&](Chunk& c, int k0) {
 #pragma unroll
         for (int u = 0; u < CH; ++u) {
+            const int k = k0 + 32 * u + 8 * quad;
+            const bool inside = k < k_end;
             bf16x8 a = c.a[u];
-            if (k0 + 32 * u + 8 * quad >= k_end) a = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+            if (!inside) a = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, c.b[u][t], acc[t], 0, 0, 0);
+            for (int t = 0; t < MT; ++t) {
+                bf16x8 b = c.b[u][t];
+                if (PRO == SWIGLU) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float gate = (float)b[e];
+                        b[e] = (bf16_t)(gate / (1.f + expf(-gate)) * (float)c.b2[u][t][e]);
+                    }
+                } else if (PRO == NORM) {
+                    const int ks = min(k, k_safe);
+                    const f32x4 w0 = *reinterpret_cast<const f32x4*>(norm_weight_lds + ks);
+                    const f32x4 w1 = *reinterpret_cast<const f32x4*>(norm_weight_lds + ks + 4);
+                    bf16x8 sum = b;
+                    if (has_second) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) sum[e] = (bf16_t)((float)b[e] + (float)c.b2[u][t][e]);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float v = inside ? (float)sum[e] : 0.f;
+                        sumsq[t] += v * v;
+                        b[e] = (bf16_t)(v * (e < 4 ? w0[e] : w1[e - 4]));
+                    }
+                    const int m = 16 * t + col;
+                    if (has_second && blockIdx.x == 0 && inside && m < M)
+                        *reinterpret_cast<bf16x8*>(pro.resid_out + (size_t)m * K + k) = sum;
+                }
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+            }
         }
     };
     if (k_begin < k_end) {
@@ -87,9 +156,16 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
         }
     }
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
+    for (int t = 0; t < MT; ++t) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) partial[wave][t][(4 * quad + r) + 16 * col] = acc[t][r];     // [m in tile][n in tile]
+        if (PRO == NORM) {
+            float sq = sumsq[t];
+            sq += __shfl_xor(sq, 16, 64);
+            sq += __shfl_xor(sq, 32, 64);
+            if (quad == 0) squares[wave][t][col] = sq;
+        }
+    }
     __syncthreads();
     for (int e = threadIdx.x; e < MT * 256; e += GEMM_WAVES * 64) {
         const int t = e >> 8, in_tile = e & 255;
@@ -97,18 +173,26 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
         float total = 0.f;
 #pragma unroll
         for (int v = 0; v < GEMM_WAVES; ++v) total += partial[v][t][in_tile];
+        if (PRO == NORM) {
+            float sq = 0.f;
+#pragma unroll
+            for (int v = 0; v < GEMM_WAVES; ++v) sq += squares[v][t][in_tile >> 4];
+            total *= rsqrtf(sq / (float)K + pro.eps);
+        }
         if (m < M && n < N) y[(size_t)m * N + n] = (OutT)total;
     }
 }
 
-template <typename OutT>
-static int launch(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
+template <typename OutT, int PRO>
+static int launch(const void* x, const void* w, void* y, int M, int N, int K, Prologue pro, hipStream_t stream) {
     const dim3 grid((N + 15) / 16), block(GEMM_WAVES * 64);
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
-    if (M <= 16) gemm_skinny_kernel<1, OutT><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K);
-    else if (M <= 32) gemm_skinny_kernel<2, OutT><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K);
-    else gemm_skinny_kernel<4, OutT><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K);
+    const size_t lds = PRO == NORM ? (size_t)K * sizeof(float) : 0;
+    if (M <= 16) gemm_skinny_kernel<1, OutT, PRO><<<grid, block, lds, stream>>>(xb, wb, (OutT*)y, M, N, K, pro);
+    else if (PRO != PLAIN) return -1;
+    else if (M <= 32) gemm_skinny_kernel<2, OutT, PLAIN><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro);
+    else gemm_skinny_kernel<4, OutT, PLAIN><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro);
     LSA_LAUNCH_CHECK();
 }
 
@@ -116,5 +200,24 @@ static int launch(const void* x, const void* w, void* y, int M, int N, int K, hi
 LSA_EXPORT int lsa_gemm_skinny(int out_float32, const void* x, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K % 8 != 0 || K < 8) return -1;
-    return out_float32 ? launch<float>(x, w, y, M, N, K, stream) : launch<bf16_t>(x, w, y, M, N, K, stream);
+    Prologue pro = {nullptr, nullptr, nullptr, 0.f};
+    return out_float32 ? launch<float, PLAIN>(x, w, y, M, N, K, pro, stream) : launch<bf16_t, PLAIN>(x, w, y, M, N, K, pro, stream);
+}
+
+// Y = (silu(gate) * up) . W^T with gate_up [M, 2K]; M <= 16.
+LSA_EXPORT int lsa_gemm_skinny_swiglu(const void* gate_up, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 8 != 0 || K < 8) return -1;
+    Prologue pro = {nullptr, nullptr, nullptr, 0.f};
+    return launch<bf16_t, SWIGLU>(gate_up, w, y, M, N, K, pro, stream);
+}
+
+// Y = rmsnorm(resid + delta) * norm_weight . W^T; resid_out = resid + delta (delta may be null: then
+// nothing is written and resid_out is ignored).  resid_out must not alias resid.  M <= 16, K <= 16384.
+LSA_EXPORT int lsa_gemm_skinny_norm(int out_float32, const void* resid, const void* delta, const float* norm_weight, float eps,
+                                    void* resid_out, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 8 != 0 || K < 8 || K > 16384 || (delta && resid_out == resid)) return -1;
+    Prologue pro = {(const bf16_t*)delta, norm_weight, (bf16_t*)resid_out, eps};
+    return out_float32 ? launch<float, NORM>(resid, w, y, M, N, K, pro, stream) : launch<bf16_t, NORM>(resid, w, y, M, N, K, pro, stream);
 }

@@ -1,92 +1,124 @@
-// Sampling from float32 logits, one block per row: greedy (temperature 0) takes the first
-// maximum; otherwise the token is drawn from softmax(logits / temperature) by inverting the
-// cumulative distribution at a uniform number the host supplies per row (so a request's
-// tokens do not depend on what else is in the batch).  The maximum, the sum of exponentials and
-// the running sums are 32-bit and walk the vocabulary in a fixed order.
+// Sampling from float32 logits: greedy (temperature 0) takes the first maximum; otherwise the
+// token is drawn from softmax(logits / temperature) by inverting the cumulative distribution at a
+// uniform number the host supplies per row (so a request's tokens do not depend on what else is
+// in the batch).  Two kernels: the first cuts every row into up to 64 contiguous chunks and
+// finds each chunk's maximum, first position of it, and sum of exponentials; the second merges a
+// row's chunks, finds the chunk in which the running sum passes the target and walks only that
+// chunk.  Maximum, sums and running sums are 32-bit and walk the vocabulary in a fixed order.
 #include "common.hpp"
 
 using namespace lsa;
 
-constexpr int SAMPLE_THREADS = 1024;
-constexpr int SAMPLE_WAVES = SAMPLE_THREADS / 64;
+constexpr int MAX_CHUNKS = 64;
+constexpr float MINUS_INF = -__builtin_huge_valf();
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
-                                                                const float* __restrict__ uniform, int* __restrict__ out, int vocab) {
-    __shared__ float s_val[SAMPLE_WAVES];
-    __shared__ int s_idx[SAMPLE_WAVES];
-    __shared__ float s_sum[SAMPLE_WAVES];
-    const float* x = logits + (size_t)blockIdx.x * vocab;
+struct ChunkStat { float top; int first; float sum; int pad; };
+
+__device__ inline void better(float& top, int& first, float other_top, int other_first) {
+    if (other_top > top || (other_top == top && other_first < first)) { top = other_top; first = other_first; }
+}
+
+__global__ __launch_bounds__(256) void sample_chunks_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                            ChunkStat* __restrict__ stats, int vocab, int chunk_len) {
+    __shared__ float s_top[4];
+    __shared__ int s_first[4];
+    __shared__ float s_sum[4];
+    const int row = blockIdx.x, chunk = blockIdx.y;
+    const float* x = logits + (size_t)row * vocab;
+    const int begin = chunk * chunk_len, end = min(vocab, begin + chunk_len);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // Each wavefront owns a contiguous segment of the vocabulary (a multiple of 64 long).
-    const int per_wave = ((vocab + SAMPLE_WAVES - 1) / SAMPLE_WAVES + 63) / 64 * 64;
-    const int seg_begin = wave * per_wave, seg_end = min(vocab, seg_begin + per_wave);
-
-    float best = -__builtin_huge_valf();
-    int best_i = 0x7fffffff;
-    for (int i = seg_begin + lane; i < seg_end; i += 64) {
-        const float v = x[i];
-        if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
-    }
+    float top = MINUS_INF;
+    int first = 0x7fffffff;
+    for (int i = begin + threadIdx.x; i < end; i += 256) better(top, first, x[i], i);
 #pragma unroll
-    for (int offset = 32; offset > 0; offset >>= 1) {
-        const float ov = __shfl_xor(best, offset, 64);
-        const int oi = __shfl_xor(best_i, offset, 64);
-        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
-    }
-    if (lane == 0) { s_val[wave] = best; s_idx[wave] = best_i; }
+    for (int offset = 32; offset > 0; offset >>= 1) better(top, first, __shfl_xor(top, offset, 64), __shfl_xor(first, offset, 64));
+    if (lane == 0) { s_top[wave] = top; s_first[wave] = first; }
     __syncthreads();
-    best = s_val[0]; best_i = s_idx[0];
-    for (int w = 1; w < SAMPLE_WAVES; ++w)
-        if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) { best = s_val[w]; best_i = s_idx[w]; }
-    const float temp = temperature[blockIdx.x];
-    if (!(temp > 0.f)) {
-        if (threadIdx.x == 0) out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+    top = s_top[0]; first = s_first[0];
+    for (int w = 1; w < 4; ++w) better(top, first, s_top[w], s_first[w]);
+    const float temp = temperature[row];
+    float total = 0.f;
+    if (temp > 0.f && top > MINUS_INF) {
+        const float inv_temp = 1.f / temp;
+        // Fixed order: the chunk in groups of 64 consecutive tokens, a wavefront per group in turn.
+        float part = 0.f;
+        for (int base = begin + 64 * wave; base < end; base += 256) {
+            const int i = base + lane;
+            part += i < end ? expf((x[i] - top) * inv_temp) : 0.f;
+        }
+        part = wave_sum(part);
+        if (lane == 0) s_sum[wave] = part;
+        __syncthreads();
+        total = s_sum[0] + s_sum[1] + s_sum[2] + s_sum[3];
+    }
+    if (threadIdx.x == 0) stats[(size_t)row * gridDim.y + chunk] = ChunkStat{top, first, total, 0};
+}
+
+__global__ __launch_bounds__(64) void sample_pick_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                         const float* __restrict__ uniform, const ChunkStat* __restrict__ stats,
+                                                         int* __restrict__ out, int vocab, int chunk_len, int chunks) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    const ChunkStat mine = lane < chunks ? stats[(size_t)row * chunks + lane] : ChunkStat{MINUS_INF, 0x7fffffff, 0.f, 0};
+    float top = mine.top;
+    int first = mine.first;
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) better(top, first, __shfl_xor(top, offset, 64), __shfl_xor(first, offset, 64));
+    const float temp = temperature[row];
+    if (!(temp > 0.f) || !(top > MINUS_INF)) {
+        if (lane == 0) out[row] = first == 0x7fffffff ? 0 : first;
         return;
     }
     const float inv_temp = 1.f / temp;
-    float part = 0.f;
-    for (int i = seg_begin + lane; i < seg_end; i += 64) part += expf((x[i] - best) * inv_temp);
-    part = wave_sum(part);
-    if (lane == 0) s_sum[wave] = part;
-    __syncthreads();
-    float total = 0.f;
-    for (int w = 0; w < SAMPLE_WAVES; ++w) total += s_sum[w];
-    const float target = uniform[blockIdx.x] * total;
-    // The segment in which the running sum passes the target (the last non-empty one if rounding leaves none).
-    float before = 0.f;
-    int chosen = 0;
-    for (int w = 0; w < SAMPLE_WAVES; ++w) {
-        if (w * per_wave >= vocab) break;
-        chosen = w;
-        if (before + s_sum[w] > target) break;
-        if ((w + 1) * per_wave < vocab) before += s_sum[w];
+    // Each chunk's sum, rescaled from its own maximum to the row's; inclusive running sums over the chunks.
+    const float scaled = mine.top > MINUS_INF ? mine.sum * expf((mine.top - top) * inv_temp) : 0.f;
+    float running = scaled;
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        const float up = __shfl_up(running, offset, 64);
+        if (lane >= offset) running += up;
     }
-    if (wave != chosen) return;
-    int result = seg_end - 1;
+    const float total = __shfl(running, 63, 64);
+    const float target = uniform[row] * total;
+    const unsigned long long passed = __ballot(lane < chunks && running > target);
+    const int chunk = passed ? __builtin_ctzll(passed) : chunks - 1;          // rounding may leave none: the last chunk
+    float before = __shfl(running - scaled, chunk, 64);
+    const float* x = logits + (size_t)row * vocab;
+    const int begin = chunk * chunk_len, end = min(vocab, begin + chunk_len);
+    int result = end - 1;
     bool found = false;
-    for (int base = seg_begin; base < seg_end && !found; base += 64) {
+    for (int base = begin; base < end && !found; base += 64) {
         const int i = base + lane;
-        const float p = i < seg_end ? expf((x[i] - best) * inv_temp) : 0.f;
-        float scan = p;                       // inclusive prefix sum over the 64 lanes
+        const float p = i < end ? expf((x[i] - top) * inv_temp) : 0.f;
+        float scan = p;
 #pragma unroll
         for (int offset = 1; offset < 64; offset <<= 1) {
             const float up = __shfl_up(scan, offset, 64);
             if (lane >= offset) scan += up;
         }
-        const bool hit = i < seg_end && before + scan > target;
-        const unsigned long long mask = __ballot(hit);
-        if (mask) {
-            result = base + __builtin_ctzll(mask);
+        const unsigned long long hit = __ballot(i < end && before + scan > target);
+        if (hit) {
+            result = base + __builtin_ctzll(hit);
             found = true;
         }
         before += __shfl(scan, 63, 64);
     }
-    if (lane == 0) out[blockIdx.x] = result;
+    if (lane == 0) out[row] = result;
 }
 
-LSA_EXPORT int lsa_sample(const float* logits, const float* temperature, const float* uniform, int* out, int n_rows, int vocab,
-                          hipStream_t stream) {
+LSA_EXPORT int lsa_sample_chunks(int vocab) {
+    int chunks = (vocab + 2047) / 2048;
+    return chunks < 1 ? 1 : (chunks > MAX_CHUNKS ? MAX_CHUNKS : chunks);
+}
+
+// workspace: n_rows * lsa_sample_chunks(vocab) * 16 bytes
+LSA_EXPORT int lsa_sample(const float* logits, const float* temperature, const float* uniform, int* out, void* workspace, int n_rows,
+                          int vocab, hipStream_t stream) {
     if (n_rows <= 0) return 0;
-    sample_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, temperature, uniform, out, vocab);
+    const int chunks = lsa_sample_chunks(vocab);
+    const int chunk_len = ((vocab + chunks - 1) / chunks + 63) / 64 * 64;
+    sample_chunks_kernel<<<dim3(n_rows, chunks), 256, 0, stream>>>(logits, temperature, (ChunkStat*)workspace, vocab, chunk_len);
+    int err = (int)hipGetLastError();
+    if (err) return err;
+    sample_pick_kernel<<<n_rows, 64, 0, stream>>>(logits, temperature, uniform, (const ChunkStat*)workspace, out, vocab, chunk_len, chunks);
     LSA_LAUNCH_CHECK();
 }

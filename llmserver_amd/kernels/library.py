@@ -15,12 +15,15 @@ _SIGNATURES = {
     "lsa_add_bias": [c_int, _P, _P, c_int, c_int, _P],
     "lsa_qk_norm_rope_kv_write": [c_int, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int,
                                   c_int, c_int, _P],
-    "lsa_sample": [_P, _P, _P, _P, c_int, c_int, _P],
+    "lsa_sample": [_P, _P, _P, _P, _P, c_int, c_int, _P],
+    "lsa_sample_chunks": [c_int],
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, _P, _P, _P, c_int,
                             c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
     "lsa_attention_head_dim": [],
     "lsa_attention_is_bf16": [],
     "lsa_gemm_skinny": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_gemm_skinny_swiglu": [_P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_gemm_skinny_norm": [c_int, _P, _P, _P, c_float, _P, _P, _P, c_int, c_int, c_int, _P],
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

@@ -115,7 +115,7 @@ class DecoderModel:
         resid = self.embedding.forward(ctx.token_ids, ctx)
         delta = None
         for call in self.order:
-            delta = self.blocks[call.block].forward(resid, delta, ctx, caches.view(call))
+            resid, delta = self.blocks[call.block].forward(resid, delta, ctx, caches.view(call))
         if ctx.n_out == 0:
             return torch.empty((0, self.head.out_features), device=resid.device, dtype=torch.float32)
         selected = self.final_norm.add_norm(resid, delta, ctx, rows=ctx.logit_idx)

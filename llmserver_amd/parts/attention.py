@@ -130,6 +130,7 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
 
 class GQAttention(Mixer):
     graph_safe = True
+    accepts_pending_norm = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  qk_norm_eps: Optional[float] = None, bias: bool = False, out_bias: Optional[bool] = None,
@@ -197,9 +198,9 @@ class GQAttention(Mixer):
         ctx.ops.qk_norm_rope_kv_write(
             qkv, cache.keys, cache.values, table, ctx.token_row, ctx.positions,
             self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
-            self.position.rotary_table(x.device), cache.page_size, self.n_heads, self.n_kv_heads, self.head_dim,
+            self.position.rotary_table(qkv.device), cache.page_size, self.n_heads, self.n_kv_heads, self.head_dim,
             cache.writable)
-        out = ctx.empty((x.shape[0], self.n_heads * self.head_dim))
+        out = ctx.empty((qkv.shape[0], self.n_heads * self.head_dim))
         ctx.ops.paged_attention(
             qkv, out, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
             ctx.get_plan(self.plan_key()), self.scale, self.window, cache.page_size,

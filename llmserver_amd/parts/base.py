@@ -70,6 +70,28 @@ class Norm(Part):
         raise NotImplementedError
 
 
+class PendingNorm:
+    """A normalisation that has not run yet: ``norm(resid + delta)``.
+
+    A part that starts with a projection can hand this to its :class:`~llmserver_amd.parts.linear.Linear`,
+    which may compute the sum, the norm and the product in one kernel.  ``tensor()`` carries the
+    normalisation out the plain way.  Afterwards ``resid`` is the residual stream with ``delta`` added."""
+
+    def __init__(self, norm: "Norm", resid, delta, ctx):
+        self.norm, self.resid, self.delta, self.ctx = norm, resid, delta, ctx
+        self._done = None
+
+    def tensor(self):
+        if self._done is None:
+            self._done = self.norm.add_norm(self.resid, self.delta, self.ctx)
+            self.delta = None
+        return self._done
+
+    def consumed(self, resid_after):
+        """A fused kernel has used the pending sum; ``resid_after`` holds ``resid + delta``."""
+        self.resid, self.delta = resid_after, None
+
+
 class PositionEncoding(Part):
     """How token positions enter a mixer.  ``rotary_table()`` returns the float32 inverse
     frequencies ``[rotary_dim/2]`` of a rotate-half rotation, or None if nothing is rotated."""
@@ -85,6 +107,8 @@ class Mixer(Part):
     # staged arrays (no host-side loops over rows, no host reads): such a step can be captured
     # into a graph once and replayed.
     graph_safe = False
+    # True if ``forward`` passes its input straight to a Linear and so can take a PendingNorm.
+    accepts_pending_norm = False
 
     def cache_spec(self):
         """:class:`PagedKVSpec`, :class:`StateSpec` or None."""
@@ -99,6 +123,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_pending_norm = False
+
     def forward(self, x, ctx):
         raise NotImplementedError
 

@@ -29,8 +29,21 @@ class PreNormBlock(Block):
         for part in self._parts().values():
             part.finalize()
 
+    @staticmethod
+    def _feed(norm, consumer, resid, delta, ctx, *args):
+        """Run ``consumer`` on ``norm(resid + delta)``; returns ``(resid + delta, consumer's output)``.
+
+        A consumer that starts with a projection gets the normalisation still pending, so that the
+        projection's kernel may do the sum and the norm itself (few rows); otherwise the norm runs
+        first, in its own kernel."""
+        if consumer.accepts_pending_norm and hasattr(norm, "defer"):
+            pending = norm.defer(resid, delta, ctx)
+            out = consumer.forward(pending, ctx, *args)
+            if pending.delta is not None:          # nobody used it: the update must still be added
+                pending.tensor()
+            return pending.resid, out
+        return resid, consumer.forward(norm.add_norm(resid, delta, ctx), ctx, *args)
+
     def forward(self, resid, delta, ctx, cache):
-        normed = self.mixer_norm.add_norm(resid, delta, ctx)
-        mixed = self.mixer.forward(normed, ctx, cache)
-        normed = self.ffn_norm.add_norm(resid, mixed, ctx)
-        return self.ffn.forward(normed, ctx)
+        resid, mixed = self._feed(self.mixer_norm, self.mixer, resid, delta, ctx, cache)
+        return self._feed(self.ffn_norm, self.ffn, resid, mixed, ctx)

@@ -12,7 +12,7 @@ from typing import Dict, List, Sequence
 
 import torch
 
-from .base import MATRIX, VECTOR, ParamSpec, Part
+from .base import MATRIX, VECTOR, ParamSpec, Part, PendingNorm
 
 
 class Linear(Part):
@@ -62,6 +62,19 @@ class Linear(Part):
         self._b.clear()
 
     def forward(self, x, ctx, out=None):
+        if isinstance(x, PendingNorm):
+            fused = getattr(ctx.ops, "norm_linear", None)
+            weight = getattr(x.norm, "weight", None)
+            done = None
+            if fused is not None and x._done is None and weight is not None and hasattr(x.norm, "eps"):
+                done = fused(x.resid, x.delta, weight, x.norm.eps, self.weight, self.out_float32)
+            if done is not None:
+                y, resid_after = done
+                x.consumed(resid_after)
+                if self.bias is not None:
+                    ctx.ops.add_bias_(y, self.bias)
+                return y
+            x = x.tensor()
         y = ctx.ops.linear(x, self.weight, out=out, out_float32=self.out_float32)
         if self.bias is not None:
             ctx.ops.add_bias_(y, self.bias)

@@ -11,6 +11,8 @@ from .linear import Linear
 
 
 class GatedMLP(FeedForward):
+    accepts_pending_norm = True
+
     def __init__(self, width: int, intermediate: int, activation: str = "silu", bias: bool = False):
         if activation not in ("silu", "swish"):
             raise ValueError(f"Unsupported activation {activation!r}; supported: ['silu', 'swish']")
@@ -31,6 +33,11 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, ctx):
         gate_up = self.gate_up.forward(x, ctx)
-        hidden = ctx.empty((x.shape[0], self.intermediate))
+        fused = getattr(ctx.ops, "swiglu_linear", None)
+        if fused is not None and self.down.bias is None:
+            y = fused(gate_up, self.down.weight)          # few rows: activation inside the down projection's kernel
+            if y is not None:
+                return y
+        hidden = ctx.empty((gate_up.shape[0], self.intermediate))
         ctx.ops.swiglu(gate_up, hidden)
         return self.down.forward(hidden, ctx)

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import VECTOR, Norm, ParamSpec
+from .base import VECTOR, Norm, ParamSpec, PendingNorm
 
 
 class RMSNorm(Norm):
@@ -30,3 +30,7 @@ class RMSNorm(Norm):
         out = ctx.empty((n, self.width))
         ctx.ops.add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
         return out
+
+    def defer(self, resid, delta, ctx) -> PendingNorm:
+        """The same normalisation, left to whoever consumes it (a projection may fuse it)."""
+        return PendingNorm(self, resid, delta, ctx)

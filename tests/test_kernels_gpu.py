@@ -298,3 +298,37 @@ def test_skinny_gemm(ops, rows, n, k):
         ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, None)
         if ops._gemm_refusal_check != 0:
             raise RuntimeError("refused")
+
+
+@pytest.mark.parametrize("rows", [1, 5, 8])
+@pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (6144, 1000)])
+def test_skinny_gemm_with_fused_prologues(ops, rows, n, k):
+    """The few-row product with the activation or the residual sum and norm inside it, against the
+    separate kernels' twins."""
+    print(f"fused prologues rows {rows} n {n} k {k}", flush=True)
+    torch.manual_seed(rows + n + k)
+    w = (torch.randn(n, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
+    gate_up = (2 * torch.randn(rows, 2 * k, device=DEV)).to(torch.bfloat16)
+    hidden = torch.empty(rows, k, device=DEV, dtype=torch.bfloat16)
+    TorchOps().swiglu(gate_up, hidden)
+    expected = (hidden.double() @ w.double().t()).float()
+    got = ops.swiglu_linear(gate_up, w, force=True)
+    torch.testing.assert_close(got.float(), expected, atol=3e-2, rtol=2e-2)
+
+    resid = (3 * torch.randn(rows, k, device=DEV)).to(torch.bfloat16)
+    delta = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
+    norm_weight = 1 + 0.2 * torch.randn(k, device=DEV)
+    for d in (delta, None):
+        ref_resid, normed = resid.clone(), torch.empty_like(resid)
+        TorchOps().add_rmsnorm(ref_resid, d, norm_weight, 1e-5, normed)
+        expected = (normed.double() @ w.double().t()).float()
+        for out32 in (False, True):
+            kept = resid.clone()
+            got, after = ops.norm_linear(kept, d, norm_weight, 1e-5, w, out_float32=out32, force=True)
+            assert torch.equal(kept, resid)                                  # the input stream is not written
+            assert torch.equal(after, ref_resid)                             # the sum is rounded once, identically
+            assert (after.data_ptr() == kept.data_ptr()) == (d is None)
+            assert got.dtype == (torch.float32 if out32 else torch.bfloat16)
+            torch.testing.assert_close(got.float(), expected, atol=3e-2, rtol=2e-2)
+    assert ops.swiglu_linear(torch.zeros(9, 2 * k, device=DEV, dtype=torch.bfloat16), w, force=True) is None          # too many rows: not fused
+    assert ops.norm_linear(torch.zeros(9, k, device=DEV, dtype=torch.bfloat16), None, norm_weight, 1e-5, w, force=True) is None

@@ -110,10 +110,21 @@ def test_attention_part_and_block(dtype, bias):
             if what == "attention":
                 outs.append(attention.forward(chunk, ctx, view).double().cpu())
             else:
-                resid = chunk.clone()
-                delta = block.forward(resid, None, ctx, view)
+                resid, delta = block.forward(chunk.clone(), None, ctx, view)
                 outs.append((resid.double() + delta.double()).cpu())
             cache.advance("r", end)
         got = torch.cat(outs)
         expected = expected_attention if what == "attention" else expected_block
         assert float((got - expected).abs().max()) < TOL[dtype] * (4 if what == "attention" else 10), what
+
+
+def test_block_with_fused_prologues_switched_on():
+    """The same block with the sum + norm and the activation inside the few-row products."""
+    from llmserver_amd.kernels import default_ops
+    ops = default_ops()
+    ops.fuse_prologues = True
+    try:
+        test_attention_part_and_block(torch.bfloat16, True)
+        test_attention_part_and_block(torch.bfloat16, False)
+    finally:
+        ops.fuse_prologues = False
