@@ -208,24 +208,36 @@ class CacheManager:
         payload = json.dumps([parent, list(tokens), self.model_identity, "none"], separators=(",", ":")).encode("utf-8")
         return hashlib.sha256(payload).hexdigest()
 
-    def share_prefix(self, request_id, prompt: Sequence[int]) -> int:
+    def prefix_digests(self, prompt: Sequence[int]) -> List[str]:
+        """The chained digests of the prompt's complete pages that may be shared (at least one
+        prompt token always remains to be computed)."""
+        digests, parent = [], "root"
+        for block in range((len(prompt) - 1) // self.page_size):
+            parent = self.digest(parent, prompt[block * self.page_size:(block + 1) * self.page_size])
+            digests.append(parent)
+        return digests
+
+    def share_prefix(self, request_id, prompt: Sequence[int], digests: Optional[List[str]] = None) -> int:
         """Attach the longest chain of cached complete pages; always leaves at least one prompt
-        token to compute (/root/reference/utils/engine.py:197-208).  Returns tokens covered."""
+        token to compute (/root/reference/utils/engine.py:197-208).  May be called again while
+        the request has computed nothing itself: the chain is then continued.  Returns the
+        tokens newly covered."""
         if not self.prefix_caching_possible:
             return 0
         record = self.record(request_id)
-        if any(record.tables[group.index] for group in self.groups):
-            raise CacheStateError("a prefix can only be shared into an empty block table")
-        parent, covered = "root", 0
-        for block in range((len(prompt) - 1) // self.page_size):
-            digest = self.digest(parent, prompt[block * self.page_size:(block + 1) * self.page_size])
+        have = len(record.tables[0])
+        if any(len(record.tables[group.index]) != have for group in self.groups) or record.num_computed != have * self.page_size:
+            raise CacheStateError("a prefix can only be shared into a block table that holds shared pages only")
+        if digests is None:
+            digests = self.prefix_digests(prompt)
+        covered = 0
+        for digest in digests[have:]:
             if any(group.pool.find(digest) is None for group in self.groups):
                 break
             for group in self.groups:
                 group.pool.share(digest, record.tables[group.index])
             covered += self.page_size
-            parent = digest
-        record.num_computed = covered
+        record.num_computed += covered
         return covered
 
     def register_prefix(self, request_id, prompt: Sequence[int], old_computed: int, new_computed: int) -> None:

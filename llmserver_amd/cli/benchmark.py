@@ -77,6 +77,12 @@ def main(argv=None) -> int:
     parser.add_argument("--prefill-chunk-size", type=int, default=None)
     parser.add_argument("--temperature", type=float, default=0.0)
     parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--mixed-requests", type=int, default=0,
+                        help="instead of the matrix: this many concurrent requests under continuous batching with chunked prefill")
+    parser.add_argument("--mixed-prompt-range", default="16,2048", help="prompt lengths of the mixed workload, uniform in [lo, hi]")
+    parser.add_argument("--shared-prefix-tokens", type=int, default=512, help="length of the prefix that some mixed requests share")
+    parser.add_argument("--shared-fraction", type=float, default=0.5, help="fraction of mixed requests that start with the shared prefix")
+    parser.add_argument("--max-batch-size", type=int, default=None, help="requests running at a time (default: the largest batch)")
     parser.add_argument("--profile", action="store_true", help="print the engine's per-phase step counters")
     parser.add_argument("--json", default=None, help="write the results to this file")
     args = parser.parse_args(argv)
@@ -102,6 +108,9 @@ def main(argv=None) -> int:
     print(f"loaded {model.name} in {time.perf_counter() - started:.1f} s", flush=True)
     vocab = model.config.vocab_size
     prompt_lengths, batches = parse_ints(args.prompt_tokens), parse_ints(args.batch_sizes)
+    if args.mixed_requests:
+        low, high = parse_ints(args.mixed_prompt_range)
+        prompt_lengths, batches = [high], [args.max_batch_size or args.mixed_requests]
     max_batch, max_length = max(batches), max(prompt_lengths) + args.output_tokens
     bytes_per_block = CacheManager.bytes_per_token(model.cache_specs(), model.dtype) * args.block_size
     wanted = max_batch * math.ceil(max_length / args.block_size) + 8          # /root/reference/benchmark_cuda.py:107-111
@@ -111,6 +120,34 @@ def main(argv=None) -> int:
                     kv_cache_num_blocks=wanted, kv_cache_block_size=args.block_size, stream_text=False, max_completed_requests=0,
                     ignore_eos=True, temperature=args.temperature, seed=args.seed, enable_prefix_caching=True)
     results = []
+    if args.mixed_requests:
+        import random
+        rng = random.Random(args.seed)
+        prefix = build_prompts(vocab, args.shared_prefix_tokens, 1, "shared-prefix", args.seed)[0]
+        prompts = []
+        for index in range(args.mixed_requests):
+            length = rng.randint(low, high)
+            body = build_prompts(vocab, length, 1, f"mixed-{index}", args.seed)[0]
+            if index < args.shared_fraction * args.mixed_requests and length > args.shared_prefix_tokens:
+                body = prefix + body[args.shared_prefix_tokens:]
+            prompts.append(body)
+        rng.shuffle(prompts)
+        run_once(engine, build_prompts(vocab, 64, min(4, max_batch), "warm-mixed", args.seed), 4)
+        for key in ("steps", "decode_steps", "prefill_steps", "tokens", "prefix_hit_tokens", "preemptions"):
+            engine.step_profile[key] = 0
+        seconds, generated = run_once(engine, prompts, args.output_tokens)
+        prompt_total = sum(len(p) for p in prompts)
+        entry = {"workload": "mixed", "requests": args.mixed_requests, "prompt_tokens_total": prompt_total,
+                 "output_tokens": args.output_tokens, "total_s": seconds,
+                 "generated_tok_s": args.mixed_requests * args.output_tokens / seconds,
+                 "processed_tok_s": (prompt_total + args.mixed_requests * args.output_tokens) / seconds,
+                 "prefix_hit_tokens": engine.step_profile["prefix_hit_tokens"], "steps": engine.step_profile["steps"],
+                 "preemptions": engine.step_profile["preemptions"]}
+        print(f"mixed: {args.mixed_requests} requests, {prompt_total} prompt tokens ({entry['prefix_hit_tokens']} served from cached prefix pages), "
+              f"{args.output_tokens} new tokens each: {seconds:.3f} s, {entry['generated_tok_s']:.1f} generated tok/s, "
+              f"{entry['processed_tok_s']:.1f} processed tok/s, {entry['steps']} steps, {entry['preemptions']} preemptions", flush=True)
+        results.append(entry)
+        prompt_lengths = []
     for prompt_length in prompt_lengths:
         for batch in batches:
             entry = {"prompt_tokens": prompt_length, "batch": batch, "output_tokens": args.output_tokens}

@@ -131,10 +131,19 @@ class Engine:
         (/root/reference/utils/engine.py:197-208)."""
         record = self.kv_cache.open(request.request_id)
         request.block_table = record.tables[0] if record.tables else []
-        if self.enable_prefix_caching:
-            covered = self.kv_cache.share_prefix(request.request_id, request.prompt_token_ids)
-            request.num_computed_tokens += covered
-            self.step_profile["prefix_hit_tokens"] += covered
+        self._share_prefix(request)
+
+    def _share_prefix(self, request: Request) -> None:
+        """Attach cached pages of the prompt's prefix.  Done when the request arrives, as in the
+        reference, and again each time it is up for admission, because requests that arrived
+        together may by then find what an earlier one of them has computed."""
+        if not self.enable_prefix_caching:
+            return
+        if request.prefix_digests is None:
+            request.prefix_digests = self.kv_cache.prefix_digests(request.prompt_token_ids)
+        covered = self.kv_cache.share_prefix(request.request_id, request.prompt_token_ids, request.prefix_digests)
+        request.num_computed_tokens += covered
+        self.step_profile["prefix_hit_tokens"] += covered
 
     # -- history -----------------------------------------------------------------------------
     def prune_completed_requests(self, now=None):
@@ -227,6 +236,8 @@ class Engine:
             for request in self.scheduler.waiting:      # a preempted request gets a fresh table (and any cached prefix) back
                 if not self.kv_cache.has(request.request_id):
                     self._open_cache(request)
+                elif request.num_computed_tokens < len(request.prefix_digests or ()) * self.block_size:
+                    self._share_prefix(request)
             available = self.available_blocks()
             out = self.scheduler.plan(available, self.block_size)
             needed = sum(max(0, math.ceil((r.num_computed_tokens + n) / self.block_size) - len(r.block_table))

@@ -10,18 +10,21 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("case", ["A", "B"])
-def test_replayed_steps_equal_eager_steps(case, dtype):
+@pytest.mark.parametrize("case, n_live", [("A", 3), ("B", 3), ("B", 12)])
+def test_replayed_steps_equal_eager_steps(case, n_live, dtype):
+    """Three rows keep the products in the hand-written few-row kernel; twelve rows put the
+    library's products inside the captured graph."""
     from llmserver_amd.cache import CacheManager
     from llmserver_amd.engine import ModelRunner, StepEntry, load_model
-    print(f"graph replay {case} {dtype}", flush=True)
+    print(f"graph replay {case} {n_live} rows {dtype}", flush=True)
     raw, _, page = CASES[case]
     model = load_model(model_folder(case), "cuda", dtype)
     runners = []
     for use_graphs in (True, False):
         cache = CacheManager(model.cache_specs(), page, 200, device="cuda", dtype=model.dtype)
         runners.append(ModelRunner(model, cache, use_graphs=use_graphs))
-    prompts = {"a": random_tokens(raw["vocab_size"], 37, 1), "b": random_tokens(raw["vocab_size"], 5, 2), "c": random_tokens(raw["vocab_size"], 64, 3)}
+    lengths = [37, 5, 64, 1, 90, 16, 17, 33, 2, 70, 48, 9][:n_live]
+    prompts = {f"r{i}": random_tokens(raw["vocab_size"], n, 1 + i) for i, n in enumerate(lengths)}
     feed = {rid: random_tokens(raw["vocab_size"], 80, 10 + i) for i, rid in enumerate(prompts)}
     for runner in runners:
         for rid, tokens in prompts.items():
@@ -29,7 +32,7 @@ def test_replayed_steps_equal_eager_steps(case, dtype):
             runner.step([StepEntry(rid, tokens, [])])
     worst = 0.0
     for turn in range(70):
-        live = ["a", "b", "c"] if turn % 9 else ["a", "c"]             # another number of rows now and then: another graph
+        live = list(prompts) if turn % 9 else list(prompts)[::2]        # another number of rows now and then: another graph
         entries = [StepEntry(rid, [feed[rid][turn]], [0]) for rid in live]
         outs = [runner.step(entries).clone() for runner in runners]
         torch.cuda.synchronize()

@@ -315,3 +315,22 @@ def test_real_model_under_a_small_budget_and_few_pages_generates_the_same_tokens
         engine.kv_cache.check_invariants()
         assert min(engine.kv_cache.available_pages()) == pages
     assert engine.step_profile["preemptions"] > 0
+
+
+def test_requests_that_arrive_together_share_what_the_first_of_them_computed():
+    """Both arrive before any step; only one fits into the first step; when the second is admitted it
+    finds the first one's complete prompt pages and computes the rest only."""
+    prompt = list(range(10, 20))
+    engine, script = scripted_engine([[50], [51, 60]], max_batch_size=2, max_num_batched_tokens=10, kv_cache_num_blocks=8,
+                                     kv_cache_block_size=4)
+    first, second = engine.add_request(None, prompt), engine.add_request(None, prompt)
+    assert second.num_computed_tokens == 0
+    engine.step()
+    assert script.calls[0]["requests"] == [first.request_id]
+    engine.step()
+    call = script.calls[1]
+    assert call["requests"] == [first.request_id, second.request_id]
+    assert call["tokens"][1] == prompt[8:] and call["start"][1] == 8
+    assert second.block_table[:2] == first.block_table[:2]
+    assert engine.step_profile["prefix_hit_tokens"] == 8
+    engine.kv_cache.check_invariants()
