@@ -76,6 +76,7 @@ class StepContext:
     def __init__(self, ops, device, dtype, staging: Staging):
         self.ops, self.device, self.dtype, self.staging = ops, torch.device(device), dtype, staging
         self._plans: Dict[object, dict] = {}
+        self._computed: Dict[object, object] = {}
         self._tables: Dict[int, torch.Tensor] = {}
         self.static_max_keys: Optional[int] = None      # set when the step's array shapes must be fixed (graph capture)
 
@@ -121,6 +122,17 @@ class StepContext:
 
     def block_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
+
+    def computed(self, key, make):
+        """A value computed on the device once per run of the step's kernels (e.g. the rotation
+        table of a position encoding), shared by all layers that ask for it under ``key``."""
+        if key not in self._computed:
+            self._computed[key] = make()
+        return self._computed[key]
+
+    def forget_computed(self):
+        """Before the step's kernels are recorded again (graph capture after an eager run)."""
+        self._computed.clear()
 
     def has_plan(self, key) -> bool:
         return key in self._plans

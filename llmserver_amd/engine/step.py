@@ -130,6 +130,7 @@ class ModelRunner:
             ctx.static_max_keys = key[1] * self.cache.page_size
             logits = self.model.forward(ctx, self.cache)              # this step's result, run eagerly
             torch.cuda.synchronize(self.device)
+            ctx.forget_computed()                # what the eager run computed on the device must be recorded too
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 static_logits = self.model.forward(ctx, self.cache)   # recorded, not run

@@ -15,6 +15,7 @@ _SIGNATURES = {
     "lsa_add_bias": [c_int, _P, _P, c_int, c_int, _P],
     "lsa_qk_norm_rope_kv_write": [c_int, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int,
                                   c_int, c_int, _P],
+    "lsa_rotary_table": [_P, _P, _P, c_int, c_int, _P],
     "lsa_sample": [_P, _P, _P, _P, _P, c_int, c_int, _P],
     "lsa_sample_chunks": [c_int],
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, _P, _P, _P, c_int,

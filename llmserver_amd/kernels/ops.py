@@ -176,7 +176,16 @@ class HipOps:
         _check(bias, "bias", torch.float32, (width,))
         _launched(self._elementwise.lsa_add_bias(_code(y), _ptr(y), _ptr(bias), n, width, _stream()), "add_bias")
 
-    def qk_norm_rope_kv_write(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, inv_freq,
+    def rotary_table(self, positions, inv_freq):
+        """cos and sin of ``position * inv_freq`` for every token: float32 ``[T, 2 * len(inv_freq)]``, cos first."""
+        n, half = positions.shape[0], inv_freq.shape[0]
+        _check(positions, "positions", torch.int32)
+        _check(inv_freq, "inv_freq", torch.float32)
+        out = torch.empty((n, 2 * half), device=positions.device, dtype=torch.float32)
+        _launched(self._rope_kv.lsa_rotary_table(_ptr(positions), _ptr(inv_freq), _ptr(out), half, n, _stream()), "rotary_table")
+        return out
+
+    def qk_norm_rope_kv_write(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin,
                               page_size, n_q, n_kv, head_dim, write_cache=True):
         n = qkv.shape[0]
         _check(qkv, "qkv", None, (n, (n_q + 2 * n_kv) * head_dim))
@@ -196,11 +205,11 @@ class HipOps:
                 _check(w, name, torch.float32, (head_dim,))
         if (q_weight is None) != (k_weight is None):
             raise ValueError("q and k norm weights must come together")
-        if inv_freq is not None:
-            _check(inv_freq, "inv_freq", torch.float32, (head_dim // 2,))
+        if cos_sin is not None:
+            _check(cos_sin, "cos_sin", torch.float32, (n, head_dim))
         _launched(self._rope_kv.lsa_qk_norm_rope_kv_write(
             _code(qkv), _ptr(qkv), _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(token_row), _ptr(positions),
-            _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(inv_freq), page_size, n_q, n_kv, head_dim,
+            _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), page_size, n_q, n_kv, head_dim,
             1 if write_cache else 0, n, _stream()), "qk_norm_rope_kv_write")
 
     def _attention_library(self, dtype, head_dim):

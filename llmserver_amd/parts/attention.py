@@ -198,7 +198,7 @@ class GQAttention(Mixer):
         ctx.ops.qk_norm_rope_kv_write(
             qkv, cache.keys, cache.values, table, ctx.token_row, ctx.positions,
             self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
-            self.position.rotary_table(qkv.device), cache.page_size, self.n_heads, self.n_kv_heads, self.head_dim,
+            self.position.cos_sin(ctx), cache.page_size, self.n_heads, self.n_kv_heads, self.head_dim,
             cache.writable)
         out = ctx.empty((qkv.shape[0], self.n_heads * self.head_dim))
         ctx.ops.paged_attention(

@@ -99,6 +99,10 @@ class PositionEncoding(Part):
     def rotary_table(self, device) -> Optional[torch.Tensor]:
         return None
 
+    def cos_sin(self, ctx) -> Optional[torch.Tensor]:
+        """float32 ``[T, rotary_dim]`` (cos of every pair, then sin) for the step's tokens, or None."""
+        return None
+
 
 class Mixer(Part):
     """Token mixer: reads and writes its own cache through the view the step gives it."""

@@ -33,6 +33,11 @@ class RotaryPosition(PositionEncoding):
             self._tables[key] = self.inverse_frequencies().to(device=device, dtype=torch.float32).contiguous()
         return self._tables[key]
 
+    def cos_sin(self, ctx):
+        """cos and sin of the step's tokens, float32 ``[T, rotary_dim]``: computed once a step, whatever
+        the number of layers that rotate with this encoding."""
+        return ctx.computed(("rotary", id(self)), lambda: ctx.ops.rotary_table(ctx.positions, self.rotary_table(ctx.device)))
+
 
 class NoPosition(PositionEncoding):
     """Tokens enter the mixer unrotated."""

@@ -96,11 +96,12 @@ def make_cache(n_pages, n_kv, page, d, dtype):
 def test_qk_norm_rope_kv_write(ops, dtype, n_q, n_kv, d, page):
     print(f"qk_norm_rope_kv_write {dtype} {n_q}/{n_kv} d{d} page{page}", flush=True)
     torch.manual_seed(d + n_q)
-    lens, starts = [5, 1, 23], [0, 700, 37]                        # a fresh prompt, a decoded token far out, a later portion
+    lens, starts = ([5, 1, 23], [0, 700, 37]) if d != 128 else ([300, 1, 23], [401, 1, 37])    # portions and decoded tokens; a long portion
     rows = len(lens)
     n_pages = 200 if page < 500 else 8
     width = max(-(-(s + n) // page) for s, n in zip(starts, lens))
     table = torch.full((rows, width), -1, dtype=torch.int32)
+    n_pages = max(n_pages, sum(-(-(s + n) // page) for s, n in zip(starts, lens)) + 2)
     perm = torch.randperm(n_pages)
     used = 0
     for r, (s, n) in enumerate(zip(starts, lens)):
@@ -114,11 +115,13 @@ def test_qk_norm_rope_kv_write(ops, dtype, n_q, n_kv, d, page):
     qw, kw = 1 + 0.2 * torch.randn(d, device=DEV), 1 + 0.2 * torch.randn(d, device=DEV)
     inv_freq = (1.0 / (1e6 ** (torch.arange(0, d, 2).float() / d))).to(DEV)
     table, positions, token_row = table.to(DEV), positions.to(DEV), token_row.to(DEV)
+    cos_sin = ops.rotary_table(positions, inv_freq)
+    torch.testing.assert_close(cos_sin, TorchOps().rotary_table(positions, inv_freq), atol=2e-6, rtol=0)
     for norm, rope, write in ((True, True, True), (False, True, True), (True, False, True), (True, True, False)):
         got_qkv, ref_qkv = qkv.clone(), qkv.clone()
         got_k, got_v = make_cache(n_pages, n_kv, page, d, dtype)
         ref_k, ref_v = make_cache(n_pages, n_kv, page, d, dtype)
-        args = (table, token_row, positions, qw if norm else None, kw if norm else None, 1e-6, inv_freq if rope else None, page, n_q, n_kv, d, write)
+        args = (table, token_row, positions, qw if norm else None, kw if norm else None, 1e-6, cos_sin if rope else None, page, n_q, n_kv, d, write)
         ops.qk_norm_rope_kv_write(got_qkv, got_k, got_v, *args)
         TorchOps().qk_norm_rope_kv_write(ref_qkv, ref_k, ref_v, *args)
         close(got_qkv[:, :n_q * d], ref_qkv[:, :n_q * d], dtype)

@@ -52,7 +52,11 @@ class TorchOps:
     def add_bias_(self, y, bias):
         y.copy_((y.float() + bias).to(y.dtype))
 
-    def qk_norm_rope_kv_write(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, inv_freq,
+    def rotary_table(self, positions, inv_freq):
+        angles = positions.float()[:, None] * inv_freq[None, :]
+        return torch.cat([torch.cos(angles), torch.sin(angles)], dim=1)
+
+    def qk_norm_rope_kv_write(self, qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin,
                               page_size, n_q, n_kv, head_dim, write_cache=True):
         n = qkv.shape[0]
         heads = qkv.view(n, n_q + 2 * n_kv, head_dim)
@@ -60,10 +64,9 @@ class TorchOps:
         if q_weight is not None:
             weight = torch.cat([q_weight.expand(n_q, -1), k_weight.expand(n_kv, -1)], dim=0)
             qk = qk * torch.rsqrt(qk.pow(2).mean(dim=-1, keepdim=True) + eps) * weight
-        if inv_freq is not None:
-            angles = positions.float()[:, None] * inv_freq[None, :]
-            cos, sin = torch.cos(angles)[:, None, :], torch.sin(angles)[:, None, :]
+        if cos_sin is not None:
             half = head_dim // 2
+            cos, sin = cos_sin[:, None, :half], cos_sin[:, None, half:]
             x1, x2 = qk[..., :half], qk[..., half:]
             qk = torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
         heads[:, :n_q] = qk[:, :n_q].to(qkv.dtype)
