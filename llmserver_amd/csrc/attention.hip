@@ -374,8 +374,13 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES) void paged_attention_tile_
     const Item* __restrict__ tiles, Geometry g) {
     __shared__ __attribute__((aligned(16))) unsigned char lds[2][K_TILE_BYTES + V_TILE_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const Item tile = tiles[blockIdx.x];
-    const int kv_head = blockIdx.y / g.gtiles, gtile = blockIdx.y % g.gtiles;
+    // Workgroups are handed to the eight XCDs in turn, and each XCD has its own L2: with the KV head
+    // running fastest over the workgroup index, an XCD keeps meeting the same few KV heads, whose
+    // keys and values then stay in its L2 for all the tiles that read them.
+    const int heads = g.n_kv * g.gtiles;
+    const Item tile = tiles[blockIdx.x / heads];
+    const int head_index = blockIdx.x % heads;
+    const int kv_head = head_index / g.gtiles, gtile = head_index % g.gtiles;
     const int col = lane & 15, quad = lane >> 4;
     const int row = tile.row;
     const int n = row_len[row], first_pos = row_ctx[row] - n;
@@ -673,7 +678,7 @@ LSA_EXPORT int lsa_paged_attention(
     g.page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     if (n_tiles > 0) {
 #if LSA_BF16
-        dim3 tgrid(n_tiles, n_kv * gtiles);
+        dim3 tgrid(n_tiles * n_kv * gtiles);
         paged_attention_tile_kernel<<<tgrid, 256, 0, stream>>>(
             (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
             row_start, row_len, row_ctx, (const Item*)tiles, g);

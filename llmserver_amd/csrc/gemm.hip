@@ -34,7 +34,11 @@ struct Prologue {
     float eps;
 };
 
-template <int MT, typename OutT, int PRO>
+// GATED: W stacks a gate matrix on an up matrix ([2I, K], gate first) and the result wanted is
+// silu(x . gate^T) * (x . up^T), [M, I].  A workgroup then takes 8 gate rows and the 8 up rows that
+// belong to them as its 16 rows of W, so both halves of a product meet in its epilogue and the
+// activation costs no launch and no trip of the [M, 2I] intermediate through memory.
+template <int MT, typename OutT, int PRO, bool GATED = false>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                       OutT* __restrict__ y, int M, int N, int K, Prologue pro) {
     constexpr int CH = (PRO != PLAIN || MT > 2) ? 4 : 8;          // 32-wide k steps loaded together (one chunk)
@@ -43,11 +47,12 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
     extern __shared__ float norm_weight_lds[];                     // NORM: the norm weights, [K]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, quad = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    const int n0 = blockIdx.x * (GATED ? 8 : 16);
     const int k_per_wave = ((K + GEMM_WAVES - 1) / GEMM_WAVES + 31) / 32 * 32;
     const int k_begin = min(K, wave * k_per_wave), k_end = min(K, k_begin + k_per_wave);
     const int x_stride = PRO == SWIGLU ? 2 * K : K;
-    const bf16_t* wp = w + (size_t)min(n0 + col, N - 1) * K + 8 * quad;
+    const int w_row = GATED ? (col < 8 ? min(n0 + col, N / 2 - 1) : N / 2 + min(n0 + col - 8, N / 2 - 1)) : min(n0 + col, N - 1);
+    const bf16_t* wp = w + (size_t)w_row * K + 8 * quad;
     const bf16_t* xp[MT];
     const bf16_t* x2p[MT];
 #pragma unroll
@@ -179,6 +184,22 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
             for (int v = 0; v < GEMM_WAVES; ++v) sq += squares[v][t][in_tile >> 4];
             total *= rsqrtf(sq / (float)K + pro.eps);
         }
+        if (GATED) {
+            const int j = in_tile & 15;
+            if (j < 8) {
+                float up = 0.f;
+#pragma unroll
+                for (int v = 0; v < GEMM_WAVES; ++v) up += partial[v][t][in_tile + 8];
+                if (PRO == NORM) {
+                    float sq = 0.f;
+#pragma unroll
+                    for (int v = 0; v < GEMM_WAVES; ++v) sq += squares[v][t][in_tile >> 4];
+                    up *= rsqrtf(sq / (float)K + pro.eps);
+                }
+                if (m < M && n0 + j < N / 2) y[(size_t)m * (N / 2) + n0 + j] = (OutT)(total / (1.f + expf(-total)) * up);
+            }
+            continue;
+        }
         if (m < M && n < N) y[(size_t)m * N + n] = (OutT)total;
     }
 }
@@ -220,4 +241,14 @@ LSA_EXPORT int lsa_gemm_skinny_norm(int out_float32, const void* resid, const vo
     if (M > 16 || K % 8 != 0 || K < 8 || K > 16384 || (delta && resid_out == resid)) return -1;
     Prologue pro = {(const bf16_t*)delta, norm_weight, (bf16_t*)resid_out, eps};
     return out_float32 ? launch<float, NORM>(resid, w, y, M, N, K, pro, stream) : launch<bf16_t, NORM>(resid, w, y, M, N, K, pro, stream);
+}
+
+// hidden[M, I] = silu(x . gate^T) * (x . up^T) with gate_up [2I, K] (gate rows first); M <= 16, I a multiple of 8.
+LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* hidden, int M, int I, int K, hipStream_t stream) {
+    if (M <= 0 || I <= 0) return 0;
+    if (M > 16 || K % 8 != 0 || K < 8 || I % 8 != 0) return -1;
+    Prologue pro = {nullptr, nullptr, nullptr, 0.f};
+    gemm_skinny_kernel<1, bf16_t, PLAIN, true><<<dim3(I / 8), dim3(GEMM_WAVES * 64), 0, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)hidden, M, 2 * I, K, pro);
+    LSA_LAUNCH_CHECK();
 }

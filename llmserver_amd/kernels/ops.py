@@ -103,6 +103,20 @@ class HipOps:
             return torch.mm(x, weight.t(), out_dtype=torch.float32)
         return torch.mm(x, weight.t(), out=out) if out is not None else torch.mm(x, weight.t())
 
+    def linear_gated(self, x, gate_up_weight):
+        """``silu(x @ gate^T) * (x @ up^T)`` with ``gate_up_weight [2I, K]`` in one launch for few rows (the
+        activation sits in the product's epilogue), or None if this is not such a case."""
+        rows, width = x.shape
+        inter = gate_up_weight.shape[0] // 2
+        if x.dtype != torch.bfloat16 or not 0 < rows <= self.skinny_rows or width % 8 or inter % 8 or gate_up_weight.shape[1] != width:
+            return None
+        _check(x, "x", torch.bfloat16)
+        _check(gate_up_weight, "gate_up_weight", torch.bfloat16)
+        out = torch.empty((rows, inter), device=x.device, dtype=torch.bfloat16)
+        _launched(self._gemm.lsa_gemm_skinny_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, _stream()),
+                  "gemm_skinny_gated")
+        return out
+
     def swiglu_linear(self, gate_up, weight, force=False):
         """``(silu(gate) * up) @ weight^T`` in one launch for few rows, or None if this is not such a case."""
         rows, inter = gate_up.shape[0], gate_up.shape[1] // 2

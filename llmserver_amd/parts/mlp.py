@@ -6,7 +6,7 @@ the activation kernel.
 """
 from __future__ import annotations
 
-from .base import FeedForward
+from .base import FeedForward, PendingNorm
 from .linear import Linear
 
 
@@ -32,6 +32,13 @@ class GatedMLP(FeedForward):
         self.down.finalize()
 
     def forward(self, x, ctx):
+        gated = getattr(ctx.ops, "linear_gated", None)
+        if gated is not None and self.gate_up.bias is None and not getattr(ctx.ops, "fuse_prologues", False):
+            tensor = x.tensor() if isinstance(x, PendingNorm) else x
+            hidden = gated(tensor, self.gate_up.weight)       # few rows: the activation in the product's epilogue
+            if hidden is not None:
+                return self.down.forward(hidden, ctx)
+            x = tensor
         gate_up = self.gate_up.forward(x, ctx)
         fused = getattr(ctx.ops, "swiglu_linear", None)
         if fused is not None and self.down.bias is None:

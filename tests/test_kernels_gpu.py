@@ -335,3 +335,18 @@ def test_skinny_gemm_with_fused_prologues(ops, rows, n, k):
             torch.testing.assert_close(got.float(), expected, atol=3e-2, rtol=2e-2)
     assert ops.swiglu_linear(torch.zeros(9, 2 * k, device=DEV, dtype=torch.bfloat16), w, force=True) is None          # too many rows: not fused
     assert ops.norm_linear(torch.zeros(9, k, device=DEV, dtype=torch.bfloat16), None, norm_weight, 1e-5, w, force=True) is None
+
+
+@pytest.mark.parametrize("rows", [1, 5, 8])
+@pytest.mark.parametrize("inter, k", [(8, 16), (104, 72), (12288, 4096), (1000, 1000)])
+def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
+    print(f"gated product rows {rows} inter {inter} k {k}", flush=True)
+    torch.manual_seed(rows + inter + k)
+    x = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
+    gate_up = x.double() @ w.double().t()
+    expected = (torch.nn.functional.silu(gate_up[:, :inter]) * gate_up[:, inter:]).float()
+    got = ops.linear_gated(x, w)
+    assert got.shape == (rows, inter) and got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), expected, atol=2e-2, rtol=2e-2)
+    assert ops.linear_gated(torch.zeros(9, k, device=DEV, dtype=torch.bfloat16), w) is None
