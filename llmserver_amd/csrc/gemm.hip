@@ -38,10 +38,13 @@ struct Prologue {
 // silu(x . gate^T) * (x . up^T), [M, I].  A workgroup then takes 8 gate rows and the 8 up rows that
 // belong to them as its 16 rows of W, so both halves of a product meet in its epilogue and the
 // activation costs no launch and no trip of the [M, 2I] intermediate through memory.
-template <int MT, typename OutT, int PRO, bool GATED = false>
+// CHUNK is the number of 32-wide k steps whose loads are issued together (0: 8 for the plain product
+// of up to 32 rows, else 4); the launcher picks the one that divides a wavefront's share of K with
+// the least waste.
+template <int MT, typename OutT, int PRO, bool GATED = false, int CHUNK = 0>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                       OutT* __restrict__ y, int M, int N, int K, Prologue pro) {
-    constexpr int CH = (PRO != PLAIN || MT > 2) ? 4 : 8;          // 32-wide k steps loaded together (one chunk)
+    constexpr int CH = CHUNK ? CHUNK : (PRO != PLAIN || MT > 2) ? 4 : 8;
     __shared__ float partial[GEMM_WAVES][MT][256];
     __shared__ float squares[GEMM_WAVES][MT][16];
     extern __shared__ float norm_weight_lds[];                     // NORM: the norm weights, [K]
@@ -204,25 +207,182 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
     }
 }
 
+// Two tiles of W per wavefront (32 rows of W per workgroup, or 16 gate rows and their 16 up rows):
+// every slice of X that a wavefront loads then meets twice as much of W, which matters because X,
+// though it comes from cache, competes with the weight stream for the path into the compute unit
+// (at 8 rows of X and one tile, X is a third of what a workgroup loads).  For M <= 16 only, and worth
+// it only where N gives enough workgroups of this size to fill the chip.
+// CH is the number of 32-wide k steps whose loads are issued together; the launcher picks the one
+// that divides a wavefront's share of K with the least waste.
+template <typename OutT, bool GATED, int CH>
+__global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                           OutT* __restrict__ y, int M, int N, int K) {
+    __shared__ float partial[GEMM_WAVES][2][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, quad = lane >> 4;
+    const int half = N / 2;                                        // GATED: rows of the gate matrix
+    const int n0 = blockIdx.x * (GATED ? 16 : 32);
+    const int k_per_wave = ((K + GEMM_WAVES - 1) / GEMM_WAVES + 31) / 32 * 32;
+    const int k_begin = min(K, wave * k_per_wave), k_end = min(K, k_begin + k_per_wave);
+    const int row0 = GATED ? min(n0 + col, half - 1) : min(n0 + col, N - 1);
+    const int row1 = GATED ? half + min(n0 + col, half - 1) : min(n0 + 16 + col, N - 1);
+    const bf16_t* wp0 = w + (size_t)row0 * K + 8 * quad;
+    const bf16_t* wp1 = w + (size_t)row1 * K + 8 * quad;
+    const bf16_t* xp = x + (size_t)min(col, M - 1) * K + 8 * quad;
+    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    struct Chunk {
+        bf16x8 a0[CH], a1[CH], b[CH];
+    };
+    const int k_safe = K - 8;
+    auto load_chunk = [&](Chunk& c, int k0) {
+#pragma unroll
+        for (int u = 0; u < CH; ++u) c.b[u] = *reinterpret_cast<const bf16x8*>(xp + min(k0 + 32 * u + 8 * quad, k_safe) - 8 * quad);
+#pragma unroll
+        for (int u = 0; u < CH; ++u) {
+            const int k = min(k0 + 32 * u + 8 * quad, k_safe) - 8 * quad;
+            c.a0[u] = *reinterpret_cast<const bf16x8*>(wp0 + k);
+            c.a1[u] = *reinterpret_cast<const bf16x8*>(wp1 + k);
+        }
+    };
+    auto multiply_chunk = [&](Chunk& c, int k0) {
+#pragma unroll
+        for (int u = 0; u < CH; ++u) {
+            const bool inside = k0 + 32 * u + 8 * quad < k_end;
+            bf16x8 a0 = c.a0[u], a1 = c.a1[u];
+            if (!inside) {
+                a0 = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+                a1 = a0;
+            }
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, c.b[u], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, c.b[u], acc1, 0, 0, 0);
+        }
+    };
+    if (k_begin < k_end) {
+        constexpr int SPAN = 32 * CH;
+        Chunk p, q;
+        int k0 = k_begin;
+        int chunks = (k_end - k_begin + SPAN - 1) / SPAN;
+        load_chunk(p, k0);
+        while (chunks >= 3) {
+            load_chunk(q, k0 + SPAN);
+            multiply_chunk(p, k0);
+            load_chunk(p, k0 + 2 * SPAN);
+            multiply_chunk(q, k0 + SPAN);
+            k0 += 2 * SPAN;
+            chunks -= 2;
+        }
+        if (chunks == 2) {
+            load_chunk(q, k0 + SPAN);
+            multiply_chunk(p, k0);
+            multiply_chunk(q, k0 + SPAN);
+        } else {
+            multiply_chunk(p, k0);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        partial[wave][0][(4 * quad + r) + 16 * col] = acc0[r];      // [m][n in tile]
+        partial[wave][1][(4 * quad + r) + 16 * col] = acc1[r];
+    }
+    __syncthreads();
+    const int e = threadIdx.x, tile = e >> 8, in_tile = e & 255;
+    const int m = in_tile >> 4, j = in_tile & 15;
+    if (GATED) {
+        if (tile) return;
+        float gate = 0.f, up = 0.f;
+#pragma unroll
+        for (int v = 0; v < GEMM_WAVES; ++v) {
+            gate += partial[v][0][in_tile];
+            up += partial[v][1][in_tile];
+        }
+        if (m < M && n0 + j < half) y[(size_t)m * half + n0 + j] = (OutT)(gate / (1.f + expf(-gate)) * up);
+        return;
+    }
+    float total = 0.f;
+#pragma unroll
+    for (int v = 0; v < GEMM_WAVES; ++v) total += partial[v][tile][in_tile];
+    const int n = n0 + 16 * tile + j;
+    if (m < M && n < N) y[(size_t)m * N + n] = (OutT)total;
+}
+
+// The chunk size in 4..8 that wastes the fewest loads past the end of a wavefront's share of K.
+static int best_chunk(int K) {
+    const int steps = ((K + GEMM_WAVES - 1) / GEMM_WAVES + 31) / 32;          // k steps of one wavefront
+    int chunk = 8, least = 1 << 30;
+    for (int c = 8; c >= 4; --c) {
+        const int waste = (steps + c - 1) / c * c - steps;
+        if (waste < least) {
+            least = waste;
+            chunk = c;
+        }
+    }
+    return chunk;
+}
+
+template <typename OutT, bool GATED>
+static int launch_wide(const bf16_t* x, const bf16_t* w, OutT* y, int M, int N, int K, int workgroups, hipStream_t stream) {
+    const int chunk = best_chunk(K);
+    const dim3 grid(workgroups), block(GEMM_WAVES * 64);
+    switch (chunk) {
+        case 4: gemm_skinny_wide_kernel<OutT, GATED, 4><<<grid, block, 0, stream>>>(x, w, y, M, N, K); break;
+        case 5: gemm_skinny_wide_kernel<OutT, GATED, 5><<<grid, block, 0, stream>>>(x, w, y, M, N, K); break;
+        case 6: gemm_skinny_wide_kernel<OutT, GATED, 6><<<grid, block, 0, stream>>>(x, w, y, M, N, K); break;
+        case 7: gemm_skinny_wide_kernel<OutT, GATED, 7><<<grid, block, 0, stream>>>(x, w, y, M, N, K); break;
+        default: gemm_skinny_wide_kernel<OutT, GATED, 8><<<grid, block, 0, stream>>>(x, w, y, M, N, K); break;
+    }
+    LSA_LAUNCH_CHECK();
+}
+
+// Whether workgroups of two tiles suit `tiles` 16-row tiles of W: they halve the activations' share
+// of the traffic, which saves `gain_percent` of the time (measured: about 15 with the gated epilogue,
+// where one tile means two half tiles; for the plain product about 10 at 9 to 16 rows, 3 at 4 to 8
+// and a loss below that), but must still fill the compute units in whole rounds.
+static bool two_tiles_pay(int M, long tiles, int tiling, int gain_percent) {
+    if (M > 16 || tiling == 1) return false;
+    if (tiling == 2) return true;
+    if (gain_percent <= 0) return false;
+    static int units = 0;
+    if (!units) {
+        int device = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) return false;
+        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    const long rounds_one = (tiles + units - 1) / units, rounds_two = ((tiles + 1) / 2 + units - 1) / units;
+    return 2 * rounds_two * (100 - gain_percent) < rounds_one * 100;
+}
+
 template <typename OutT, int PRO>
-static int launch(const void* x, const void* w, void* y, int M, int N, int K, Prologue pro, hipStream_t stream) {
+static int launch(const void* x, const void* w, void* y, int M, int N, int K, Prologue pro, int tiling, hipStream_t stream) {
     const dim3 grid((N + 15) / 16), block(GEMM_WAVES * 64);
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
+    if (PRO == PLAIN && two_tiles_pay(M, grid.x, tiling, M > 8 ? 10 : M >= 4 ? 3 : 0)) return launch_wide<OutT, false>(xb, wb, (OutT*)y, M, N, K, (N + 31) / 32, stream);
     const size_t lds = PRO == NORM ? (size_t)K * sizeof(float) : 0;
-    if (M <= 16) gemm_skinny_kernel<1, OutT, PRO><<<grid, block, lds, stream>>>(xb, wb, (OutT*)y, M, N, K, pro);
+    if (M <= 16 && PRO == PLAIN) {
+        switch (best_chunk(K)) {
+            case 4: gemm_skinny_kernel<1, OutT, PLAIN, false, 4><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro); break;
+            case 5: gemm_skinny_kernel<1, OutT, PLAIN, false, 5><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro); break;
+            case 6: gemm_skinny_kernel<1, OutT, PLAIN, false, 6><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro); break;
+            case 7: gemm_skinny_kernel<1, OutT, PLAIN, false, 7><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro); break;
+            default: gemm_skinny_kernel<1, OutT, PLAIN, false, 8><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro); break;
+        }
+    } else if (M <= 16) gemm_skinny_kernel<1, OutT, PRO><<<grid, block, lds, stream>>>(xb, wb, (OutT*)y, M, N, K, pro);
     else if (PRO != PLAIN) return -1;
     else if (M <= 32) gemm_skinny_kernel<2, OutT, PLAIN><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro);
     else gemm_skinny_kernel<4, OutT, PLAIN><<<grid, block, 0, stream>>>(xb, wb, (OutT*)y, M, N, K, pro);
     LSA_LAUNCH_CHECK();
 }
 
-// out_float32: 0 writes bfloat16, 1 writes float32.  Refuses (returns -1) what it cannot take.
-LSA_EXPORT int lsa_gemm_skinny(int out_float32, const void* x, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
+// out_float32: 0 writes bfloat16, 1 writes float32.  tiling: tiles of W per workgroup, 1 or 2 (2 only for
+// M <= 16), or 0 to let the size decide.  Refuses (returns -1) what it cannot take.
+LSA_EXPORT int lsa_gemm_skinny(int out_float32, const void* x, const void* w, void* y, int M, int N, int K, int tiling,
+                               hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 64 || K % 8 != 0 || K < 8) return -1;
+    if (M > 64 || K % 8 != 0 || K < 8 || tiling < 0 || tiling > 2 || (tiling == 2 && M > 16)) return -1;
     Prologue pro = {nullptr, nullptr, nullptr, 0.f};
-    return out_float32 ? launch<float, PLAIN>(x, w, y, M, N, K, pro, stream) : launch<bf16_t, PLAIN>(x, w, y, M, N, K, pro, stream);
+    return out_float32 ? launch<float, PLAIN>(x, w, y, M, N, K, pro, tiling, stream)
+                       : launch<bf16_t, PLAIN>(x, w, y, M, N, K, pro, tiling, stream);
 }
 
 // Y = (silu(gate) * up) . W^T with gate_up [M, 2K]; M <= 16.
@@ -230,7 +390,7 @@ LSA_EXPORT int lsa_gemm_skinny_swiglu(const void* gate_up, const void* w, void* 
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || K % 8 != 0 || K < 8) return -1;
     Prologue pro = {nullptr, nullptr, nullptr, 0.f};
-    return launch<bf16_t, SWIGLU>(gate_up, w, y, M, N, K, pro, stream);
+    return launch<bf16_t, SWIGLU>(gate_up, w, y, M, N, K, pro, 1, stream);
 }
 
 // Y = rmsnorm(resid + delta) * norm_weight . W^T; resid_out = resid + delta (delta may be null: then
@@ -240,14 +400,17 @@ LSA_EXPORT int lsa_gemm_skinny_norm(int out_float32, const void* resid, const vo
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || K % 8 != 0 || K < 8 || K > 16384 || (delta && resid_out == resid)) return -1;
     Prologue pro = {(const bf16_t*)delta, norm_weight, (bf16_t*)resid_out, eps};
-    return out_float32 ? launch<float, NORM>(resid, w, y, M, N, K, pro, stream) : launch<bf16_t, NORM>(resid, w, y, M, N, K, pro, stream);
+    return out_float32 ? launch<float, NORM>(resid, w, y, M, N, K, pro, 1, stream) : launch<bf16_t, NORM>(resid, w, y, M, N, K, pro, 1, stream);
 }
 
 // hidden[M, I] = silu(x . gate^T) * (x . up^T) with gate_up [2I, K] (gate rows first); M <= 16, I a multiple of 8.
-LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* hidden, int M, int I, int K, hipStream_t stream) {
+LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* hidden, int M, int I, int K, int tiling,
+                                     hipStream_t stream) {
     if (M <= 0 || I <= 0) return 0;
-    if (M > 16 || K % 8 != 0 || K < 8 || I % 8 != 0) return -1;
+    if (M > 16 || K % 8 != 0 || K < 8 || I % 8 != 0 || tiling < 0 || tiling > 2) return -1;
     Prologue pro = {nullptr, nullptr, nullptr, 0.f};
+    if (two_tiles_pay(M, I / 8, tiling, 15))
+        return launch_wide<bf16_t, true>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)hidden, M, 2 * I, K, (I + 15) / 16, stream);
     gemm_skinny_kernel<1, bf16_t, PLAIN, true><<<dim3(I / 8), dim3(GEMM_WAVES * 64), 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)hidden, M, 2 * I, K, pro);
     LSA_LAUNCH_CHECK();

@@ -3,7 +3,7 @@
 //
 // rotary_table: cos and sin of position * inv_freq for every token of the step, once per step
 //   (the angles depend on the token and the pair of dimensions only, not on the layer or head).
-// qk_norm_rope_kv_write: one wavefront per (token, head), four heads per workgroup.  q heads are
+// qk_norm_rope_kv_write: d / 16 lanes per (token, head), vector accesses throughout.  q heads are
 //   normalised, rotated and written back in place into the projection buffer; k heads are
 //   normalised, rotated and stored at keys[page][kv_head][slot][:]; v heads are stored transposed
 //   at values[page][kv_head][:][slot].  The page of a token is table[row][position / page_size];
@@ -25,6 +25,48 @@ __global__ void rotary_table_kernel(const int* __restrict__ positions, const flo
     cos_sin[(size_t)token * 2 * half + half + pair] = sinf(angle);
 }
 
+// A (token, head) pair is handled by d / 16 neighbouring lanes: lane j of them owns dimensions
+// [8j, 8j + 8) of the first half and their rotation partners [d/2 + 8j, d/2 + 8j + 8), both as one
+// vector load, so a wavefront covers 64 / (d / 16) pairs at once and every access is 16 bytes or more.
+template <typename T> struct Eight {
+    float v[8];
+};
+template <typename T>
+__device__ inline Eight<T> load8(const T* p) {
+    Eight<T> r;
+    if (sizeof(T) == 2) {
+        const Vec16<T> x = load_vec16(p);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r.v[e] = (float)x.v[e];
+    } else {
+        const Vec16<T> x = load_vec16(p), y = load_vec16(p + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            r.v[e] = (float)x.v[e];
+            r.v[4 + e] = (float)y.v[e];
+        }
+    }
+    return r;
+}
+template <typename T>
+__device__ inline void store8(T* p, const float (&v)[8]) {
+    if (sizeof(T) == 2) {
+        Vec16<T> x;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x.v[e] = (T)v[e];
+        store_vec16(p, x);
+    } else {
+        Vec16<T> x, y;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x.v[e] = (T)v[e];
+            y.v[e] = (T)v[4 + e];
+        }
+        store_vec16(p, x);
+        store_vec16(p + 4, y);
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     T* __restrict__ qkv,                 // [tokens, (Hq + 2 Hkv) * d]
@@ -34,13 +76,25 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     const int* __restrict__ token_row, const int* __restrict__ positions,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
     const float* __restrict__ cos_sin,   // [tokens, d] (cos of the d/2 pairs, then sin) or nullptr
-    int page_size, int n_q, int n_kv, int d, int write_cache, int n_heads) {
-    const int token = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (head >= n_heads) return;
+    int page_size, int n_q, int n_kv, int d, int write_cache, int n_heads, int n_tokens) {
+    const int lanes_per_pair = d >> 4, pairs_per_wave = 64 / lanes_per_pair;
+    const int lane = threadIdx.x & 63, wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int slot_in_wave = lane / lanes_per_pair, j = lane % lanes_per_pair;
+    const long pair = (long)wave * pairs_per_wave + slot_in_wave;
+    const bool active = slot_in_wave < pairs_per_wave && pair < (long)n_tokens * n_heads;
+    const int token = active ? (int)(pair / n_heads) : 0, head = active ? (int)(pair % n_heads) : 0;
     const int half = d >> 1;
     const bool is_q = head < n_q, is_k = !is_q && head < n_q + n_kv;
-    if (!is_q && !write_cache) return;
     T* src = qkv + (size_t)token * (n_q + 2 * n_kv) * d + (size_t)head * d;
+    const Eight<T> lo = load8(src + 8 * j), hi = load8(src + half + 8 * j);
+    // Sum of squares of the head over its lanes (every lane of the wavefront takes part in the shuffles).
+    float sq = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sq += lo.v[e] * lo.v[e] + hi.v[e] * hi.v[e];
+    float total = 0.f;
+    const int first_lane = lane - j;
+    for (int other = 0; other < lanes_per_pair; ++other) total += __shfl(sq, first_lane + other, 64);
+    if (!active || (!is_q && !write_cache)) return;
     size_t page = 0;
     int slot = 0;
     if (!is_q) {
@@ -52,36 +106,42 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     }
     if (!is_q && !is_k) {                // value head: copy, transposed
         T* dst = values + ((page * n_kv + (head - n_q - n_kv)) * d) * page_size + slot;
-        for (int i = lane; i < d; i += 64) dst[(size_t)i * page_size] = src[i];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            dst[(size_t)(8 * j + e) * page_size] = (T)lo.v[e];
+            dst[(size_t)(half + 8 * j + e) * page_size] = (T)hi.v[e];
+        }
         return;
     }
     const float* w = is_q ? q_weight : k_weight;
-    float rstd = 1.f;
+    float x1[8], x2[8];
     if (w) {
-        float sq = 0.f;
-        for (int i = lane; i < d; i += 64) {
-            const float x = (float)src[i];
-            sq += x * x;
+        const float rstd = rsqrtf(total / (float)d + eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            x1[e] = lo.v[e] * rstd * w[8 * j + e];
+            x2[e] = hi.v[e] * rstd * w[half + 8 * j + e];
         }
-        rstd = rsqrtf(wave_sum(sq) / (float)d + eps);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            x1[e] = lo.v[e];
+            x2[e] = hi.v[e];
+        }
+    }
+    if (cos_sin) {
+        const float* cs = cos_sin + (size_t)token * d + 8 * j;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float c = cs[e], s = cs[half + e];
+            const float r1 = x1[e] * c - x2[e] * s, r2 = x2[e] * c + x1[e] * s;
+            x1[e] = r1;
+            x2[e] = r2;
+        }
     }
     T* dst = is_q ? src : keys + ((page * n_kv + (head - n_q)) * page_size + slot) * d;
-    const float* cs = cos_sin ? cos_sin + (size_t)token * d : nullptr;
-    for (int i = lane; i < half; i += 64) {
-        float x1 = (float)src[i], x2 = (float)src[i + half];
-        if (w) {
-            x1 = x1 * rstd * w[i];
-            x2 = x2 * rstd * w[i + half];
-        }
-        float r1 = x1, r2 = x2;
-        if (cs) {
-            const float c = cs[i], s = cs[half + i];
-            r1 = x1 * c - x2 * s;
-            r2 = x2 * c + x1 * s;
-        }
-        dst[i] = (T)r1;
-        dst[i + half] = (T)r2;
-    }
+    store8(dst + 8 * j, x1);
+    store8(dst + half + 8 * j, x2);
 }
 
 constexpr int VT_TOKENS = 64;
@@ -118,10 +178,13 @@ static int launch(void* qkv, void* keys, void* values, const int* table, int tab
     // Long portions: the v heads take the tiled path, the main kernel then covers q and k heads only.
     const bool tiled_values = write_cache && n_tokens >= 4 * VT_TOKENS;
     const int n_heads = tiled_values ? n_q + n_kv : n_q + 2 * n_kv;
-    dim3 grid(n_tokens, (n_heads + 3) / 4);
+    if (d % 16 != 0 || d > 1024) return -1;
+    const long pairs = (long)n_tokens * n_heads;
+    const int pairs_per_block = 4 * (64 / (d / 16));
+    dim3 grid((unsigned)((pairs + pairs_per_block - 1) / pairs_per_block));
     qk_norm_rope_kv_write_kernel<T><<<grid, 256, 0, stream>>>((T*)qkv, (T*)keys, (T*)values, table, table_stride, token_row,
                                                               positions, q_weight, k_weight, eps, cos_sin, page_size,
-                                                              n_q, n_kv, d, write_cache, n_heads);
+                                                              n_q, n_kv, d, write_cache, n_heads, n_tokens);
     int err = (int)hipGetLastError();
     if (err || !tiled_values) return err;
     dim3 vgrid((n_tokens + VT_TOKENS - 1) / VT_TOKENS, n_kv);

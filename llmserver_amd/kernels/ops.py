@@ -84,8 +84,9 @@ class HipOps:
         library.preload(self.required_modules(head_dims, dtype))
 
     # -- library matrix product ------------------------------------------------------------
-    def linear(self, x, weight, out=None, out_float32=False):
-        """``x [T, in] @ weight[out, in]^T``; float32 result if asked (the output head)."""
+    def linear(self, x, weight, out=None, out_float32=False, tiling=0):
+        """``x [T, in] @ weight[out, in]^T``; float32 result if asked (the output head).  ``tiling`` picks the
+        few-row kernel's workgroup shape (1 or 2 tiles of the weight; 0 lets the size decide)."""
         if x.shape[1] != weight.shape[1]:
             raise ValueError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
         rows, width = x.shape
@@ -97,13 +98,13 @@ class HipOps:
                 out = torch.empty((rows, weight.shape[0]), device=x.device, dtype=torch.float32 if out_float32 else torch.bfloat16)
             _check(out, "out", None, (rows, weight.shape[0]))
             _launched(self._gemm.lsa_gemm_skinny(1 if out_float32 else 0, _ptr(x), _ptr(weight), _ptr(out), rows,
-                                                 weight.shape[0], width, _stream()), "gemm_skinny")
+                                                 weight.shape[0], width, int(tiling), _stream()), "gemm_skinny")
             return out
         if out_float32 and x.dtype != torch.float32:
             return torch.mm(x, weight.t(), out_dtype=torch.float32)
         return torch.mm(x, weight.t(), out=out) if out is not None else torch.mm(x, weight.t())
 
-    def linear_gated(self, x, gate_up_weight):
+    def linear_gated(self, x, gate_up_weight, tiling=0):
         """``silu(x @ gate^T) * (x @ up^T)`` with ``gate_up_weight [2I, K]`` in one launch for few rows (the
         activation sits in the product's epilogue), or None if this is not such a case."""
         rows, width = x.shape
@@ -113,7 +114,7 @@ class HipOps:
         _check(x, "x", torch.bfloat16)
         _check(gate_up_weight, "gate_up_weight", torch.bfloat16)
         out = torch.empty((rows, inter), device=x.device, dtype=torch.bfloat16)
-        _launched(self._gemm.lsa_gemm_skinny_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, _stream()),
+        _launched(self._gemm.lsa_gemm_skinny_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, int(tiling), _stream()),
                   "gemm_skinny_gated")
         return out
 
@@ -212,8 +213,8 @@ class HipOps:
         _check(table, "table", torch.int32)
         _check(token_row, "token_row", torch.int32, (n,))
         _check(positions, "positions", torch.int32, (n,))
-        if head_dim % 2:
-            raise ValueError(f"head_dim must be even: {head_dim}")
+        if head_dim % 16:
+            raise ValueError(f"the q/k kernel takes head sizes in steps of 16, got {head_dim}")
         for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
             if w is not None:
                 _check(w, name, torch.float32, (head_dim,))

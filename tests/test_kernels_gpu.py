@@ -278,10 +278,12 @@ def test_sampling(ops, vocab):
 
 
 @pytest.mark.parametrize("rows", [1, 3, 8, 16, 17, 33, 64])
-@pytest.mark.parametrize("n, k", [(16, 8), (100, 72), (301, 4096), (6144, 1000), (4096, 12288)])
+@pytest.mark.parametrize("n, k", [(16, 8), (100, 72), (301, 4096), (6144, 1000), (4096, 12288), (200, 5120), (77, 1536),
+                                  (130, 1792)])
 def test_skinny_gemm(ops, rows, n, k):
     """The weight-streaming product against a float64 product of the same bfloat16 values: widths and
-    output sizes that are no multiple of the tiles, float32 and bfloat16 results."""
+    output sizes that are no multiple of the tiles, widths that give a wavefront 4, 5, 6, 7 or 8 k steps
+    at a time, one or two tiles of the weight per workgroup, float32 and bfloat16 results."""
     print(f"skinny gemm rows {rows} n {n} k {k}", flush=True)
     torch.manual_seed(rows * n + k)
     x = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
@@ -290,15 +292,16 @@ def test_skinny_gemm(ops, rows, n, k):
     saved = ops.skinny_rows
     try:
         ops.skinny_rows = 64
-        got32 = ops.linear(x, w, out_float32=True)
-        got16 = ops.linear(x, w)
+        for tiling in (0, 1, 2) if rows <= 16 else (0, 1):
+            got32 = ops.linear(x, w, out_float32=True, tiling=tiling)
+            got16 = ops.linear(x, w, tiling=tiling)
+            assert got32.dtype == torch.float32 and got16.dtype == torch.bfloat16
+            torch.testing.assert_close(got32, expected, atol=2e-4, rtol=1e-4)          # 32-bit accumulation of exact products
+            torch.testing.assert_close(got16.float(), expected, atol=2e-2, rtol=1e-2)
     finally:
         ops.skinny_rows = saved
-    assert got32.dtype == torch.float32 and got16.dtype == torch.bfloat16
-    torch.testing.assert_close(got32, expected, atol=2e-4, rtol=1e-4)                  # 32-bit accumulation of exact products
-    torch.testing.assert_close(got16.float(), expected, atol=2e-2, rtol=1e-2)
     with pytest.raises(RuntimeError):
-        ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, None)
+        ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, 0, None)
         if ops._gemm_refusal_check != 0:
             raise RuntimeError("refused")
 
@@ -338,7 +341,7 @@ def test_skinny_gemm_with_fused_prologues(ops, rows, n, k):
 
 
 @pytest.mark.parametrize("rows", [1, 5, 8])
-@pytest.mark.parametrize("inter, k", [(8, 16), (104, 72), (12288, 4096), (1000, 1000)])
+@pytest.mark.parametrize("inter, k", [(8, 16), (104, 72), (12288, 4096), (1000, 1000), (264, 5120), (40, 1536), (72, 1792)])
 def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
     print(f"gated product rows {rows} inter {inter} k {k}", flush=True)
     torch.manual_seed(rows + inter + k)
@@ -346,7 +349,8 @@ def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
     w = (torch.randn(2 * inter, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
     gate_up = x.double() @ w.double().t()
     expected = (torch.nn.functional.silu(gate_up[:, :inter]) * gate_up[:, inter:]).float()
-    got = ops.linear_gated(x, w)
-    assert got.shape == (rows, inter) and got.dtype == torch.bfloat16
-    torch.testing.assert_close(got.float(), expected, atol=2e-2, rtol=2e-2)
+    for tiling in (0, 1, 2):
+        got = ops.linear_gated(x, w, tiling=tiling)
+        assert got.shape == (rows, inter) and got.dtype == torch.bfloat16
+        torch.testing.assert_close(got.float(), expected, atol=2e-2, rtol=2e-2)
     assert ops.linear_gated(torch.zeros(9, k, device=DEV, dtype=torch.bfloat16), w) is None
