@@ -67,11 +67,9 @@ class HipOps:
         self._gemm = library.load("gemm")
         self._attention = {}
         self.skinny_rows = SKINNY_GEMM_ROWS
-        # The few-row product can take the residual sum + RMSNorm, or SwiGLU, as a prologue.  Every
-        # workgroup then redoes that work for its 16 output columns, and measured on Qwen3-8B shapes
-        # the fused launches are slower than the separate kernels (gate/up 60 vs 42 us, down 57 vs
-        # 25 us at 1 row), so the parts do not use them unless this is switched on.
-        self.fuse_prologues = False
+        # Whether projections may fold the residual sum and the norm between two few-row products into their
+        # epilogues (see linear_into_stream); off, every such sum and norm is a kernel of its own.
+        self.fuse_stream_updates = True
 
     @staticmethod
     def required_modules(head_dims, dtype):
@@ -83,77 +81,103 @@ class HipOps:
     def preload(self, head_dims, dtype):
         library.preload(self.required_modules(head_dims, dtype))
 
-    # -- library matrix product ------------------------------------------------------------
+    # -- matrix products -------------------------------------------------------------------
+    FUSED_ROWS = 8          # most rows the few-row product's fused epilogues take
+    SCALE_PARTS = 512       # most partial sums per row its row scale takes
+
+    def _few_rows(self, x, weight):
+        rows, width = x.shape
+        return x.dtype == torch.bfloat16 and 0 < rows <= self.skinny_rows and width % 8 == 0 and width >= 8 \
+            and weight.dtype == torch.bfloat16
+
+    def _row_scale_args(self, row_scale, rows):
+        """``row_scale = (square_sums [rows, P] float32, eps)`` or None -> kernel arguments."""
+        if row_scale is None:
+            return None, 0, 0.0
+        square_sums, eps = row_scale
+        _check(square_sums, "square_sums", torch.float32)
+        if square_sums.dim() != 2 or square_sums.shape[0] != rows:
+            raise ValueError(f"square_sums: expected [{rows}, parts], got {tuple(square_sums.shape)}")
+        return _ptr(square_sums), square_sums.shape[1], float(eps)
+
+    def _row_scale_fits(self, row_scale, rows):
+        return row_scale is None or (rows <= self.FUSED_ROWS and 0 < row_scale[0].shape[1] <= self.SCALE_PARTS)
+
+    def row_scale_fits(self, x, weight, row_scale) -> bool:
+        """Whether the few-row products take ``x`` with this ``row_scale`` (then they do not return None for it)."""
+        return x.shape[1] == weight.shape[1] and self._few_rows(x, weight) and self._row_scale_fits(row_scale, x.shape[0])
+
     def linear(self, x, weight, out=None, out_float32=False, tiling=0):
         """``x [T, in] @ weight[out, in]^T``; float32 result if asked (the output head).  ``tiling`` picks the
         few-row kernel's workgroup shape (1 or 2 tiles of the weight; 0 lets the size decide)."""
         if x.shape[1] != weight.shape[1]:
             raise ValueError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
-        rows, width = x.shape
-        if x.dtype == torch.bfloat16 and 0 < rows <= self.skinny_rows and width % 8 == 0:
+        if self._few_rows(x, weight):
             # Few rows: the product is a stream over the weights; the hand-written kernel reads them once at HBM rate.
-            _check(x, "x", torch.bfloat16)
-            _check(weight, "weight", torch.bfloat16)
-            if out is None or out_float32:
-                out = torch.empty((rows, weight.shape[0]), device=x.device, dtype=torch.float32 if out_float32 else torch.bfloat16)
-            _check(out, "out", None, (rows, weight.shape[0]))
-            _launched(self._gemm.lsa_gemm_skinny(1 if out_float32 else 0, _ptr(x), _ptr(weight), _ptr(out), rows,
-                                                 weight.shape[0], width, int(tiling), _stream()), "gemm_skinny")
-            return out
+            return self.linear_few_rows(x, weight, out=out, out_float32=out_float32, tiling=tiling)
         if out_float32 and x.dtype != torch.float32:
             return torch.mm(x, weight.t(), out_dtype=torch.float32)
         return torch.mm(x, weight.t(), out=out) if out is not None else torch.mm(x, weight.t())
 
-    def linear_gated(self, x, gate_up_weight, tiling=0):
+    def linear_few_rows(self, x, weight, out=None, out_float32=False, tiling=0, row_scale=None):
+        """The weight-streaming product, or None if this is no case for it.
+
+        ``row_scale = (square_sums [T, P], eps)``: ``x`` is a residual stream already multiplied by a norm's
+        weights, ``square_sums`` are partial sums of the stream's squares, and the result rows are divided by the
+        stream's root mean square, so that the result is the product of the normalised stream (up to 8 rows)."""
+        rows, width = x.shape
+        if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or not self._row_scale_fits(row_scale, rows):
+            return None
+        _check(x, "x", torch.bfloat16)
+        _check(weight, "weight", torch.bfloat16)
+        if out is None or out_float32:
+            out = torch.empty((rows, weight.shape[0]), device=x.device, dtype=torch.float32 if out_float32 else torch.bfloat16)
+        _check(out, "out", None, (rows, weight.shape[0]))
+        sums, parts, eps = self._row_scale_args(row_scale, rows)
+        _launched(self._gemm.lsa_gemm_skinny(1 if out_float32 else 0, _ptr(x), _ptr(weight), _ptr(out), rows, weight.shape[0], width,
+                                             int(tiling), sums, parts, eps, _stream()), "gemm_skinny")
+        return out
+
+    def linear_into_stream(self, x, weight, resid, norm_weight, tiling=0, row_scale=None):
+        """The few-row product as an update of the residual stream ``resid [T, out]`` that a norm with weights
+        ``norm_weight`` follows, in one launch: returns ``(stream, weighted, square_sums)`` with
+        ``stream = resid + x @ weight^T`` (a new tensor), ``weighted = stream * norm_weight`` and
+        ``square_sums [T, ceil(out / 16)]`` partial sums of ``stream^2``, which is what ``row_scale`` of the next
+        product takes.  None if this is no case for it (more than 8 rows, other types)."""
+        rows, width = x.shape
+        n = weight.shape[0]
+        if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or rows > self.FUSED_ROWS \
+                or not self._row_scale_fits(row_scale, rows) or resid.dtype != torch.bfloat16:
+            return None
+        _check(x, "x", torch.bfloat16)
+        _check(weight, "weight", torch.bfloat16)
+        _check(resid, "resid", torch.bfloat16, (rows, n))
+        _check(norm_weight, "norm_weight", torch.float32, (n,))
+        stream = torch.empty_like(resid)
+        weighted = torch.empty_like(resid)
+        square_sums = torch.empty((rows, (n + 15) // 16), device=x.device, dtype=torch.float32)
+        sums, parts, eps = self._row_scale_args(row_scale, rows)
+        _launched(self._gemm.lsa_gemm_skinny_stream(_ptr(x), _ptr(weight), rows, n, width, int(tiling), sums, parts, eps, _ptr(resid),
+                                                    _ptr(norm_weight), _ptr(stream), _ptr(weighted), _ptr(square_sums), _stream()),
+                  "gemm_skinny_stream")
+        return stream, weighted, square_sums
+
+    def linear_gated(self, x, gate_up_weight, tiling=0, row_scale=None):
         """``silu(x @ gate^T) * (x @ up^T)`` with ``gate_up_weight [2I, K]`` in one launch for few rows (the
-        activation sits in the product's epilogue), or None if this is not such a case."""
+        activation sits in the product's epilogue), or None if this is not such a case.  ``row_scale`` as in
+        :meth:`linear_few_rows`."""
         rows, width = x.shape
         inter = gate_up_weight.shape[0] // 2
-        if x.dtype != torch.bfloat16 or not 0 < rows <= self.skinny_rows or width % 8 or inter % 8 or gate_up_weight.shape[1] != width:
+        if not self._few_rows(x, gate_up_weight) or inter % 8 or gate_up_weight.shape[1] != width or rows > 16 \
+                or not self._row_scale_fits(row_scale, rows):
             return None
         _check(x, "x", torch.bfloat16)
         _check(gate_up_weight, "gate_up_weight", torch.bfloat16)
         out = torch.empty((rows, inter), device=x.device, dtype=torch.bfloat16)
-        _launched(self._gemm.lsa_gemm_skinny_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, int(tiling), _stream()),
-                  "gemm_skinny_gated")
+        sums, parts, eps = self._row_scale_args(row_scale, rows)
+        _launched(self._gemm.lsa_gemm_skinny_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, int(tiling), sums, parts,
+                                                   eps, _stream()), "gemm_skinny_gated")
         return out
-
-    def swiglu_linear(self, gate_up, weight, force=False):
-        """``(silu(gate) * up) @ weight^T`` in one launch for few rows, or None if this is not such a case."""
-        rows, inter = gate_up.shape[0], gate_up.shape[1] // 2
-        if not (self.fuse_prologues or force):
-            return None
-        if gate_up.dtype != torch.bfloat16 or not 0 < rows <= self.skinny_rows or inter % 8 or weight.shape[1] != inter:
-            return None
-        _check(gate_up, "gate_up", torch.bfloat16)
-        _check(weight, "weight", torch.bfloat16)
-        out = torch.empty((rows, weight.shape[0]), device=gate_up.device, dtype=torch.bfloat16)
-        _launched(self._gemm.lsa_gemm_skinny_swiglu(_ptr(gate_up), _ptr(weight), _ptr(out), rows, weight.shape[0], inter, _stream()),
-                  "gemm_skinny_swiglu")
-        return out
-
-    def norm_linear(self, resid, delta, norm_weight, eps, weight, out_float32=False, force=False):
-        """``rmsnorm(resid + delta) * norm_weight @ weight^T`` in one launch for few rows.
-
-        Returns ``(y, resid_after)`` where ``resid_after`` holds ``resid + delta`` (a new tensor; ``resid`` itself
-        when ``delta`` is None), or None if this is not a case for the fused kernel."""
-        rows, width = resid.shape
-        if not (self.fuse_prologues or force):
-            return None
-        if resid.dtype != torch.bfloat16 or not 0 < rows <= self.skinny_rows or width % 8 or width > 16384 or weight.shape[1] != width:
-            return None
-        _check(resid, "resid", torch.bfloat16)
-        _check(weight, "weight", torch.bfloat16)
-        _check(norm_weight, "norm_weight", torch.float32, (width,))
-        resid_after = resid
-        if delta is not None:
-            _check(delta, "delta", torch.bfloat16, (rows, width))
-            resid_after = torch.empty_like(resid)
-        out = torch.empty((rows, weight.shape[0]), device=resid.device, dtype=torch.float32 if out_float32 else torch.bfloat16)
-        _launched(self._gemm.lsa_gemm_skinny_norm(1 if out_float32 else 0, _ptr(resid), _ptr(delta), _ptr(norm_weight), float(eps),
-                                                  _ptr(resid_after), _ptr(weight), _ptr(out), rows, weight.shape[0], width,
-                                                  _stream()), "gemm_skinny_norm")
-        return out, resid_after
 
     # -- hand-written kernels ----------------------------------------------------------------
     def embedding(self, table, token_ids, out):

@@ -13,7 +13,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import Block, Norm, ParamSpec
+from ..parts.base import Block, Norm, ParamSpec, StreamUpdate
 from ..parts.embedding import TokenEmbedding
 from ..parts.linear import Linear
 
@@ -114,8 +114,16 @@ class DecoderModel:
         """Run the step's tokens through every call of the order; float32 logits ``[n_out, vocab]``."""
         resid = self.embedding.forward(ctx.token_ids, ctx)
         delta = None
-        for call in self.order:
-            resid, delta = self.blocks[call.block].forward(resid, delta, ctx, caches.view(call))
+        for index, call in enumerate(self.order):
+            block = self.blocks[call.block]
+            if block.takes_following and index + 1 < len(self.order):
+                # The block may add its last update itself and prepare the next block's first norm.
+                following = self.blocks[self.order[index + 1].block].entry_norm()
+                resid, delta = block.forward(resid, delta, ctx, caches.view(call), following=following)
+            else:
+                resid, delta = block.forward(resid, delta, ctx, caches.view(call))
+        if isinstance(delta, StreamUpdate):
+            resid, delta = delta.resid, None
         if ctx.n_out == 0:
             return torch.empty((0, self.head.out_features), device=resid.device, dtype=torch.float32)
         selected = self.final_norm.add_norm(resid, delta, ctx, rows=ctx.logit_idx)

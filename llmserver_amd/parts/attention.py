@@ -131,6 +131,7 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
 class GQAttention(Mixer):
     graph_safe = True
     accepts_pending_norm = True
+    takes_sink = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  qk_norm_eps: Optional[float] = None, bias: bool = False, out_bias: Optional[bool] = None,
@@ -192,7 +193,7 @@ class GQAttention(Mixer):
             "n_slots": plan.n_slots,
         })
 
-    def forward(self, x, ctx, cache):
+    def forward(self, x, ctx, cache, sink=None):
         qkv = self.qkv.forward(x, ctx)
         table = ctx.block_table(cache.group)
         ctx.ops.qk_norm_rope_kv_write(
@@ -205,4 +206,4 @@ class GQAttention(Mixer):
             qkv, out, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
             ctx.get_plan(self.plan_key()), self.scale, self.window, cache.page_size,
             self.n_heads, self.n_kv_heads, self.head_dim, ctx)
-        return self.o.forward(out, ctx)
+        return self.o.forward(out, ctx, sink=sink)

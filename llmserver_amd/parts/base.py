@@ -70,14 +70,34 @@ class Norm(Part):
         raise NotImplementedError
 
 
+class StreamUpdate:
+    """What a part may return instead of a plain update of the residual stream, when its last
+    projection has already added the update and prepared the norm that follows.
+
+    ``resid [T, H]`` is the stream with the update added, ``weighted [T, H] = resid * norm.weight``,
+    ``square_sums [T, P]`` float32 partial sums of ``resid^2`` over P parts of each row, ``norm`` the
+    norm they were prepared for.  A projection that reads ``weighted`` and divides its result rows
+    by ``sqrt(sum(square_sums) / H + eps)`` has multiplied the normalised stream."""
+
+    def __init__(self, norm: "Norm", resid, weighted, square_sums):
+        self.norm, self.resid, self.weighted, self.square_sums = norm, resid, weighted, square_sums
+
+
 class PendingNorm:
     """A normalisation that has not run yet: ``norm(resid + delta)``.
 
-    A part that starts with a projection can hand this to its :class:`~llmserver_amd.parts.linear.Linear`,
-    which may compute the sum, the norm and the product in one kernel.  ``tensor()`` carries the
-    normalisation out the plain way.  Afterwards ``resid`` is the residual stream with ``delta`` added."""
+    A part that starts with a projection can hand this to its :class:`~llmserver_amd.parts.linear.Linear`.
+    If ``delta`` came as a :class:`StreamUpdate` prepared for this very norm, the sum is done already
+    and ``prepared`` holds what lets the projection apply the norm in its epilogue.  ``tensor()``
+    carries the normalisation out the plain way.  Afterwards ``resid`` is the residual stream with
+    ``delta`` added."""
 
     def __init__(self, norm: "Norm", resid, delta, ctx):
+        self.prepared = None
+        if isinstance(delta, StreamUpdate):
+            if delta.norm is norm:
+                self.prepared = delta
+            resid, delta = delta.resid, None
         self.norm, self.resid, self.delta, self.ctx = norm, resid, delta, ctx
         self._done = None
 
@@ -87,9 +107,25 @@ class PendingNorm:
             self.delta = None
         return self._done
 
-    def consumed(self, resid_after):
-        """A fused kernel has used the pending sum; ``resid_after`` holds ``resid + delta``."""
-        self.resid, self.delta = resid_after, None
+    def row_scale(self):
+        """``(weighted stream, (square_sums, eps))`` if a projection may apply the norm as a row scale, else None."""
+        if self.prepared is None or self._done is not None or not hasattr(self.norm, "eps"):
+            return None
+        return self.prepared.weighted, (self.prepared.square_sums, self.norm.eps)
+
+
+class ResidualSink:
+    """Told to a part with ``takes_sink``: its output will be added to the residual stream and
+    ``norm`` will follow.  The part's last projection may then do both (returning a
+    :class:`StreamUpdate`); ``stream()`` is the residual stream it has to add to."""
+
+    def __init__(self, pending: PendingNorm, norm: "Norm"):
+        self.pending, self.norm = pending, norm
+
+    def stream(self):
+        if self.pending.delta is not None:          # nobody has added the previous update yet
+            self.pending.tensor()
+        return self.pending.resid
 
 
 class PositionEncoding(Part):
@@ -113,6 +149,8 @@ class Mixer(Part):
     graph_safe = False
     # True if ``forward`` passes its input straight to a Linear and so can take a PendingNorm.
     accepts_pending_norm = False
+    # True if ``forward`` takes ``sink=`` (a ResidualSink or None) and may return a StreamUpdate.
+    takes_sink = False
 
     def cache_spec(self):
         """:class:`PagedKVSpec`, :class:`StateSpec` or None."""
@@ -128,16 +166,25 @@ class Mixer(Part):
 
 class FeedForward(Part):
     accepts_pending_norm = False
+    takes_sink = False
 
     def forward(self, x, ctx):
         raise NotImplementedError
 
 
 class Block(Part):
-    """An arrangement of parts.  ``forward(resid, delta, ctx, cache) -> delta'``: ``resid`` is
-    the residual stream (updated in place), ``delta`` the pending update not yet added to it."""
+    """An arrangement of parts.  ``forward(resid, delta, ctx, cache) -> (resid', delta')``:
+    ``resid`` is the residual stream, ``delta`` the pending update not yet added to it (a tensor,
+    None, or a :class:`StreamUpdate`, which carries the stream it was added to)."""
 
     mixer: Mixer
+    # True if ``forward`` takes ``following=``: the norm that will be applied to the block's
+    # output (the next block's ``entry_norm()``), or None.  Such a block may return a StreamUpdate.
+    takes_following = False
+
+    def entry_norm(self):
+        """The norm this block applies first to what it is given, or None."""
+        return None
 
     def forward(self, resid, delta, ctx, cache):
         raise NotImplementedError

@@ -12,7 +12,7 @@ from typing import Dict, List, Sequence
 
 import torch
 
-from .base import MATRIX, VECTOR, ParamSpec, Part, PendingNorm
+from .base import MATRIX, VECTOR, ParamSpec, Part, PendingNorm, StreamUpdate
 
 
 class Linear(Part):
@@ -61,21 +61,27 @@ class Linear(Part):
         self._w.clear()
         self._b.clear()
 
-    def forward(self, x, ctx, out=None):
+    def forward(self, x, ctx, out=None, sink=None):
+        """``x`` is a tensor or a :class:`PendingNorm`.  With ``sink`` (a :class:`ResidualSink`) the result may
+        come back as a :class:`StreamUpdate`: already added to the residual stream, the following norm prepared."""
+        ops = ctx.ops
+        fused = getattr(ops, "fuse_stream_updates", False)
+        row_scale = None
         if isinstance(x, PendingNorm):
-            fused = getattr(ctx.ops, "norm_linear", None)
-            weight = getattr(x.norm, "weight", None)
-            done = None
-            if fused is not None and x._done is None and weight is not None and hasattr(x.norm, "eps"):
-                done = fused(x.resid, x.delta, weight, x.norm.eps, self.weight, self.out_float32)
+            scaled = x.row_scale() if fused else None
+            if scaled is not None and ops.row_scale_fits(scaled[0], self.weight, scaled[1]):
+                x, row_scale = scaled            # the norm becomes a scale of the product's rows
+            else:
+                x = x.tensor()
+        if sink is not None and fused and self.bias is None and not self.out_float32 \
+                and getattr(sink.norm, "weight", None) is not None and hasattr(sink.norm, "eps"):
+            done = ops.linear_into_stream(x, self.weight, sink.stream(), sink.norm.weight, row_scale=row_scale)
             if done is not None:
-                y, resid_after = done
-                x.consumed(resid_after)
-                if self.bias is not None:
-                    ctx.ops.add_bias_(y, self.bias)
-                return y
-            x = x.tensor()
-        y = ctx.ops.linear(x, self.weight, out=out, out_float32=self.out_float32)
+                return StreamUpdate(sink.norm, *done)
+        if row_scale is not None:
+            y = ops.linear_few_rows(x, self.weight, out=out, out_float32=self.out_float32, row_scale=row_scale)
+        else:
+            y = ops.linear(x, self.weight, out=out, out_float32=self.out_float32)
         if self.bias is not None:
-            ctx.ops.add_bias_(y, self.bias)
+            ops.add_bias_(y, self.bias)
         return y

@@ -12,6 +12,7 @@ from .linear import Linear
 
 class GatedMLP(FeedForward):
     accepts_pending_norm = True
+    takes_sink = True
 
     def __init__(self, width: int, intermediate: int, activation: str = "silu", bias: bool = False):
         if activation not in ("silu", "swish"):
@@ -31,20 +32,26 @@ class GatedMLP(FeedForward):
         self.gate_up.finalize()
         self.down.finalize()
 
-    def forward(self, x, ctx):
-        gated = getattr(ctx.ops, "linear_gated", None)
-        if gated is not None and self.gate_up.bias is None and not getattr(ctx.ops, "fuse_prologues", False):
-            tensor = x.tensor() if isinstance(x, PendingNorm) else x
-            hidden = gated(tensor, self.gate_up.weight)       # few rows: the activation in the product's epilogue
+    def forward(self, x, ctx, sink=None):
+        ops = ctx.ops
+        gated = getattr(ops, "linear_gated", None)
+        if gated is not None and self.gate_up.bias is None:
+            # Few rows: one launch for both products with the activation in its epilogue.
+            row_scale = None
+            tensor = x
+            if isinstance(x, PendingNorm):
+                scaled = x.row_scale() if getattr(ops, "fuse_stream_updates", False) else None
+                if scaled is not None and ops.row_scale_fits(scaled[0], self.gate_up.weight, scaled[1]):
+                    tensor, row_scale = scaled
+                else:
+                    tensor = x.tensor()
+            hidden = gated(tensor, self.gate_up.weight, row_scale=row_scale)
             if hidden is not None:
-                return self.down.forward(hidden, ctx)
+                return self.down.forward(hidden, ctx, sink=sink)
+            if row_scale is not None:
+                tensor = x.tensor()
             x = tensor
         gate_up = self.gate_up.forward(x, ctx)
-        fused = getattr(ctx.ops, "swiglu_linear", None)
-        if fused is not None and self.down.bias is None:
-            y = fused(gate_up, self.down.weight)          # few rows: activation inside the down projection's kernel
-            if y is not None:
-                return y
         hidden = ctx.empty((gate_up.shape[0], self.intermediate))
-        ctx.ops.swiglu(gate_up, hidden)
-        return self.down.forward(hidden, ctx)
+        ops.swiglu(gate_up, hidden)
+        return self.down.forward(hidden, ctx, sink=sink)

@@ -301,43 +301,74 @@ def test_skinny_gemm(ops, rows, n, k):
     finally:
         ops.skinny_rows = saved
     with pytest.raises(RuntimeError):
-        ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, 0, None)
+        ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, 0, None, 0, 0.0, None)
         if ops._gemm_refusal_check != 0:
             raise RuntimeError("refused")
 
 
 @pytest.mark.parametrize("rows", [1, 5, 8])
-@pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (6144, 1000)])
-def test_skinny_gemm_with_fused_prologues(ops, rows, n, k):
-    """The few-row product with the activation or the residual sum and norm inside it, against the
-    separate kernels' twins."""
-    print(f"fused prologues rows {rows} n {n} k {k}", flush=True)
+@pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (6144, 1000), (200, 5120), (8192, 64)])
+def test_skinny_gemm_with_row_scale_and_stream_update(ops, rows, n, k):
+    """The few-row product with a norm folded in on either side, against the separate kernels' twins:
+    as a consumer it reads the stream times the norm's weights and divides its rows by the stream's rms,
+    which it gets as partial sums of squares; as a producer it adds its result to a residual stream and
+    writes what the next product needs of the norm that follows."""
+    print(f"row scale and stream update rows {rows} n {n} k {k}", flush=True)
     torch.manual_seed(rows + n + k)
     w = (torch.randn(n, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
-    gate_up = (2 * torch.randn(rows, 2 * k, device=DEV)).to(torch.bfloat16)
-    hidden = torch.empty(rows, k, device=DEV, dtype=torch.bfloat16)
-    TorchOps().swiglu(gate_up, hidden)
-    expected = (hidden.double() @ w.double().t()).float()
-    got = ops.swiglu_linear(gate_up, w, force=True)
-    torch.testing.assert_close(got.float(), expected, atol=3e-2, rtol=2e-2)
-
-    resid = (3 * torch.randn(rows, k, device=DEV)).to(torch.bfloat16)
-    delta = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
+    stream = (3 * torch.randn(rows, k, device=DEV)).to(torch.bfloat16)
     norm_weight = 1 + 0.2 * torch.randn(k, device=DEV)
-    for d in (delta, None):
-        ref_resid, normed = resid.clone(), torch.empty_like(resid)
-        TorchOps().add_rmsnorm(ref_resid, d, norm_weight, 1e-5, normed)
-        expected = (normed.double() @ w.double().t()).float()
+    eps = 1e-5
+    # consumer: partial sums over an arbitrary split of the rows (here 7 uneven parts)
+    bounds = [0, 1, k // 5, k // 3, k // 2, k - 3, k - 1, k]
+    squares = stream.float() ** 2
+    square_sums = torch.stack([squares[:, a:b].sum(1) for a, b in zip(bounds, bounds[1:])], dim=1).contiguous()
+    weighted = (stream.float() * norm_weight).to(torch.bfloat16)
+    rstd = torch.rsqrt(squares.double().sum(1, keepdim=True) / k + eps)
+    expected = (weighted.double() @ w.double().t()) * rstd
+    for tiling in (0, 1, 2):
         for out32 in (False, True):
-            kept = resid.clone()
-            got, after = ops.norm_linear(kept, d, norm_weight, 1e-5, w, out_float32=out32, force=True)
-            assert torch.equal(kept, resid)                                  # the input stream is not written
-            assert torch.equal(after, ref_resid)                             # the sum is rounded once, identically
-            assert (after.data_ptr() == kept.data_ptr()) == (d is None)
+            got = ops.linear_few_rows(weighted, w, out_float32=out32, tiling=tiling, row_scale=(square_sums, eps))
             assert got.dtype == (torch.float32 if out32 else torch.bfloat16)
-            torch.testing.assert_close(got.float(), expected, atol=3e-2, rtol=2e-2)
-    assert ops.swiglu_linear(torch.zeros(9, 2 * k, device=DEV, dtype=torch.bfloat16), w, force=True) is None          # too many rows: not fused
-    assert ops.norm_linear(torch.zeros(9, k, device=DEV, dtype=torch.bfloat16), None, norm_weight, 1e-5, w, force=True) is None
+            torch.testing.assert_close(got.double(), expected, atol=2e-4 if out32 else 3e-2, rtol=1e-4 if out32 else 2e-2)
+    # ... and it is the product of the normalised stream, up to the rounding of the normalised values
+    normed = torch.empty_like(stream)
+    TorchOps().add_rmsnorm(stream.clone(), None, norm_weight, eps, normed)
+    torch.testing.assert_close(expected, normed.double() @ w.double().t(), atol=3e-2, rtol=3e-2)
+    # producer: y added to a residual stream of width n, the next norm's weights applied, squares summed per 16 columns
+    x = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
+    resid = (2 * torch.randn(rows, n, device=DEV)).to(torch.bfloat16)
+    next_weight = 1 + 0.2 * torch.randn(n, device=DEV)
+    y = (x.double() @ w.double().t()).float().to(torch.bfloat16)
+    want_stream = (resid.float() + y.float()).to(torch.bfloat16)
+    want_weighted = (want_stream.float() * next_weight).to(torch.bfloat16)
+    for tiling in (0, 1, 2):
+        kept = resid.clone()
+        got_stream, got_weighted, got_sums = ops.linear_into_stream(x, w, kept, next_weight, tiling=tiling)
+        assert torch.equal(kept, resid)
+        # y is rounded once to bfloat16 before the sum, as the separate kernels do; a product that lands on a
+        # rounding boundary may differ by one step of bfloat16
+        torch.testing.assert_close(got_stream.float(), want_stream.float(), atol=4e-2, rtol=1e-2)
+        assert float((got_stream.float() - want_stream.float()).abs().gt(0).float().mean()) < 0.02
+        torch.testing.assert_close(got_weighted.float(), (got_stream.float() * next_weight).to(torch.bfloat16).float(), atol=0, rtol=0)
+        assert got_sums.shape == (rows, (n + 15) // 16)
+        torch.testing.assert_close(got_sums.sum(1), (got_stream.float() ** 2).sum(1), atol=1e-3, rtol=1e-5)
+    # chained: the producer's outputs feed a consumer of width n
+    w2 = (torch.randn(72, n, device=DEV) / n ** 0.5).to(torch.bfloat16)
+    got_stream, got_weighted, got_sums = ops.linear_into_stream(weighted, w, resid, next_weight, row_scale=(square_sums, eps))
+    if n % 8:
+        assert ops.linear_few_rows(got_weighted, w2, row_scale=(got_sums, eps)) is None          # widths in steps of 8 only
+    elif got_sums.shape[1] <= ops.SCALE_PARTS:
+        chained = ops.linear_few_rows(got_weighted, w2, out_float32=True, row_scale=(got_sums, eps))
+        normed = torch.empty_like(got_stream)
+        TorchOps().add_rmsnorm(got_stream.clone(), None, next_weight, eps, normed)
+        torch.testing.assert_close(chained.double(), normed.double() @ w2.double().t(), atol=3e-2, rtol=3e-2)
+    else:
+        assert ops.linear_few_rows(got_weighted, w2, row_scale=(got_sums, eps)) is None
+    # more rows than the fused epilogues take
+    nine = torch.zeros(9, k, device=DEV, dtype=torch.bfloat16)
+    assert ops.linear_into_stream(nine, w, torch.zeros(9, n, device=DEV, dtype=torch.bfloat16), next_weight) is None
+    assert ops.linear_few_rows(nine, w, row_scale=(torch.ones(9, 4, device=DEV), eps)) is None
 
 
 @pytest.mark.parametrize("rows", [1, 5, 8])
@@ -349,8 +380,13 @@ def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
     w = (torch.randn(2 * inter, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
     gate_up = x.double() @ w.double().t()
     expected = (torch.nn.functional.silu(gate_up[:, :inter]) * gate_up[:, inter:]).float()
+    square_sums = torch.rand(rows, 5, device=DEV) * k
+    rstd = torch.rsqrt(square_sums.double().sum(1, keepdim=True) / k + 1e-6)
+    scaled = (torch.nn.functional.silu(gate_up[:, :inter] * rstd) * gate_up[:, inter:] * rstd).float()
     for tiling in (0, 1, 2):
         got = ops.linear_gated(x, w, tiling=tiling)
         assert got.shape == (rows, inter) and got.dtype == torch.bfloat16
         torch.testing.assert_close(got.float(), expected, atol=2e-2, rtol=2e-2)
+        got = ops.linear_gated(x, w, tiling=tiling, row_scale=(square_sums, 1e-6))
+        torch.testing.assert_close(got.float(), scaled, atol=2e-2, rtol=2e-2)
     assert ops.linear_gated(torch.zeros(9, k, device=DEV, dtype=torch.bfloat16), w) is None

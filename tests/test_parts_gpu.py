@@ -118,13 +118,14 @@ def test_attention_part_and_block(dtype, bias):
         assert float((got - expected).abs().max()) < TOL[dtype] * (4 if what == "attention" else 10), what
 
 
-def test_block_with_fused_prologues_switched_on():
-    """The same block with the sum + norm and the activation inside the few-row products."""
+def test_block_without_fused_stream_updates():
+    """The same block with every residual sum and norm as a kernel of its own (the few-row projections
+    otherwise fold them into their epilogues)."""
     from llmserver_amd.kernels import default_ops
     ops = default_ops()
-    ops.fuse_prologues = True
+    ops.fuse_stream_updates = False
     try:
         test_attention_part_and_block(torch.bfloat16, True)
         test_attention_part_and_block(torch.bfloat16, False)
     finally:
-        ops.fuse_prologues = False
+        ops.fuse_stream_updates = True
