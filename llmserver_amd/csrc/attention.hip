@@ -48,6 +48,20 @@ struct Geometry {
     float scale;
 };
 
+// Decode steps (every row brings one token) can leave the per-head norm and the rotation of q and
+// of the new key, and the new key's and value's way into the cache, to this kernel: a wavefront
+// then reads its queries raw from the projection, and the one whose key range ends at the new
+// token takes that token's key and value from the projection too (normalised, rotated, written to
+// the cache on the side) instead of from the pages.  One launch less between the projection and
+// the attention.  bfloat16 and head sizes in steps of 64 only.
+struct DecodeFusion {
+    const float* q_weight;     // [D] or null: no norm
+    const float* k_weight;
+    const float* cos_sin;      // [tokens, D] (cos of the D/2 pairs, then sin) or null: no rotation
+    float eps;
+    int mode;                  // 0: off; 1: q from the raw projection; 3: and the new key and value
+};
+
 #if LSA_BF16
 typedef bf16_t elem_t;
 constexpr int KEY_STEP = 32;                 // keys per loop step (one 16x16x32 MFMA in the output product)
@@ -60,11 +74,11 @@ constexpr int NS = D / 16;                   // 16-dim steps (four 16x16x4 MFMAs
 
 __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
-    const elem_t* __restrict__ keys, const elem_t* __restrict__ values,
+    const elem_t* keys, const elem_t* values,
     const int* __restrict__ table, int table_stride,
     const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
     const Item* __restrict__ items, const int* __restrict__ item_slot, int n_items,
-    float* __restrict__ part_acc, float* __restrict__ part_ml, Geometry g) {
+    float* __restrict__ part_acc, float* __restrict__ part_ml, Geometry g, DecodeFusion fusion) {
     const int lane = threadIdx.x & 63;
     const int item_index = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (item_index >= n_items) return;
@@ -95,6 +109,59 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
             x = *reinterpret_cast<const bf16x8*>(q + (size_t)(token0 + pair_token) * q_token_stride + (size_t)head * D + dim);
         qf[s] = x;
     }
+    // A head in the operand layout (this lane: dims 32 s + 8 quad .. + 8 of every s), normalised over
+    // the head and rotated as the separate kernel does it; the four quads of a column share a head.
+    auto norm_rotate = [&](bf16x8 (&h)[NS], const float* weight, const float* cs) {
+        if (NS % 2) return;                               // head sizes in steps of 64 only (the host checks)
+        float x[NS][8];
+        float sq = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[s][e] = (float)h[s][e];
+                sq += x[s][e] * x[s][e];
+            }
+        if (weight) {
+            sq += __shfl_xor(sq, 16, 64);
+            sq += __shfl_xor(sq, 32, 64);
+            const float rstd = rsqrtf(sq / (float)D + fusion.eps);
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const f32x4 w0 = *reinterpret_cast<const f32x4*>(weight + 32 * s + 8 * quad);
+                const f32x4 w1 = *reinterpret_cast<const f32x4*>(weight + 32 * s + 8 * quad + 4);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[s][e] = x[s][e] * rstd * (e < 4 ? w0[e] : w1[e - 4]);
+            }
+        }
+        if (cs) {
+#pragma unroll
+            for (int s = 0; s < NS / 2; ++s) {
+                const float* c = cs + 32 * s + 8 * quad;
+                const f32x4 c0 = *reinterpret_cast<const f32x4*>(c), c1 = *reinterpret_cast<const f32x4*>(c + 4);
+                const f32x4 s0 = *reinterpret_cast<const f32x4*>(c + D / 2), s1 = *reinterpret_cast<const f32x4*>(c + D / 2 + 4);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float co = e < 4 ? c0[e] : c1[e - 4], si = e < 4 ? s0[e] : s1[e - 4];
+                    const float x1 = x[s][e], x2 = x[s + NS / 2][e];
+                    x[s][e] = x1 * co - x2 * si;
+                    x[s + NS / 2][e] = x2 * co + x1 * si;
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[s][e] = (bf16_t)x[s][e];
+    };
+    const float* token_cos_sin = fusion.cos_sin ? fusion.cos_sin + (size_t)token0 * D : nullptr;
+    if (fusion.mode & 1) {
+        norm_rotate(qf, fusion.q_weight, token_cos_sin);
+        if (!pair_valid) {
+#pragma unroll
+            for (int s = 0; s < NS; ++s) qf[s] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
 #else
     f32x4 qf[NS];
 #pragma unroll
@@ -111,7 +178,54 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     for (int c = 0; c < ND; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float run_max = NEG_INF, run_sum = 0.f;    // run_sum: this lane's share (its keys) of the pair's sum
 
-    const int k_begin = item.k_begin, k_end = item.k_end;
+    int item_k_end = item.k_end;
+#if LSA_BF16
+    if ((fusion.mode & 2) && item.k_begin < item.k_end && item.k_end == row_ctx[row]) {
+        // This item ends at the row's new token.  Its key and value come from the projection, not from the
+        // pages: the online softmax starts from this one key (maximum = its score, sum = 1, output = its
+        // value) and the walk over the pages stops before it.  Column 0 puts both into the cache.
+        const int new_pos = item.k_end - 1;
+        const elem_t* token_qkv = q + (size_t)token0 * q_token_stride;
+        bf16x8 kh[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) kh[s] = *reinterpret_cast<const bf16x8*>(token_qkv + (size_t)(g.n_q + kv_head) * D + 32 * s + 8 * quad);
+        norm_rotate(kh, fusion.k_weight, token_cos_sin);
+        float dot = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dot += (float)kh[s][e] * (float)qf[s][e];
+        dot += __shfl_xor(dot, 16, 64);
+        dot += __shfl_xor(dot, 32, 64);
+        const elem_t* vh = token_qkv + (size_t)(g.n_q + g.n_kv + kv_head) * D + 4 * quad;
+        bf16x4 vnew[ND];
+#pragma unroll
+        for (int c = 0; c < ND; ++c) vnew[c] = *reinterpret_cast<const bf16x4*>(vh + 16 * c);
+        if (pair_valid) {
+            run_max = dot * g.scale;
+            run_sum = quad == 0 ? 1.f : 0.f;
+#pragma unroll
+            for (int c = 0; c < ND; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[c][r] = (float)vnew[c][r];
+        }
+        if (col == 0) {
+            const int block = (int)__umulhi((unsigned)new_pos, g.page_magic);
+            const int slot = new_pos - block * ps;
+            const size_t page = (size_t)row_table[block] * page_elems;
+            elem_t* kp = const_cast<elem_t*>(keys) + page + kv_head_keys + (size_t)slot * D + 8 * quad;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) *reinterpret_cast<bf16x8*>(kp + 32 * s) = kh[s];
+            elem_t* vp = const_cast<elem_t*>(values) + page + kv_head_values + (size_t)(4 * quad) * ps + slot;
+#pragma unroll
+            for (int c = 0; c < ND; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vp[(size_t)(16 * c + r) * ps] = vnew[c][r];
+        }
+        item_k_end = new_pos;
+    }
+#endif
+    const int k_begin = item.k_begin, k_end = item_k_end;
 
     // One step of KEY_STEP keys: the K rows and V^T pieces this lane feeds to the MFMAs.  Steps are
     // loaded one ahead of the step being computed, so the loads of the next step are in flight
@@ -670,8 +784,13 @@ LSA_EXPORT int lsa_paged_attention(
     const void* q, long q_token_stride, void* out, const void* keys, const void* values, const int* table, int table_stride,
     const int* row_start, const int* row_len, const int* row_ctx, const void* items, const int* item_slot, int n_items,
     const void* merges, int n_merges, float* part_acc, float* part_ml, const void* tiles, int n_tiles, float scale, int window,
-    int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles, hipStream_t stream) {
+    int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
+    int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, hipStream_t stream) {
     if (n_items <= 0 && n_tiles <= 0) return 0;
+    // decode_fusion (see DecodeFusion::mode): the caller promises that every row of the step brings one token.
+    DecodeFusion fusion = {q_weight, k_weight, cos_sin, norm_eps, decode_fusion};
+    if (decode_fusion != 0 && decode_fusion != 1 && decode_fusion != 3) return -1;
+    if (decode_fusion && (!LSA_BF16 || D % 64 != 0 || n_tiles > 0 || (q_weight == nullptr) != (k_weight == nullptr))) return -1;
     Geometry g;
     g.n_q = n_q; g.n_kv = n_kv; g.group = n_q / n_kv; g.gheads = gheads; g.tokens_per_tile = tokens_per_tile;
     g.gtiles = gtiles; g.page_size = page_size; g.window = window; g.scale = scale;
@@ -692,7 +811,7 @@ LSA_EXPORT int lsa_paged_attention(
     dim3 grid((n_items + 3) / 4, n_kv * gtiles);
     paged_attention_kernel<<<grid, 256, 0, stream>>>(
         (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
-        row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g);
+        row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g, fusion);
     int err = (int)hipGetLastError();
     if (err || n_merges <= 0) return err;
     dim3 mgrid(n_merges, n_kv * gtiles, 16);

@@ -257,12 +257,23 @@ class HipOps:
             self._attention[key] = library.load(build.attention_module(dtype == torch.bfloat16, head_dim))
         return self._attention[key]
 
+    @staticmethod
+    def decode_fusion_fits(dtype, head_dim) -> bool:
+        """Whether the attention kernel can take the q/k norm, the rotation and the new token's way into the cache
+        on itself in a step in which every row brings one token."""
+        return dtype == torch.bfloat16 and head_dim % 64 == 0
+
     def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
-                        n_q, n_kv, head_dim, ctx):
+                        n_q, n_kv, head_dim, ctx, decode_fusion=None):
         """Attention of the step's tokens over their requests' pages.
 
         ``qkv [T, (n_q + 2 n_kv) * d]`` holds the normalised, rotated queries in its first
         ``n_q * d`` columns; ``out [T, n_q * d]``; ``plan`` is the staged work list.
+
+        ``decode_fusion = (q_weight, k_weight, eps, cos_sin, write_cache)`` instead of a call of
+        :meth:`qk_norm_rope_kv_write` before this one: ``qkv`` is then the raw projection, every row of the step
+        must bring exactly one token, and the kernel normalises and rotates q and the new key itself and (with
+        ``write_cache``) takes the new key and value from ``qkv`` and puts them into the pages.
         """
         n = qkv.shape[0]
         _check(qkv, "qkv", None, (n, (n_q + 2 * n_kv) * head_dim))
@@ -295,12 +306,26 @@ class HipOps:
         if n_slots:
             part_acc = ctx.empty((n_slots, n_kv * gtiles, 16, head_dim), dtype=torch.float32)
             part_ml = ctx.empty((n_slots, n_kv * gtiles, 16, 2), dtype=torch.float32)
+        fusion_mode, q_weight, k_weight, norm_eps, cos_sin = 0, None, None, 0.0, None
+        if decode_fusion is not None:
+            q_weight, k_weight, norm_eps, cos_sin, write_cache = decode_fusion
+            if not self.decode_fusion_fits(qkv.dtype, head_dim) or n_tiles or n != rows:
+                raise ValueError("decode fusion takes bfloat16, head sizes in steps of 64 and steps of one token per row")
+            for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+                if w is not None:
+                    _check(w, name, torch.float32, (head_dim,))
+            if (q_weight is None) != (k_weight is None):
+                raise ValueError("q and k norm weights must come together")
+            if cos_sin is not None:
+                _check(cos_sin, "cos_sin", torch.float32, (n, head_dim))
+            fusion_mode = 3 if write_cache else 1
         lib = self._attention_library(qkv.dtype, head_dim)
         _launched(lib.lsa_paged_attention(
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(row_start),
             _ptr(row_len), _ptr(row_ctx), _ptr(plan["items"]), _ptr(plan["item_slot"]), n_items, _ptr(plan["merges"]),
             n_merges, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), n_tiles, float(scale), int(window) if window else 0,
-            page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, _stream()), "paged_attention")
+            page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, fusion_mode, _ptr(q_weight), _ptr(k_weight), float(norm_eps),
+            _ptr(cos_sin), _stream()), "paged_attention")
 
     def sample(self, logits, temperature, uniform, out):
         n, vocab = logits.shape

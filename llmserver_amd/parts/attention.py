@@ -196,14 +196,21 @@ class GQAttention(Mixer):
     def forward(self, x, ctx, cache, sink=None):
         qkv = self.qkv.forward(x, ctx)
         table = ctx.block_table(cache.group)
-        ctx.ops.qk_norm_rope_kv_write(
-            qkv, cache.keys, cache.values, table, ctx.token_row, ctx.positions,
-            self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
-            self.position.cos_sin(ctx), cache.page_size, self.n_heads, self.n_kv_heads, self.head_dim,
-            cache.writable)
+        eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
+        cos_sin = self.position.cos_sin(ctx)
+        # A step of single tokens: the attention kernel does the norm, the rotation and the cache write itself.
+        fits = getattr(ctx.ops, "decode_fusion_fits", None)
+        fusion = None
+        if fits is not None and ctx.n_tokens == ctx.n_rows and fits(qkv.dtype, self.head_dim):
+            fusion = (self.q_norm_weight, self.k_norm_weight, eps, cos_sin, cache.writable)
+        else:
+            ctx.ops.qk_norm_rope_kv_write(
+                qkv, cache.keys, cache.values, table, ctx.token_row, ctx.positions, self.q_norm_weight, self.k_norm_weight, eps,
+                cos_sin, cache.page_size, self.n_heads, self.n_kv_heads, self.head_dim, cache.writable)
         out = ctx.empty((qkv.shape[0], self.n_heads * self.head_dim))
+        extra = {"decode_fusion": fusion} if fusion is not None else {}
         ctx.ops.paged_attention(
             qkv, out, cache.keys, cache.values, table, ctx.row_start, ctx.row_len, ctx.row_ctx,
             ctx.get_plan(self.plan_key()), self.scale, self.window, cache.page_size,
-            self.n_heads, self.n_kv_heads, self.head_dim, ctx)
+            self.n_heads, self.n_kv_heads, self.head_dim, ctx, **extra)
         return self.o.forward(out, ctx, sink=sink)

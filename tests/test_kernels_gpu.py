@@ -196,6 +196,87 @@ def test_attention_mixed_batch(ops, dtype, n_q, n_kv, d, page):
     assert plan.n_slots > 0                                     # long contexts of single tokens were split
 
 
+@pytest.mark.parametrize("n_q, n_kv, d, page", [(32, 8, 128, 16), (4, 2, 64, 8), (20, 1, 64, 16), (6, 3, 192, 12), (2, 1, 256, 64)])
+@pytest.mark.parametrize("window", [None, 40])
+def test_attention_decode_fusion(ops, n_q, n_kv, d, page, window):
+    """A step of single tokens with the q/k norm, the rotation and the cache write left to the attention kernel,
+    against the two separate kernels and against the plain twin: outputs and what lands in the cache; with and
+    without norm and rotation; reading a cache that another layer has written; with key ranges split evenly as
+    captured steps do (trailing ranges are then empty and must not count the new token twice)."""
+    print(f"attention decode fusion {n_q}/{n_kv} d{d} page{page} window {window}", flush=True)
+    dtype = torch.bfloat16
+    torch.manual_seed(n_q + d)
+    ctxs = [1, 2, 33, 300, 1025, 64, 65]
+    rows = len(ctxs)
+    lens = [1] * rows
+    n_pages = sum(-(-c // page) for c in ctxs) + 3
+    keys0 = (5 * torch.randn(n_pages, n_kv, page, d, device=DEV)).to(dtype)
+    values0 = (5 * torch.randn(n_pages, n_kv, d, page, device=DEV)).to(dtype)
+    perm = torch.randperm(n_pages)
+    width = max(-(-c // page) for c in ctxs)
+    table = torch.full((rows, width), -1, dtype=torch.int32)
+    used = 0
+    for r, c in enumerate(ctxs):
+        blocks = -(-c // page)
+        table[r, :blocks] = perm[used:used + blocks].int()
+        used += blocks
+        place = torch.arange(c - 1)
+        pages = table[r].long()[place // page].to(DEV)
+        keys0[pages, :, (place % page).to(DEV), :] = torch.randn(c - 1, n_kv, d, device=DEV).to(dtype)
+        values0[pages, :, :, (place % page).to(DEV)] = torch.randn(c - 1, n_kv, d, device=DEV).to(dtype)
+        first = 0 if window is None else max(0, c - window) // page
+        table[r, :first] = -1
+    table = table.to(DEV)
+    t = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
+    row_start, row_len, row_ctx = t(list(range(rows))), t(lens), t(ctxs)
+    positions, token_row = t([c - 1 for c in ctxs]), t(list(range(rows)))
+    qkv = torch.randn(rows, (n_q + 2 * n_kv) * d, device=DEV).to(dtype)
+    qw, kw = 1 + 0.2 * torch.randn(d, device=DEV), 1 + 0.2 * torch.randn(d, device=DEV)
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, d, 2).float() / d))).to(DEV)
+    cos_sin = ops.rotary_table(positions, inv_freq)
+    scale = d ** -0.5
+    for fixed in (None, 8):
+        plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, fixed_splits=fixed)
+        staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
+                  "merges": torch.from_numpy(plan.merges).to(DEV), "n_items": len(plan.items), "n_merges": len(plan.merges),
+                  "n_slots": plan.n_slots}
+        assert plan.n_slots > 0 or window is not None                       # long contexts are split, unless a window keeps them short
+        for norm, rope in ((True, True), (False, True), (True, False)):
+            w_q, w_k, cs = (qw if norm else None), (kw if norm else None), (cos_sin if rope else None)
+            # the separate kernels, and the plain twin of both
+            sep_qkv, sep_k, sep_v = qkv.clone(), keys0.clone(), values0.clone()
+            ops.qk_norm_rope_kv_write(sep_qkv, sep_k, sep_v, table.clamp(min=0), token_row, positions, w_q, w_k, 1e-6, cs, page, n_q, n_kv, d, True)
+            sep_out = torch.zeros(rows, n_q * d, device=DEV, dtype=dtype)
+            ops.paged_attention(sep_qkv, sep_out, sep_k, sep_v, table, row_start, row_len, row_ctx, staged, scale, window, page, n_q, n_kv, d, Ctx())
+            ref_qkv, ref_k, ref_v = qkv.clone(), keys0.clone(), values0.clone()
+            TorchOps().qk_norm_rope_kv_write(ref_qkv, ref_k, ref_v, table.clamp(min=0), token_row, positions, w_q, w_k, 1e-6, cs, page, n_q, n_kv, d, True)
+            ref_out = torch.zeros_like(sep_out)
+            TorchOps().paged_attention(ref_qkv, ref_out, ref_k, ref_v, table.clamp(min=0), row_start, row_len, row_ctx, None, scale, window, page, n_q, n_kv, d, None)
+            # fused, writing the cache
+            raw, got_k, got_v = qkv.clone(), keys0.clone(), values0.clone()
+            got = torch.zeros_like(sep_out)
+            ops.paged_attention(raw, got, got_k, got_v, table, row_start, row_len, row_ctx, staged, scale, window, page, n_q, n_kv, d, Ctx(),
+                                decode_fusion=(w_q, w_k, 1e-6, cs, True))
+            torch.cuda.synchronize()
+            assert torch.equal(raw, qkv)                                     # the projection is read, not rewritten
+            close(got, ref_out, dtype)
+            torch.testing.assert_close(got.float(), sep_out.float(), atol=2e-2, rtol=2e-2)
+            close(got_k, ref_k, dtype)
+            assert torch.equal(got_v, ref_v)
+            # fused, reading a cache that already holds the new token (another layer wrote it)
+            kept_k, kept_v = sep_k.clone(), sep_v.clone()
+            got = torch.zeros_like(sep_out)
+            ops.paged_attention(raw, got, kept_k, kept_v, table, row_start, row_len, row_ctx, staged, scale, window, page, n_q, n_kv, d, Ctx(),
+                                decode_fusion=(w_q, w_k, 1e-6, cs, False))
+            close(got, ref_out, dtype)
+            assert torch.equal(kept_k, sep_k) and torch.equal(kept_v, sep_v)
+    with pytest.raises(ValueError):                                          # a row with two tokens
+        ops.paged_attention(torch.zeros(rows + 1, (n_q + 2 * n_kv) * d, device=DEV, dtype=dtype), torch.zeros(rows + 1, n_q * d, device=DEV, dtype=dtype),
+                            keys0, values0, table, row_start, row_len, row_ctx, staged, scale, window, page, n_q, n_kv, d, Ctx(),
+                            decode_fusion=(qw, kw, 1e-6, cos_sin, True))
+    assert not ops.decode_fusion_fits(torch.float32, d) and not ops.decode_fusion_fits(dtype, 80)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_long_context_splits_and_needle(ops, dtype):
     print(f"attention long {dtype}", flush=True)
