@@ -17,8 +17,8 @@
 //     rsqrt(sum / K + eps) in the epilogue.
 //   * Stream update.  The result is an update of a residual stream that a norm follows.  The
 //     epilogue then forms s' = round(resid + round(y)), and writes s', round(s' * norm_weight) and
-//     the sum of s'^2 over each 16 columns ([M, ceil(N / 16)]): exactly what the row scale of the
-//     next product takes.
+//     the sums of s'^2 over the columns of each of its tiles ([M, P]): exactly what the row scale of
+//     the next product takes.
 #include "common.hpp"
 
 using namespace lsa;
@@ -40,7 +40,7 @@ struct Fusion {
     const float* norm_weight;            // [N]
     bf16_t* resid_out;                   // [M, N]
     bf16_t* weighted_out;                // [M, N]
-    float* square_sums_out;              // [M, ceil(N / 16)]
+    float* square_sums_out;              // [M, P], P as lsa_gemm_skinny_parts tells
 };
 
 // The partial sums of wavefront `wave`'s row are loaded behind the last operands of the product
@@ -69,8 +69,8 @@ __device__ inline void row_scale_finish(const RowScaleLoads& loads, const Fusion
 
 // Epilogue of the stream update for one element (m, n) of the result; the 16 lanes that hold
 // the 16 columns of a tile for one m are neighbours, so the sum of squares is four shuffles.
-__device__ inline void stream_update(const Fusion& f, float total, int m, int n, int M, int N, int tile_index, int tiles) {
-    const bool inside = m < M && n < N;
+__device__ inline void stream_update(const Fusion& f, float total, int m, int n, int M, int N, bool own, int tile_index, int tiles) {
+    const bool inside = own && m < M && n < N;
     float s = 0.f;
     if (inside) {
         const size_t at = (size_t)m * N + n;
@@ -94,15 +94,18 @@ __device__ inline void stream_update(const Fusion& f, float total, int m, int n,
 // launcher picks the one that divides a wavefront's share of K with the least waste.
 template <int MT, typename OutT, bool GATED, int CH>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                                      OutT* __restrict__ y, int M, int N, int K, Fusion fusion) {
+                                                                      OutT* __restrict__ y, int M, int N, int K, int R, Fusion fusion) {
     __shared__ float partial[GEMM_WAVES][MT][256];
     __shared__ float row_scale[GEMM_WAVES];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, quad = lane >> 4;
-    const int n0 = blockIdx.x * (GATED ? 8 : 16);
+    // R of the tile's 16 rows are this workgroup's own (GATED: 8 gate rows and 8 up rows); the other lanes
+    // load the last of them again, which costs no traffic, and their results are dropped.
+    const int n0 = blockIdx.x * (GATED ? 8 : R);
     const int k_per_wave = ((K + GEMM_WAVES - 1) / GEMM_WAVES + 31) / 32 * 32;
     const int k_begin = min(K, wave * k_per_wave), k_end = min(K, k_begin + k_per_wave);
-    const int w_row = GATED ? (col < 8 ? min(n0 + col, N / 2 - 1) : N / 2 + min(n0 + col - 8, N / 2 - 1)) : min(n0 + col, N - 1);
+    const int w_row = GATED ? (col < 8 ? min(n0 + col, N / 2 - 1) : N / 2 + min(n0 + col - 8, N / 2 - 1))
+                            : min(n0 + min(col, R - 1), N - 1);
     const bf16_t* wp = w + (size_t)w_row * K + 8 * quad;
     const bf16_t* xp[MT];
 #pragma unroll
@@ -192,10 +195,10 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
             continue;
         }
         if (MT == 1 && sizeof(OutT) == 2 && fusion.resid) {
-            stream_update(fusion, total, m, n, M, N, blockIdx.x, gridDim.x);
+            stream_update(fusion, total, m, n, M, N, j < R, blockIdx.x, gridDim.x);
             continue;
         }
-        if (m < M && n < N) y[(size_t)m * N + n] = (OutT)total;
+        if (m < M && j < R && n < N) y[(size_t)m * N + n] = (OutT)total;
     }
 }
 
@@ -206,17 +209,20 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
 // it only where N gives enough workgroups of this size to fill the chip.
 template <typename OutT, bool GATED, int CH>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                                           OutT* __restrict__ y, int M, int N, int K, Fusion fusion) {
+                                                                           OutT* __restrict__ y, int M, int N, int K, int R, Fusion fusion) {
     __shared__ float partial[GEMM_WAVES][2][256];
     __shared__ float row_scale[GEMM_WAVES];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, quad = lane >> 4;
     const int half = N / 2;                                        // GATED: rows of the gate matrix
-    const int n0 = blockIdx.x * (GATED ? 16 : 32);
+    // The workgroup's own rows: R (16 < R <= 32) consecutive ones, 16 in the first tile; GATED: R <= 16 gate rows
+    // in the first tile, their up rows in the second.  Lanes beyond them load the last own row again.
+    const int n0 = blockIdx.x * R;
+    const int own0 = GATED ? R : 16, own1 = GATED ? R : R - 16;                     // own rows of the two tiles
     const int k_per_wave = ((K + GEMM_WAVES - 1) / GEMM_WAVES + 31) / 32 * 32;
     const int k_begin = min(K, wave * k_per_wave), k_end = min(K, k_begin + k_per_wave);
-    const int row0 = GATED ? min(n0 + col, half - 1) : min(n0 + col, N - 1);
-    const int row1 = GATED ? half + min(n0 + col, half - 1) : min(n0 + 16 + col, N - 1);
+    const int row0 = GATED ? min(n0 + min(col, own0 - 1), half - 1) : min(n0 + col, N - 1);
+    const int row1 = GATED ? half + min(n0 + min(col, own1 - 1), half - 1) : min(n0 + 16 + min(col, own1 - 1), N - 1);
     const bf16_t* wp0 = w + (size_t)row0 * K + 8 * quad;
     const bf16_t* wp1 = w + (size_t)row1 * K + 8 * quad;
     const bf16_t* xp = x + (size_t)min(col, M - 1) * K + 8 * quad;
@@ -294,7 +300,7 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_wide_kernel(const
         }
         gate *= scale;
         up *= scale;
-        if (m < M && n0 + j < half) y[(size_t)m * half + n0 + j] = (OutT)(gate / (1.f + expf(-gate)) * up);
+        if (m < M && j < own0 && n0 + j < half) y[(size_t)m * half + n0 + j] = (OutT)(gate / (1.f + expf(-gate)) * up);
         return;
     }
     float total = 0.f;
@@ -302,11 +308,12 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_wide_kernel(const
     for (int v = 0; v < GEMM_WAVES; ++v) total += partial[v][tile][in_tile];
     total *= scale;
     const int n = n0 + 16 * tile + j;
+    const bool own = j < (tile ? own1 : own0);
     if (sizeof(OutT) == 2 && fusion.resid) {
-        stream_update(fusion, total, m, n, M, N, 2 * blockIdx.x + tile, (N + 15) / 16);
+        stream_update(fusion, total, m, n, M, N, own, 2 * blockIdx.x + tile, 2 * gridDim.x);
         return;
     }
-    if (m < M && n < N) y[(size_t)m * N + n] = (OutT)total;
+    if (m < M && own && n < N) y[(size_t)m * N + n] = (OutT)total;
 }
 
 // The chunk size in 4..8 that wastes the fewest loads past the end of a wavefront's share of K.
@@ -323,23 +330,56 @@ static int best_chunk(int K) {
     return chunk;
 }
 
-// Whether workgroups of two tiles suit `tiles` 16-row tiles of W: they halve the activations' share
-// of the traffic, which saves `gain_percent` of the time (measured: about 15 with the gated epilogue,
-// where one tile means two half tiles; for the plain product about 10 at 9 to 16 rows, 3 at 4 to 8
-// and a loss below that), but must still fill the compute units in whole rounds.
-static bool two_tiles_pay(int M, long tiles, int tiling, int gain_percent) {
-    if (M > 16 || tiling == 1) return false;
-    if (tiling == 2) return true;
-    if (gain_percent <= 0) return false;
+static int compute_units() {
     static int units = 0;
     if (!units) {
         int device = 0;
         hipDeviceProp_t prop;
-        if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) return false;
-        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
+            units = prop.multiProcessorCount;
+        else
+            units = 256;
     }
-    const long rounds_one = (tiles + units - 1) / units, rounds_two = ((tiles + 1) / 2 + units - 1) / units;
-    return 2 * rounds_two * (100 - gain_percent) < rounds_one * 100;
+    return units;
+}
+
+// Rows of W per workgroup.  The compute units work through the workgroups in rounds, a round takes
+// as long as its workgroups have rows (plus a fixed part), and a round that is not full costs as
+// much as a full one: so the best size is the one with the smallest rounds * (rows + fixed part).
+// Up to 16 rows are one tile per wavefront, 17 to 32 two tiles, which halves the activations'
+// share of what a workgroup loads (measured: worth 10 % at 9 to 16 rows of activations, 3 % at 4
+// to 8, and a loss of as much below that, where the activations come from the first-level cache).
+// GATED counts pairs of a gate row and an up row: one tile of 8 pairs, or two tiles of up to 16.
+// `request`: 0 picks, otherwise the size to use (GATED: -1 for the one-tile form).
+static int choose_rows(int M, int N, bool gated, int request) {
+    const long total = gated ? N / 2 : N;
+    const int units = compute_units();
+    if (gated) {
+        if (request == -1) return -1;
+        if (request > 0) return request;
+        long best_cost = ((total + 7) / 8 + units - 1) / units * 21;                 // one tile: 8 pairs + 2.5
+        int best = -1;
+        for (int r = 16; r >= 8; r -= 2) {
+            const long cost = ((total + r - 1) / r + units - 1) / units * (2 * r + 4);   // two tiles: r pairs + 2
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = r;
+            }
+        }
+        return best;
+    }
+    if (request > 0) return request;
+    long best_cost = -1;
+    int best = 16;
+    for (int r = (M <= 16 ? 32 : 16); r >= 8; r -= 4) {
+        long cost = ((total + r - 1) / r + units - 1) / units * (r + 4) * 100;
+        if (r > 16 && M < 4) cost = cost * 115 / 100;
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best = r;
+        }
+    }
+    return best;
 }
 
 #define LSA_FOR_CHUNK(chunk, LAUNCH)   \
@@ -351,29 +391,39 @@ static bool two_tiles_pay(int M, long tiles, int tiling, int gain_percent) {
         default: LAUNCH(8); break;     \
     }
 
+// Workgroups and partial sums of squares per row (stream update) for a size.
+static void layout(int N, bool gated, int rows, int* workgroups, int* parts) {
+    const long total = gated ? N / 2 : N;
+    const int r = rows == -1 ? 8 : rows;
+    *workgroups = (int)((total + r - 1) / r);
+    *parts = (!gated && rows > 16) ? 2 * *workgroups : *workgroups;
+}
+
 template <typename OutT, bool GATED>
-static int launch(const bf16_t* x, const bf16_t* w, OutT* y, int M, int N, int K, int tiling, const Fusion& fusion, hipStream_t stream) {
+static int launch(const bf16_t* x, const bf16_t* w, OutT* y, int M, int N, int K, int rows, const Fusion& fusion, hipStream_t stream) {
     const dim3 block(GEMM_WAVES * 64);
-    const int tiles = GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;               // workgroups of one tile
-    const int gain = GATED ? 15 : M > 8 ? 10 : M >= 4 ? 3 : 0;
-    if (two_tiles_pay(M, tiles, tiling, gain)) {
-        const dim3 grid((tiles + 1) / 2);
-#define LSA_WIDE(CH) gemm_skinny_wide_kernel<OutT, GATED, CH><<<grid, block, 0, stream>>>(x, w, y, M, N, K, fusion)
+    int workgroups, parts;
+    layout(N, GATED, rows, &workgroups, &parts);
+    const dim3 grid(workgroups);
+    const bool two_tiles = GATED ? rows != -1 : rows > 16;
+    if (two_tiles) {
+        if (M > 16 || rows > (GATED ? 16 : 32)) return -1;
+#define LSA_WIDE(CH) gemm_skinny_wide_kernel<OutT, GATED, CH><<<grid, block, 0, stream>>>(x, w, y, M, N, K, rows, fusion)
         LSA_FOR_CHUNK(best_chunk(K), LSA_WIDE)
 #undef LSA_WIDE
         LSA_LAUNCH_CHECK();
     }
-    const dim3 grid(tiles);
+    if (rows < 1 && !GATED) return -1;
     if (M <= 16) {
-#define LSA_ONE(CH) gemm_skinny_kernel<1, OutT, GATED, CH><<<grid, block, 0, stream>>>(x, w, y, M, N, K, fusion)
+#define LSA_ONE(CH) gemm_skinny_kernel<1, OutT, GATED, CH><<<grid, block, 0, stream>>>(x, w, y, M, N, K, rows, fusion)
         LSA_FOR_CHUNK(best_chunk(K), LSA_ONE)
 #undef LSA_ONE
     } else if (GATED) {
         return -1;
     } else if (M <= 32) {
-        gemm_skinny_kernel<2, OutT, false, 8><<<grid, block, 0, stream>>>(x, w, y, M, N, K, fusion);
+        gemm_skinny_kernel<2, OutT, false, 8><<<grid, block, 0, stream>>>(x, w, y, M, N, K, rows, fusion);
     } else {
-        gemm_skinny_kernel<4, OutT, false, 4><<<grid, block, 0, stream>>>(x, w, y, M, N, K, fusion);
+        gemm_skinny_kernel<4, OutT, false, 4><<<grid, block, 0, stream>>>(x, w, y, M, N, K, rows, fusion);
     }
     LSA_LAUNCH_CHECK();
 }
@@ -385,43 +435,54 @@ static bool fusion_fits(int M, const float* square_sums, int n_parts, const void
     return true;
 }
 
-// out_float32: 0 writes bfloat16, 1 writes float32.  tiling: tiles of W per workgroup, 1 or 2 (2 only for
-// M <= 16), or 0 to let the size decide.  square_sums [M, n_parts] (or null) asks for the row scale
+// out_float32: 0 writes bfloat16, 1 writes float32.  rows: rows of W per workgroup, 1 to 32 (more than 16
+// only for M <= 16), or 0 to let the size decide.  square_sums [M, n_parts] (or null) asks for the row scale
 // rsqrt(sum / K + eps), M <= 8.  Refuses (returns -1) what it cannot take.
-LSA_EXPORT int lsa_gemm_skinny(int out_float32, const void* x, const void* w, void* y, int M, int N, int K, int tiling,
+LSA_EXPORT int lsa_gemm_skinny(int out_float32, const void* x, const void* w, void* y, int M, int N, int K, int rows,
                                const float* square_sums, int n_parts, float eps, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 64 || K % 8 != 0 || K < 8 || tiling < 0 || tiling > 2 || (tiling == 2 && M > 16)) return -1;
+    if (M > 64 || K % 8 != 0 || K < 8 || rows < 0 || rows > 32 || (rows > 16 && M > 16)) return -1;
     if (!fusion_fits(M, square_sums, n_parts, nullptr)) return -1;
     const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr};
-    return out_float32 ? launch<float, false>((const bf16_t*)x, (const bf16_t*)w, (float*)y, M, N, K, tiling, fusion, stream)
-                       : launch<bf16_t, false>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, tiling, fusion, stream);
+    rows = choose_rows(M, N, false, rows);
+    return out_float32 ? launch<float, false>((const bf16_t*)x, (const bf16_t*)w, (float*)y, M, N, K, rows, fusion, stream)
+                       : launch<bf16_t, false>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, rows, fusion, stream);
+}
+
+// Partial sums per row that lsa_gemm_skinny_stream writes for this size (the second dimension of square_sums_out).
+LSA_EXPORT int lsa_gemm_skinny_parts(int M, int N, int rows) {
+    if (M <= 0 || N <= 0 || rows < 0 || rows > 32) return -1;
+    int workgroups, parts;
+    layout(N, false, choose_rows(M, N, false, rows), &workgroups, &parts);
+    return parts;
 }
 
 // The product as an update of a residual stream that a norm follows (see the top of the file), M <= 8:
 //   resid_out = round(resid + round(x . w^T [/ rms, if square_sums])), weighted_out = round(resid_out * norm_weight),
-//   square_sums_out [M, ceil(N / 16)] = sums of resid_out^2 over each 16 columns.
+//   square_sums_out [M, lsa_gemm_skinny_parts(M, N, rows)] = sums of resid_out^2 over the columns of each tile.
 // resid_out may be resid itself.
-LSA_EXPORT int lsa_gemm_skinny_stream(const void* x, const void* w, int M, int N, int K, int tiling,
+LSA_EXPORT int lsa_gemm_skinny_stream(const void* x, const void* w, int M, int N, int K, int rows,
                                       const float* square_sums, int n_parts, float eps,
                                       const void* resid, const float* norm_weight, void* resid_out, void* weighted_out,
                                       float* square_sums_out, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (K % 8 != 0 || K < 8 || tiling < 0 || tiling > 2 || !resid || !norm_weight || !resid_out || !weighted_out || !square_sums_out)
+    if (K % 8 != 0 || K < 8 || rows < 0 || rows > 32 || !resid || !norm_weight || !resid_out || !weighted_out || !square_sums_out)
         return -1;
     if (!fusion_fits(M, square_sums, n_parts, resid)) return -1;
     const Fusion fusion = {square_sums, n_parts, eps, (const bf16_t*)resid, norm_weight, (bf16_t*)resid_out, (bf16_t*)weighted_out,
                            square_sums_out};
-    return launch<bf16_t, false>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)nullptr, M, N, K, tiling, fusion, stream);
+    return launch<bf16_t, false>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)nullptr, M, N, K, choose_rows(M, N, false, rows), fusion, stream);
 }
 
 // hidden[M, I] = silu(x . gate^T) * (x . up^T) with gate_up [2I, K] (gate rows first); M <= 16, I a multiple of 8.
-// square_sums as in lsa_gemm_skinny.
-LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* hidden, int M, int I, int K, int tiling,
+// rows: pairs of a gate and an up row per workgroup in the two-tile form, 1 to 16; -1: the one-tile form (8 pairs);
+// 0 to let the size decide.  square_sums as in lsa_gemm_skinny.
+LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* hidden, int M, int I, int K, int rows,
                                      const float* square_sums, int n_parts, float eps, hipStream_t stream) {
     if (M <= 0 || I <= 0) return 0;
-    if (M > 16 || K % 8 != 0 || K < 8 || I % 8 != 0 || tiling < 0 || tiling > 2) return -1;
+    if (M > 16 || K % 8 != 0 || K < 8 || I % 8 != 0 || rows < -1 || rows > 16) return -1;
     if (!fusion_fits(M, square_sums, n_parts, nullptr)) return -1;
     const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr};
-    return launch<bf16_t, true>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)hidden, M, 2 * I, K, tiling, fusion, stream);
+    return launch<bf16_t, true>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)hidden, M, 2 * I, K, choose_rows(M, 2 * I, true, rows),
+                                fusion, stream);
 }

@@ -107,26 +107,27 @@ class HipOps:
         """Whether the few-row products take ``x`` with this ``row_scale`` (then they do not return None for it)."""
         return x.shape[1] == weight.shape[1] and self._few_rows(x, weight) and self._row_scale_fits(row_scale, x.shape[0])
 
-    def linear(self, x, weight, out=None, out_float32=False, tiling=0):
-        """``x [T, in] @ weight[out, in]^T``; float32 result if asked (the output head).  ``tiling`` picks the
-        few-row kernel's workgroup shape (1 or 2 tiles of the weight; 0 lets the size decide)."""
+    def linear(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0):
+        """``x [T, in] @ weight[out, in]^T``; float32 result if asked (the output head).  ``rows_per_workgroup``
+        fixes the few-row kernel's share of the weight per workgroup (1 to 32; 0 lets the size decide)."""
         if x.shape[1] != weight.shape[1]:
             raise ValueError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
         if self._few_rows(x, weight):
             # Few rows: the product is a stream over the weights; the hand-written kernel reads them once at HBM rate.
-            return self.linear_few_rows(x, weight, out=out, out_float32=out_float32, tiling=tiling)
+            return self.linear_few_rows(x, weight, out=out, out_float32=out_float32, rows_per_workgroup=rows_per_workgroup)
         if out_float32 and x.dtype != torch.float32:
             return torch.mm(x, weight.t(), out_dtype=torch.float32)
         return torch.mm(x, weight.t(), out=out) if out is not None else torch.mm(x, weight.t())
 
-    def linear_few_rows(self, x, weight, out=None, out_float32=False, tiling=0, row_scale=None):
+    def linear_few_rows(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0, row_scale=None):
         """The weight-streaming product, or None if this is no case for it.
 
         ``row_scale = (square_sums [T, P], eps)``: ``x`` is a residual stream already multiplied by a norm's
         weights, ``square_sums`` are partial sums of the stream's squares, and the result rows are divided by the
         stream's root mean square, so that the result is the product of the normalised stream (up to 8 rows)."""
         rows, width = x.shape
-        if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or not self._row_scale_fits(row_scale, rows):
+        if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or not self._row_scale_fits(row_scale, rows) \
+                or (rows_per_workgroup > 16 and rows > 16):
             return None
         _check(x, "x", torch.bfloat16)
         _check(weight, "weight", torch.bfloat16)
@@ -135,15 +136,15 @@ class HipOps:
         _check(out, "out", None, (rows, weight.shape[0]))
         sums, parts, eps = self._row_scale_args(row_scale, rows)
         _launched(self._gemm.lsa_gemm_skinny(1 if out_float32 else 0, _ptr(x), _ptr(weight), _ptr(out), rows, weight.shape[0], width,
-                                             int(tiling), sums, parts, eps, _stream()), "gemm_skinny")
+                                             int(rows_per_workgroup), sums, parts, eps, _stream()), "gemm_skinny")
         return out
 
-    def linear_into_stream(self, x, weight, resid, norm_weight, tiling=0, row_scale=None):
+    def linear_into_stream(self, x, weight, resid, norm_weight, rows_per_workgroup=0, row_scale=None):
         """The few-row product as an update of the residual stream ``resid [T, out]`` that a norm with weights
         ``norm_weight`` follows, in one launch: returns ``(stream, weighted, square_sums)`` with
         ``stream = resid + x @ weight^T`` (a new tensor), ``weighted = stream * norm_weight`` and
-        ``square_sums [T, ceil(out / 16)]`` partial sums of ``stream^2``, which is what ``row_scale`` of the next
-        product takes.  None if this is no case for it (more than 8 rows, other types)."""
+        ``square_sums [T, P]`` partial sums of ``stream^2`` (one per tile of the kernel's workgroups), which is what
+        ``row_scale`` of the next product takes.  None if this is no case for it (more than 8 rows, other types)."""
         rows, width = x.shape
         n = weight.shape[0]
         if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or rows > self.FUSED_ROWS \
@@ -155,17 +156,21 @@ class HipOps:
         _check(norm_weight, "norm_weight", torch.float32, (n,))
         stream = torch.empty_like(resid)
         weighted = torch.empty_like(resid)
-        square_sums = torch.empty((rows, (n + 15) // 16), device=x.device, dtype=torch.float32)
+        n_sums = self._gemm.lsa_gemm_skinny_parts(rows, n, int(rows_per_workgroup))
+        if n_sums <= 0:
+            raise ValueError(f"linear_into_stream: no layout for {rows} x {n} with {rows_per_workgroup} rows per workgroup")
+        square_sums = torch.empty((rows, n_sums), device=x.device, dtype=torch.float32)
         sums, parts, eps = self._row_scale_args(row_scale, rows)
-        _launched(self._gemm.lsa_gemm_skinny_stream(_ptr(x), _ptr(weight), rows, n, width, int(tiling), sums, parts, eps, _ptr(resid),
+        _launched(self._gemm.lsa_gemm_skinny_stream(_ptr(x), _ptr(weight), rows, n, width, int(rows_per_workgroup), sums, parts, eps, _ptr(resid),
                                                     _ptr(norm_weight), _ptr(stream), _ptr(weighted), _ptr(square_sums), _stream()),
                   "gemm_skinny_stream")
         return stream, weighted, square_sums
 
-    def linear_gated(self, x, gate_up_weight, tiling=0, row_scale=None):
+    def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None):
         """``silu(x @ gate^T) * (x @ up^T)`` with ``gate_up_weight [2I, K]`` in one launch for few rows (the
-        activation sits in the product's epilogue), or None if this is not such a case.  ``row_scale`` as in
-        :meth:`linear_few_rows`."""
+        activation sits in the product's epilogue), or None if this is not such a case.  ``pairs_per_workgroup``:
+        1 to 16 pairs of a gate and an up row in two tiles, -1 for 8 pairs in one tile, 0 lets the size decide.
+        ``row_scale`` as in :meth:`linear_few_rows`."""
         rows, width = x.shape
         inter = gate_up_weight.shape[0] // 2
         if not self._few_rows(x, gate_up_weight) or inter % 8 or gate_up_weight.shape[1] != width or rows > 16 \
@@ -175,7 +180,7 @@ class HipOps:
         _check(gate_up_weight, "gate_up_weight", torch.bfloat16)
         out = torch.empty((rows, inter), device=x.device, dtype=torch.bfloat16)
         sums, parts, eps = self._row_scale_args(row_scale, rows)
-        _launched(self._gemm.lsa_gemm_skinny_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, int(tiling), sums, parts,
+        _launched(self._gemm.lsa_gemm_skinny_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, int(pairs_per_workgroup), sums, parts,
                                                    eps, _stream()), "gemm_skinny_gated")
         return out
 

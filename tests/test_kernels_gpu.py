@@ -364,7 +364,8 @@ def test_sampling(ops, vocab):
 def test_skinny_gemm(ops, rows, n, k):
     """The weight-streaming product against a float64 product of the same bfloat16 values: widths and
     output sizes that are no multiple of the tiles, widths that give a wavefront 4, 5, 6, 7 or 8 k steps
-    at a time, one or two tiles of the weight per workgroup, float32 and bfloat16 results."""
+    at a time, whole and partly used tiles of the weight per workgroup, one or two of them, float32 and
+    bfloat16 results."""
     print(f"skinny gemm rows {rows} n {n} k {k}", flush=True)
     torch.manual_seed(rows * n + k)
     x = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
@@ -373,9 +374,9 @@ def test_skinny_gemm(ops, rows, n, k):
     saved = ops.skinny_rows
     try:
         ops.skinny_rows = 64
-        for tiling in (0, 1, 2) if rows <= 16 else (0, 1):
-            got32 = ops.linear(x, w, out_float32=True, tiling=tiling)
-            got16 = ops.linear(x, w, tiling=tiling)
+        for per in (0, 16, 8, 3, 24, 32, 17) if rows <= 16 else (0, 16, 12):
+            got32 = ops.linear(x, w, out_float32=True, rows_per_workgroup=per)
+            got16 = ops.linear(x, w, rows_per_workgroup=per)
             assert got32.dtype == torch.float32 and got16.dtype == torch.bfloat16
             torch.testing.assert_close(got32, expected, atol=2e-4, rtol=1e-4)          # 32-bit accumulation of exact products
             torch.testing.assert_close(got16.float(), expected, atol=2e-2, rtol=1e-2)
@@ -407,9 +408,9 @@ def test_skinny_gemm_with_row_scale_and_stream_update(ops, rows, n, k):
     weighted = (stream.float() * norm_weight).to(torch.bfloat16)
     rstd = torch.rsqrt(squares.double().sum(1, keepdim=True) / k + eps)
     expected = (weighted.double() @ w.double().t()) * rstd
-    for tiling in (0, 1, 2):
+    for per in (0, 16, 12, 24, 32):
         for out32 in (False, True):
-            got = ops.linear_few_rows(weighted, w, out_float32=out32, tiling=tiling, row_scale=(square_sums, eps))
+            got = ops.linear_few_rows(weighted, w, out_float32=out32, rows_per_workgroup=per, row_scale=(square_sums, eps))
             assert got.dtype == (torch.float32 if out32 else torch.bfloat16)
             torch.testing.assert_close(got.double(), expected, atol=2e-4 if out32 else 3e-2, rtol=1e-4 if out32 else 2e-2)
     # ... and it is the product of the normalised stream, up to the rounding of the normalised values
@@ -423,16 +424,16 @@ def test_skinny_gemm_with_row_scale_and_stream_update(ops, rows, n, k):
     y = (x.double() @ w.double().t()).float().to(torch.bfloat16)
     want_stream = (resid.float() + y.float()).to(torch.bfloat16)
     want_weighted = (want_stream.float() * next_weight).to(torch.bfloat16)
-    for tiling in (0, 1, 2):
+    for per in (0, 16, 12, 24, 32):
         kept = resid.clone()
-        got_stream, got_weighted, got_sums = ops.linear_into_stream(x, w, kept, next_weight, tiling=tiling)
+        got_stream, got_weighted, got_sums = ops.linear_into_stream(x, w, kept, next_weight, rows_per_workgroup=per)
         assert torch.equal(kept, resid)
         # y is rounded once to bfloat16 before the sum, as the separate kernels do; a product that lands on a
         # rounding boundary may differ by one step of bfloat16
         torch.testing.assert_close(got_stream.float(), want_stream.float(), atol=4e-2, rtol=1e-2)
         assert float((got_stream.float() - want_stream.float()).abs().gt(0).float().mean()) < 0.02
         torch.testing.assert_close(got_weighted.float(), (got_stream.float() * next_weight).to(torch.bfloat16).float(), atol=0, rtol=0)
-        assert got_sums.shape == (rows, (n + 15) // 16)
+        assert got_sums.shape[0] == rows and (per == 0 or got_sums.shape[1] == -(-n // per) * (2 if per > 16 else 1))
         torch.testing.assert_close(got_sums.sum(1), (got_stream.float() ** 2).sum(1), atol=1e-3, rtol=1e-5)
     # chained: the producer's outputs feed a consumer of width n
     w2 = (torch.randn(72, n, device=DEV) / n ** 0.5).to(torch.bfloat16)
@@ -464,10 +465,10 @@ def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
     square_sums = torch.rand(rows, 5, device=DEV) * k
     rstd = torch.rsqrt(square_sums.double().sum(1, keepdim=True) / k + 1e-6)
     scaled = (torch.nn.functional.silu(gate_up[:, :inter] * rstd) * gate_up[:, inter:] * rstd).float()
-    for tiling in (0, 1, 2):
-        got = ops.linear_gated(x, w, tiling=tiling)
+    for per in (0, -1, 16, 12, 5):
+        got = ops.linear_gated(x, w, pairs_per_workgroup=per)
         assert got.shape == (rows, inter) and got.dtype == torch.bfloat16
         torch.testing.assert_close(got.float(), expected, atol=2e-2, rtol=2e-2)
-        got = ops.linear_gated(x, w, tiling=tiling, row_scale=(square_sums, 1e-6))
+        got = ops.linear_gated(x, w, pairs_per_workgroup=per, row_scale=(square_sums, 1e-6))
         torch.testing.assert_close(got.float(), scaled, atol=2e-2, rtol=2e-2)
     assert ops.linear_gated(torch.zeros(9, k, device=DEV, dtype=torch.bfloat16), w) is None
