@@ -465,22 +465,33 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
 
 #if LSA_BF16
 // ------------------------------------------------------------------------------------------------
-// Portions of prompts: four wavefronts of a workgroup take four consecutive tiles of 16 pairs of
-// one request.  They see (almost) the same keys, so each step's 32 keys and values are fetched
+// Portions of prompts: the four wavefronts of a workgroup take 4 * SUB consecutive tiles of 16 pairs
+// of one request (SUB tiles each).  They see (almost) the same keys, so each step's 32 keys and values are fetched
 // from the pages once per workgroup into LDS (double-buffered: the global loads of step i+1 are
 // issued before the products of step i and stored to the other buffer afterwards, one barrier a
 // step) and every wavefront reads its MFMA operands from there.  Rows in LDS are padded so that
 // the operand reads of a wavefront spread over the banks.  No key ranges are split here: such
-// rows have many tiles.  `tiles[i]` = {row, first token of the workgroup's 4 tiles, k_begin, k_end}.
+// rows have many tiles.  `tiles[i]` = {row, first token of the workgroup's tiles, k_begin, k_end}.
 constexpr int K_ROW = D * 2 + 16;                 // bytes of a key row in LDS
 constexpr int V_ROW = 32 * 2 + 8;                 // bytes of a value row (one head dimension, 32 keys)
 constexpr int K_TILE_BYTES = 32 * K_ROW, V_TILE_BYTES = D * V_ROW;
-constexpr int K_PIECES = 32 * (D / 8), V_PIECES = D * 8;       // 16-byte pieces of keys, 8-byte pieces of values
-constexpr int KPT = (K_PIECES + 255) / 256, VPT = (V_PIECES + 255) / 256;
-// Three wavefronts per SIMD hide the latency of a step's dependent chain (LDS read, MFMA, softmax, MFMA).
-#define LSA_TILE_MIN_WAVES (LSA_ND <= 8 ? 3 : 1)
+// A step is fetched as two halves of 16 keys (with pages of 16 or more keys each half lies in one page):
+// per half, 16-byte pieces of keys (16 keys x D, contiguous in the page) and 8-byte pieces of values (D rows of 4 keys).
+constexpr int K_HALF_PIECES = 16 * (D / 8), V_HALF_PIECES = D * 4;
+constexpr int KPH = (K_HALF_PIECES + 255) / 256, VPH = (V_HALF_PIECES + 255) / 256;      // pieces per thread and half
+// Tiles of 16 pairs per wavefront (SUB): with two, every key and value operand read from LDS feeds two products, which
+// halves the LDS traffic per flop (the kernel's limit); the accumulators of two tiles fit the registers up to a head size of 128.
+// The host picks one or two per launch: two pay when the rows are long (the longest workgroup then does not
+// decide the time), one when they are short and there are few workgroups.
+constexpr int MAX_SUB = LSA_ND <= 8 ? 2 : 1;
+// Wavefronts per SIMD wanted (they hide the latency of a step's dependent chain: LDS read, MFMA, softmax, MFMA),
+// as far as the registers of SUB tiles allow.
+#define LSA_TILE_MIN_WAVES(SUB) ((SUB) == 1 ? (LSA_ND <= 8 ? 3 : 1) : (LSA_ND <= 4 ? 3 : 2))
+struct FullStep { static constexpr bool value = true; };        // every key of the step is seen by every pair
+struct MaskedStep { static constexpr bool value = false; };
 
-__global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES) void paged_attention_tile_kernel(
+template <int SUB>
+__global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_tile_kernel(
     const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
     const elem_t* __restrict__ keys, const elem_t* __restrict__ values,
     const int* __restrict__ table, int table_stride,
@@ -498,36 +509,47 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES) void paged_attention_tile_
     const int col = lane & 15, quad = lane >> 4;
     const int row = tile.row;
     const int n = row_len[row], first_pos = row_ctx[row] - n;
-    const int q0 = tile.q0 + wave * g.tokens_per_tile;          // first token of this wavefront's tile
-    const int token0 = row_start[row] + q0;
+    const int q0 = tile.q0 + wave * SUB * g.tokens_per_tile;    // first token of this wavefront's SUB consecutive tiles
     const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
-    const bool pair_valid = pair_token < g.tokens_per_tile && q0 + pair_token < n && pair_head_in_group < g.group;
-    const int q_pos = pair_valid ? first_pos + q0 + pair_token : -1;
     const int head = kv_head * g.group + pair_head_in_group;
+    bool pair_valid[SUB];
+    int q_pos[SUB];
+#pragma unroll
+    for (int u = 0; u < SUB; ++u) {
+        const int token = q0 + u * g.tokens_per_tile + pair_token;
+        pair_valid[u] = pair_token < g.tokens_per_tile && token < n && pair_head_in_group < g.group;
+        q_pos[u] = pair_valid[u] ? first_pos + token : -1;
+    }
     const int* row_table = table + (size_t)row * table_stride;
     const int ps = g.page_size;
     const size_t kv_head_keys = (size_t)kv_head * ps * D, kv_head_values = (size_t)kv_head * D * ps;
     const size_t page_elems = (size_t)g.n_kv * ps * D;
     // Keys this wavefront's pairs can see at all: [wave_lo, wave_hi).
-    const int wave_tokens = max(0, min(g.tokens_per_tile, n - q0));
+    const int wave_tokens = max(0, min(SUB * g.tokens_per_tile, n - q0));
     const int wave_hi = wave_tokens > 0 ? first_pos + q0 + wave_tokens : 0;
     const int wave_lo = g.window > 0 ? max(0, first_pos + q0 - g.window + 1) : 0;
     const int q_pos_min = first_pos + q0;                       // smallest position among the wavefront's valid pairs
     const float scale_log2 = g.scale * 1.44269504088896340736f;
 
-    bf16x8 qf[NS];
+    bf16x8 qf[SUB][NS];
+    f32x4 acc[SUB][ND];
+    float run_max[SUB], run_sum[SUB];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        const int dim = 32 * s + 8 * quad;
-        bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (pair_valid && dim < D)
-            x = *reinterpret_cast<const bf16x8*>(q + (size_t)(token0 + pair_token) * q_token_stride + (size_t)head * D + dim);
-        qf[s] = x;
+    for (int u = 0; u < SUB; ++u) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int dim = 32 * s + 8 * quad;
+            bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (pair_valid[u] && dim < D)
+                x = *reinterpret_cast<const bf16x8*>(q + (size_t)(row_start[row] + q0 + u * g.tokens_per_tile + pair_token) * q_token_stride +
+                                                     (size_t)head * D + dim);
+            qf[u][s] = x;
+        }
+#pragma unroll
+        for (int c = 0; c < ND; ++c) acc[u][c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        run_max[u] = NEG_INF;
+        run_sum[u] = 0.f;
     }
-    f32x4 acc[ND];
-#pragma unroll
-    for (int c = 0; c < ND; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float run_max = NEG_INF, run_sum = 0.f;
 
     const int k_begin = tile.k_begin, k_end = tile.k_end;
     int chunk = -1, pages_cur = 0, pages_next = 0;
@@ -547,136 +569,146 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES) void paged_attention_tile_
     };
 
     struct Staged {
-        bf16x8 k[KPT];
-        bf16x4 v[VPT];
+        bf16x8 k[2][KPH];
+        bf16x4 v[2][VPH];
     };
-    // Where each of this thread's pieces lies inside a step: constant over the steps.
-    int k_off[KPT], v_off[VPT];
-    bool k_second[KPT], v_second[VPT];             // piece belongs to keys 16..31 of the step
+    // Where each of this thread's pieces lies inside a half step: constant over the steps.  Piece q of the keys is
+    // bytes [16 q, 16 q + 16) of the half's 16 x D block; piece q of the values is keys 4 (q & 3) .. + 4 of dimension q >> 2.
+    unsigned k_off[KPH], v_off[VPH];                // byte offsets from the half's first key in the page
 #pragma unroll
-    for (int j = 0; j < KPT; ++j) {
-        const int p = min(tid + 256 * j, K_PIECES - 1), key = p / (D / 8);
-        k_second[j] = key >= 16;
-        k_off[j] = (key & 15) * D + 8 * (p % (D / 8));
-    }
+    for (int j = 0; j < KPH; ++j) k_off[j] = 16u * (unsigned)min(tid + 256 * j, K_HALF_PIECES - 1);
 #pragma unroll
-    for (int j = 0; j < VPT; ++j) {
-        const int p = min(tid + 256 * j, V_PIECES - 1), piece = p & 7;
-        v_second[j] = piece >= 4;
-        v_off[j] = (p >> 3) * ps + 4 * (piece & 3);
+    for (int j = 0; j < VPH; ++j) {
+        const int q = min(tid + 256 * j, V_HALF_PIECES - 1);
+        v_off[j] = 2u * (unsigned)((q >> 2) * ps + 4 * (q & 3));
     }
     const bool pages_of_16 = (ps & 15) == 0;        // then each half of a step (16 keys) lies inside one page
     auto issue_loads = [&](Staged& r, int kt) {
         enter_chunk(kt);
         if (pages_of_16 && kt >= k_begin && kt + 32 <= k_end) {
-            // Interior step: two page lookups for the whole wavefront (scalar), then one add per piece.
-            const int block_a = (int)__umulhi((unsigned)kt, g.page_magic), block_b = (int)__umulhi((unsigned)(kt + 16), g.page_magic);
-            const int slot_a = kt - block_a * ps, slot_b = kt + 16 - block_b * ps;
-            const size_t page_a = (size_t)__builtin_amdgcn_readlane(pages_cur, block_a - 64 * chunk) * page_elems;
-            const size_t page_b = (size_t)__builtin_amdgcn_readlane(pages_cur, block_b - 64 * chunk) * page_elems;
-            const elem_t* ka = keys + page_a + kv_head_keys + (size_t)slot_a * D;
-            const elem_t* kb = keys + page_b + kv_head_keys + (size_t)slot_b * D;
-            const elem_t* va = values + page_a + kv_head_values + slot_a;
-            const elem_t* vb = values + page_b + kv_head_values + slot_b;
+            // Interior step: one page lookup per half for the whole wavefront (scalar); every piece is then the
+            // half's base, the same for all lanes, plus the thread's constant offset.
 #pragma unroll
-            for (int j = 0; j < KPT; ++j) r.k[j] = *reinterpret_cast<const bf16x8*>((k_second[j] ? kb : ka) + k_off[j]);
+            for (int h = 0; h < 2; ++h) {
+                const int key = kt + 16 * h;
+                const int block = (int)__umulhi((unsigned)key, g.page_magic), slot = key - block * ps;
+                const size_t page = (size_t)__builtin_amdgcn_readlane(pages_cur, block - 64 * chunk) * page_elems;
+                const char* kbase = reinterpret_cast<const char*>(keys + page + kv_head_keys + (size_t)slot * D);
+                const char* vbase = reinterpret_cast<const char*>(values + page + kv_head_values + slot);
 #pragma unroll
-            for (int j = 0; j < VPT; ++j) r.v[j] = *reinterpret_cast<const bf16x4*>((v_second[j] ? vb : va) + v_off[j]);
+                for (int j = 0; j < KPH; ++j) r.k[h][j] = *reinterpret_cast<const bf16x8*>(kbase + k_off[j]);
+#pragma unroll
+                for (int j = 0; j < VPH; ++j) r.v[h][j] = *reinterpret_cast<const bf16x4*>(vbase + v_off[j]);
+            }
             return;
         }
         const int lo = max(k_begin, kt), hi = min(k_end, kt + 32) - 1;
 #pragma unroll
-        for (int j = 0; j < KPT; ++j) {
-            const int p = min(tid + 256 * j, K_PIECES - 1);
-            int slot;
-            const int key = min(max(kt + p / (D / 8), lo), hi);
-            const size_t page = locate(key, slot);
-            r.k[j] = *reinterpret_cast<const bf16x8*>(keys + page + kv_head_keys + (size_t)slot * D + 8 * (p % (D / 8)));
-        }
+        for (int h = 0; h < 2; ++h) {
 #pragma unroll
-        for (int j = 0; j < VPT; ++j) {
-            const int p = min(tid + 256 * j, V_PIECES - 1);
-            int slot;
-            const int key0 = min(max(kt + 4 * (p & 7), lo & ~3), hi & ~3);
-            const size_t page = locate(key0, slot);
-            r.v[j] = *reinterpret_cast<const bf16x4*>(values + page + kv_head_values + (size_t)(p >> 3) * ps + slot);
+            for (int j = 0; j < KPH; ++j) {
+                const int q = min(tid + 256 * j, K_HALF_PIECES - 1);
+                int slot;
+                const int key = min(max(kt + 16 * h + q / (D / 8), lo), hi);
+                const size_t page = locate(key, slot);
+                r.k[h][j] = *reinterpret_cast<const bf16x8*>(keys + page + kv_head_keys + (size_t)slot * D + 8 * (q % (D / 8)));
+            }
+#pragma unroll
+            for (int j = 0; j < VPH; ++j) {
+                const int q = min(tid + 256 * j, V_HALF_PIECES - 1);
+                int slot;
+                const int key0 = min(max(kt + 16 * h + 4 * (q & 3), lo & ~3), hi & ~3);
+                const size_t page = locate(key0, slot);
+                r.v[h][j] = *reinterpret_cast<const bf16x4*>(values + page + kv_head_values + (size_t)(q >> 2) * ps + slot);
+            }
         }
     };
     auto store_lds = [&](int buf, Staged& r, int kt) {
         unsigned char* kl = lds[buf];
         unsigned char* vl = lds[buf] + K_TILE_BYTES;
-#pragma unroll
-        for (int j = 0; j < KPT; ++j) {
-            const int p = tid + 256 * j;
-            if (p < K_PIECES) *reinterpret_cast<bf16x8*>(kl + (p / (D / 8)) * K_ROW + 16 * (p % (D / 8))) = r.k[j];
-        }
         const bool edge = kt < k_begin || kt + 32 > k_end;
 #pragma unroll
-        for (int j = 0; j < VPT; ++j) {
-            const int p = tid + 256 * j;
-            bf16x4 piece = r.v[j];
-            if (edge) {                           // keys outside the range may hold anything: keep them out of the sums
+        for (int h = 0; h < 2; ++h) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int kpos = kt + 4 * (p & 7) + r;
-                    if (kpos < k_begin || kpos >= k_end) piece[r] = (bf16_t)0.f;
-                }
+            for (int j = 0; j < KPH; ++j) {
+                const int q = tid + 256 * j;
+                if (q < K_HALF_PIECES) *reinterpret_cast<bf16x8*>(kl + (16 * h + q / (D / 8)) * K_ROW + 16 * (q % (D / 8))) = r.k[h][j];
             }
-            if (p < V_PIECES) *reinterpret_cast<bf16x4*>(vl + (p >> 3) * V_ROW + 8 * (p & 7)) = piece;
+#pragma unroll
+            for (int j = 0; j < VPH; ++j) {
+                const int q = tid + 256 * j;
+                bf16x4 piece = r.v[h][j];
+                if (edge) {                       // keys outside the range may hold anything: keep them out of the sums
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int kpos = kt + 16 * h + 4 * (q & 3) + e;
+                        if (kpos < k_begin || kpos >= k_end) piece[e] = (bf16_t)0.f;
+                    }
+                }
+                if (q < V_HALF_PIECES) *reinterpret_cast<bf16x4*>(vl + (q >> 2) * V_ROW + 8 * (4 * h + (q & 3))) = piece;
+            }
         }
     };
-    auto compute = [&](int buf, int kt) {
-        if (kt >= wave_hi || kt + 32 <= wave_lo) return;          // nothing for this wavefront's pairs in this step
+    // Scores stay as the products left them; the scale (in units of ln 2, so that the exponential is one
+    // instruction) goes into the multiply-add that also subtracts the running maximum.  FULL: every key of
+    // the step is seen by every pair of the wavefront, nothing is masked.
+    auto compute_step = [&](auto full_tag, int buf, int kt) {
+        constexpr bool FULL = decltype(full_tag)::value;
         const unsigned char* kl = lds[buf];
         const unsigned char* vl = lds[buf] + K_TILE_BYTES;
-        // Steps every valid pair sees completely need no mask.
-        const bool full = kt >= k_begin && kt + 32 <= k_end && kt + 31 <= q_pos_min && wave_tokens == g.tokens_per_tile &&
-                          (g.window <= 0 || kt > first_pos + q0 + wave_tokens - 1 - g.window);
-        float sv[8];
-        float tile_max = NEG_INF;
+        float sv[SUB][8];
+        float tile_max[SUB];
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) tile_max[u] = NEG_INF;
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
-            f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+            f32x4 s4[SUB];
+#pragma unroll
+            for (int u = 0; u < SUB; ++u) s4[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 bf16x8 kf = {0, 0, 0, 0, 0, 0, 0, 0};
                 if (32 * s + 32 <= D || quad < 2) kf = *reinterpret_cast<const bf16x8*>(kl + (16 * t2 + col) * K_ROW + 64 * s + 16 * quad);
-                s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], s4, 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < SUB; ++u) s4[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u][s], s4[u], 0, 0, 0);
             }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float v = s4[r] * scale_log2;          // scores in units of ln 2: exp2 below is one instruction
-                if (!full) {
-                    const int kpos = kt + 16 * t2 + 4 * quad + r;
-                    const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
-                    v = seen ? v : NEG_INF;
-                } else if (!pair_valid) {
-                    v = NEG_INF;
+            for (int u = 0; u < SUB; ++u)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float v = s4[u][r];
+                    if (!FULL) {
+                        const int kpos = kt + 16 * t2 + 4 * quad + r;
+                        const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos[u] && (g.window <= 0 || kpos > q_pos[u] - g.window);
+                        v = seen ? v : NEG_INF;
+                    }
+                    sv[u][4 * t2 + r] = v;
+                    tile_max[u] = fmaxf(tile_max[u], v);
                 }
-                sv[4 * t2 + r] = v;
-                tile_max = fmaxf(tile_max, v);
-            }
         }
         // The running maximum of a pair only moves when some key of this step beats it, which
         // soon becomes rare: then the exchange between the lanes of a pair and the rescaling of
         // the accumulators are skipped (the result is the same, the maximum being unchanged).
-        if (__any(tile_max > run_max)) {
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-            const float new_max = fmaxf(run_max, tile_max);
-            const float alpha = __builtin_amdgcn_exp2f(run_max - (new_max == NEG_INF ? 0.f : new_max));
-            run_max = new_max;
-            run_sum *= alpha;
+        bf16x8 pf[SUB];
 #pragma unroll
-            for (int c = 0; c < ND; ++c) acc[c] *= alpha;
-        }
-        const float use_max = run_max == NEG_INF ? 0.f : run_max;
-        bf16x8 pf;
+        for (int u = 0; u < SUB; ++u) {
+            if (__any(tile_max[u] > run_max[u])) {
+                float top = fmaxf(tile_max[u], __shfl_xor(tile_max[u], 16, 64));
+                top = fmaxf(top, __shfl_xor(top, 32, 64));
+                const float new_max = fmaxf(run_max[u], top);
+                const float alpha = __builtin_amdgcn_exp2f((run_max[u] - (new_max == NEG_INF ? 0.f : new_max)) * scale_log2);
+                run_max[u] = new_max;
+                run_sum[u] *= alpha;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float p = __builtin_amdgcn_exp2f(sv[e] - use_max);
-            run_sum += p;
-            pf[e] = (bf16_t)p;
+                for (int c = 0; c < ND; ++c) acc[u][c] *= alpha;
+            }
+            const float shift = run_max[u] == NEG_INF ? 0.f : -run_max[u] * scale_log2;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[u][e], scale_log2, shift));
+                run_sum[u] += p;
+                pf[u][e] = (bf16_t)p;
+            }
         }
 #pragma unroll
         for (int c = 0; c < ND; ++c) {
@@ -688,8 +720,18 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES) void paged_attention_tile_
                 vf[r] = lo4[r];
                 vf[4 + r] = hi4[r];
             }
-            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[c], 0, 0, 0);
+#pragma unroll
+            for (int u = 0; u < SUB; ++u) acc[u][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], acc[u][c], 0, 0, 0);
         }
+    };
+    auto compute = [&](int buf, int kt) {
+        if (kt >= wave_hi || kt + 32 <= wave_lo) return;          // nothing for this wavefront's pairs in this step
+        // Steps every pair of the wavefront sees completely need no mask.
+        const bool full = kt >= k_begin && kt + 32 <= k_end && kt + 31 <= q_pos_min && wave_tokens == SUB * g.tokens_per_tile &&
+                          g.gheads * g.tokens_per_tile == 16 && (gtile + 1) * g.gheads <= g.group &&
+                          (g.window <= 0 || kt > first_pos + q0 + wave_tokens - 1 - g.window);
+        if (full) compute_step(FullStep{}, buf, kt);
+        else compute_step(MaskedStep{}, buf, kt);
     };
 
     if (k_begin < k_end) {
@@ -718,17 +760,21 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES) void paged_attention_tile_
             kt += 64;
         }
     }
-    run_sum += __shfl_xor(run_sum, 16, 64);
-    run_sum += __shfl_xor(run_sum, 32, 64);
-    if (!pair_valid) return;
-    const float inv = run_sum > 0.f ? 1.f / run_sum : 0.f;
-    elem_t* o = out + ((size_t)(token0 + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
-    for (int c = 0; c < ND; ++c) {
-        bf16x4 r4;
+    for (int u = 0; u < SUB; ++u) {
+        float total = run_sum[u];
+        total += __shfl_xor(total, 16, 64);
+        total += __shfl_xor(total, 32, 64);
+        if (!pair_valid[u]) continue;
+        const float inv = total > 0.f ? 1.f / total : 0.f;
+        elem_t* o = out + ((size_t)(row_start[row] + q0 + u * g.tokens_per_tile + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) r4[r] = (bf16_t)(acc[c][r] * inv);
-        *reinterpret_cast<bf16x4*>(o + 16 * c) = r4;
+        for (int c = 0; c < ND; ++c) {
+            bf16x4 r4;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) r4[r] = (bf16_t)(acc[u][c][r] * inv);
+            *reinterpret_cast<bf16x4*>(o + 16 * c) = r4;
+        }
     }
 }
 #endif  // LSA_BF16
@@ -785,7 +831,8 @@ LSA_EXPORT int lsa_paged_attention(
     const int* row_start, const int* row_len, const int* row_ctx, const void* items, const int* item_slot, int n_items,
     const void* merges, int n_merges, float* part_acc, float* part_ml, const void* tiles, int n_tiles, float scale, int window,
     int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
-    int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, hipStream_t stream) {
+    int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, int tiles_per_workgroup,
+    hipStream_t stream) {
     if (n_items <= 0 && n_tiles <= 0) return 0;
     // decode_fusion (see DecodeFusion::mode): the caller promises that every row of the step brings one token.
     DecodeFusion fusion = {q_weight, k_weight, cos_sin, norm_eps, decode_fusion};
@@ -797,10 +844,17 @@ LSA_EXPORT int lsa_paged_attention(
     g.page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     if (n_tiles > 0) {
 #if LSA_BF16
+        // The plan's entries of `tiles` span what a workgroup takes: 4 or 8 tiles.
+        if (tiles_per_workgroup != 4 && tiles_per_workgroup != 4 * MAX_SUB) return -1;
         dim3 tgrid(n_tiles * n_kv * gtiles);
-        paged_attention_tile_kernel<<<tgrid, 256, 0, stream>>>(
-            (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
-            row_start, row_len, row_ctx, (const Item*)tiles, g);
+        if (tiles_per_workgroup == 4)
+            paged_attention_tile_kernel<1><<<tgrid, 256, 0, stream>>>(
+                (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
+                row_start, row_len, row_ctx, (const Item*)tiles, g);
+        else
+            paged_attention_tile_kernel<MAX_SUB><<<tgrid, 256, 0, stream>>>(
+                (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
+                row_start, row_len, row_ctx, (const Item*)tiles, g);
         const int terr = (int)hipGetLastError();
         if (terr) return terr;
 #else
@@ -819,5 +873,14 @@ LSA_EXPORT int lsa_paged_attention(
     LSA_LAUNCH_CHECK();
 }
 
+// Most tiles of 16 pairs that one workgroup of the prompt-portion kernel takes (it also takes 4; 0: no such
+// kernel for this type).
+LSA_EXPORT int lsa_attention_workgroup_tiles() {
+#if LSA_BF16
+    return 4 * MAX_SUB;
+#else
+    return 0;
+#endif
+}
 LSA_EXPORT int lsa_attention_head_dim() { return D; }
 LSA_EXPORT int lsa_attention_is_bf16() { return LSA_BF16; }

@@ -262,6 +262,11 @@ class HipOps:
             self._attention[key] = library.load(build.attention_module(dtype == torch.bfloat16, head_dim))
         return self._attention[key]
 
+    def attention_workgroup_tiles(self, dtype, head_dim) -> int:
+        """Tiles of 16 (token, head) pairs that a workgroup of the prompt-portion attention kernel takes together
+        (what an entry of a plan's ``tiles`` must span), or 0 if this type has no such kernel."""
+        return int(self._attention_library(dtype, head_dim).lsa_attention_workgroup_tiles())
+
     @staticmethod
     def decode_fusion_fits(dtype, head_dim) -> bool:
         """Whether the attention kernel can take the q/k norm, the rotation and the new token's way into the cache
@@ -330,7 +335,7 @@ class HipOps:
             _ptr(row_len), _ptr(row_ctx), _ptr(plan["items"]), _ptr(plan["item_slot"]), n_items, _ptr(plan["merges"]),
             n_merges, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), n_tiles, float(scale), int(window) if window else 0,
             page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, fusion_mode, _ptr(q_weight), _ptr(k_weight), float(norm_eps),
-            _ptr(cos_sin), _stream()), "paged_attention")
+            _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), _stream()), "paged_attention")
 
     def sample(self, logits, temperature, uniform, out):
         n, vocab = logits.shape

@@ -47,13 +47,15 @@ class AttentionPlan:
     key, one past the last key.  ``item_slot [n_items] int32``: index of the partial-result slot,
     or -1 if the item covers all keys of its rows and writes the output itself.
     ``merges [n_merges, 4] int32``: row, first token of the tile, first slot, number of slots.
-    ``tiles [n_tiles, 4] int32``: row, first token, first key, one past the last key of four
-    consecutive tiles that one workgroup handles together, sharing the keys it loads.
+    ``tiles [n_tiles, 4] int32``: row, first token, first key, one past the last key of
+    ``tiles_per_workgroup`` (4 or 8) consecutive tiles that one workgroup handles together, sharing
+    the keys it loads.
     """
 
-    def __init__(self, items, item_slot, merges, n_slots, tiles=None):
+    def __init__(self, items, item_slot, merges, n_slots, tiles=None, tiles_per_workgroup=0):
         self.items, self.item_slot, self.merges, self.n_slots = items, item_slot, merges, n_slots
         self.tiles = tiles if tiles is not None else np.zeros((0, 4), dtype=np.int32)
+        self.tiles_per_workgroup = tiles_per_workgroup
 
 
 def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: int, target_waves: int = TARGET_WAVES) -> int:
@@ -65,18 +67,45 @@ def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: i
     return max(1, min(MAX_SPLITS, target_waves // waves, max_keys // MIN_KEYS_PER_SPLIT))
 
 
-WORKGROUP_TILES = 4     # tiles a workgroup of the prompt-portion kernel handles together
-MIN_TILES_FOR_WORKGROUPS = 16
+MIN_TILES_FOR_WORKGROUPS = 16      # rows with at least this many tiles go to the prompt-portion kernel
+
+
+def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, heads, window, most: int) -> int:
+    """4 or ``most`` tiles per workgroup of the prompt-portion kernel, whichever the step's rows finish sooner with.
+
+    A workgroup walks its keys in steps of 32.  With all compute units busy, eight tiles per workgroup get more out of
+    every step (measured on Qwen3-8B shapes: 2.9 ns a step against 2 x 2.13 ns for the same tokens in two workgroups
+    of four; setting up and draining a workgroup costs about 8 steps more), but a step of theirs takes longer
+    (1.68 against 1.5 us), and the workgroup with the most steps bounds the launch from below: one short prompt
+    finishes sooner with four, long rows and many rows with eight."""
+    if most <= 4:
+        return most
+    def estimate(per_workgroup, ns_per_step, us_per_step_alone):
+        span = per_workgroup * tokens_per_tile
+        total = longest = 0
+        for row in range(len(row_len)):
+            if tiles_per_row[row] < MIN_TILES_FOR_WORKGROUPS:
+                continue
+            n, first_pos = int(row_len[row]), int(row_ctx[row]) - int(row_len[row])
+            starts = np.arange(0, n, span)
+            k_end = first_pos + np.minimum(starts + span, n)
+            k_begin = np.zeros_like(starts) if window is None else np.maximum(0, first_pos + starts - window + 1)
+            steps = -(-(k_end - k_begin) // 32)
+            total += int(steps.sum()) + 8 * len(steps)
+            longest = max(longest, int(steps.max()))
+        return max(total * heads * ns_per_step * 1e-3, longest * us_per_step_alone)
+    return most if estimate(most, 2.9, 1.68) < estimate(4, 2.13, 1.5) else 4
 
 
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
-                         workgroup_tiles: bool = False) -> AttentionPlan:
+                         workgroup_tiles: int = 0) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
-    arrays have the same shape whatever the contexts are.  With ``workgroup_tiles`` rows with many
-    tiles (portions of prompts) go to the kernel in which four tiles share the keys they load."""
+    arrays have the same shape whatever the contexts are.  With ``workgroup_tiles`` (the number of tiles a
+    workgroup of that kernel takes, which the kernel library tells) rows with many tiles (portions of prompts) go
+    to the kernel in which the tiles of a workgroup share the keys they load."""
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
@@ -84,11 +113,13 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
     items, slots, merges, tiles = [], [], [], []
     n_slots = 0
+    per_workgroup = _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window,
+                                              int(workgroup_tiles)) if workgroup_tiles and fixed_splits is None else 0
     for row in range(len(row_len)):
         n, ctx = int(row_len[row]), int(row_ctx[row])
         first_pos = ctx - n
-        if workgroup_tiles and fixed_splits is None and tiles_per_row[row] >= MIN_TILES_FOR_WORKGROUPS:
-            span = WORKGROUP_TILES * tokens_per_tile
+        if per_workgroup and tiles_per_row[row] >= MIN_TILES_FOR_WORKGROUPS:
+            span = per_workgroup * tokens_per_tile
             for q0 in range(0, n, span):
                 k_begin = 0 if window is None else max(0, first_pos + q0 - window + 1)
                 tiles.append((row, q0, k_begin, first_pos + min(q0 + span, n)))
@@ -125,7 +156,7 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     merges = np.asarray(merges, dtype=np.int32).reshape(-1, 4)
     tiles.sort(key=lambda tile: tile[2] - tile[3])       # most keys first: the long tiles must not start last
     tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 4)
-    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, tiles)
+    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, tiles, per_workgroup)
 
 
 class GQAttention(Mixer):
@@ -185,12 +216,14 @@ class GQAttention(Mixer):
         if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
             fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys)
         import torch
+        per_workgroup = getattr(ctx.ops, "attention_workgroup_tiles", None)
+        per_workgroup = per_workgroup(ctx.dtype, self.head_dim) if per_workgroup is not None else 0
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
-                                    fixed_splits=fixed, workgroup_tiles=ctx.dtype == torch.bfloat16)
+                                    fixed_splits=fixed, workgroup_tiles=per_workgroup)
         ctx.set_plan(key, {
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
             "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),
-            "n_slots": plan.n_slots,
+            "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup,
         })
 
     def forward(self, x, ctx, cache, sink=None):

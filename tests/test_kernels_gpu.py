@@ -164,13 +164,22 @@ def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, need
         keys[pages, :, (place % page).to(DEV), :] = k.to(dtype)
         values[pages, :, :, (place % page).to(DEV)] = v.to(dtype)
         table[r, :first] = -1                                                     # pages a window has passed are gone
-    if workgroup_tiles is None:
-        workgroup_tiles = dtype == torch.bfloat16
-    plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, workgroup_tiles=workgroup_tiles,
-                                **({} if target_waves is None else {"target_waves": target_waves}))
+    # workgroup_tiles: None lets the plan choose between the tile counts the kernel offers, 0 keeps every row out of the
+    # prompt-portion kernel, 4 or 8 fixes the count.
+    from llmserver_amd.parts import attention as attention_module
+    most = ops.attention_workgroup_tiles(dtype, d) if workgroup_tiles is None or workgroup_tiles else 0
+    chooser = attention_module._workgroup_tiles_that_pay
+    if workgroup_tiles:
+        assert workgroup_tiles <= most
+        attention_module._workgroup_tiles_that_pay = lambda *args, **kwargs: workgroup_tiles
+    try:
+        plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, workgroup_tiles=most,
+                                    **({} if target_waves is None else {"target_waves": target_waves}))
+    finally:
+        attention_module._workgroup_tiles_that_pay = chooser
     staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
               "merges": torch.from_numpy(plan.merges).to(DEV), "tiles": torch.from_numpy(plan.tiles).to(DEV), "n_tiles": len(plan.tiles),
-              "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots}
+              "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup}
     t = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
     got = torch.zeros(tokens, n_q * d, device=DEV, dtype=dtype)
     ref = torch.zeros_like(got)
@@ -301,13 +310,19 @@ def test_attention_window_edge(ops, dtype, window):
 @pytest.mark.parametrize("window", [None, 40])
 def test_attention_prompt_portions_in_workgroup_tiles(ops, n_q, n_kv, d, page, window):
     """Long portions of prompts, with and without a prefix, beside decoded tokens: the portions go
-    through the kernel whose four wavefronts share the keys they load (bfloat16)."""
+    through the kernel whose four wavefronts share the keys they load (bfloat16), with one tile of 16 pairs per
+    wavefront and with two."""
     print(f"attention workgroup tiles {n_q}/{n_kv} d{d} page{page} window {window}", flush=True)
     lens = [333, 1, 200, 97, 1]
     ctxs = [333, 90, 777, 130, 400]
     plan, _ = attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d)
     assert len(plan.tiles) > 0 and len(plan.items) > 0
-    attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d, workgroup_tiles=False)
+    attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d, workgroup_tiles=0)
+    for per_workgroup in (4, 8):                                   # one and two tiles per wavefront
+        if per_workgroup <= ops.attention_workgroup_tiles(torch.bfloat16, d):
+            plan, _ = attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d,
+                                     workgroup_tiles=per_workgroup)
+            assert plan.tiles_per_workgroup == per_workgroup and len(plan.tiles) > 0
 
 
 def test_attention_refuses_sizes_it_cannot_take(ops):
