@@ -189,7 +189,7 @@ def main() -> int:
     step_bytes = weight_bytes(config, elem) + args.batch * mean_context * kv_bytes_per_token(config, elem)
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
     result = {
-        "metric": "decode tok/s at batch 8, context 4096 (Qwen3-8B-sized, random weights)", "value": round(value, 2),
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen3-8B-sized, random weights)", "value": round(value, 2),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short, "data": "synthetic",
         "config": {"model": "qwen3-8b-sized", "layers": config.num_hidden_layers, "layers_full": FULL_LAYERS,

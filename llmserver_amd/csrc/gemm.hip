@@ -9,7 +9,7 @@
 //                                            B = X^T      (lane: row 16 t + col of X, same k)
 //   result lane holds Y^T[n0 + 4 quad + r][16 t + col].
 //
-// Around the product, for up to 8 rows, two things can be fused that would otherwise be kernels
+// Around the product, for up to 16 rows, two things can be fused that would otherwise be kernels
 // of their own between two products (each costs a launch and a trip of the rows through memory):
 //   * Row scale.  X = s * w for a residual stream s and a norm's weights w, and the result wanted
 //     is rmsnorm(s) * w . W^T = (X . W^T) / rms(s).  The kernel is given partial sums of s^2
@@ -17,8 +17,8 @@
 //     rsqrt(sum / K + eps) in the epilogue.
 //   * Stream update.  The result is an update of a residual stream that a norm follows.  The
 //     epilogue then forms s' = round(resid + round(y)), and writes s', round(s' * norm_weight) and
-//     the sums of s'^2 over the columns of each of its tiles ([M, P]): exactly what the row scale of
-//     the next product takes.
+//     the sum of s'^2 over the columns of each workgroup ([M, P]): exactly what the row scale of the
+//     next product takes.
 #include "common.hpp"
 
 using namespace lsa;
@@ -27,8 +27,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int GEMM_WAVES = 8;
-constexpr int FUSED_ROWS = 8;            // most rows the fused epilogues take (one wavefront per row finds its scale)
-constexpr int SCALE_PARTS = 512;         // most partial sums per row the row scale takes
+constexpr int FUSED_ROWS = 16;           // most rows the fused epilogues take (each of the 8 wavefronts finds the scale of two rows)
+constexpr int SCALE_PARTS = 512;         // most partial sums per row the row scale takes (half as many from 9 rows on)
 
 struct Fusion {
     // Row scale (null: none).
@@ -47,29 +47,41 @@ struct Fusion {
 // (they come from cache and are there by the time those have arrived) and while few registers
 // are in use; the loads are issued whether or not a scale was asked for, from a harmless address
 // if not, so that no branch stands between the loads of the product and the waits for them.
+// Wavefront `wave` finds the scale of row `wave` from up to 512 partial sums, or, from 9 rows on, the
+// scales of rows `wave` and `wave + 8` from up to 256 each: eight loads per lane either way.
 struct RowScaleLoads {
     float part[SCALE_PARTS / 64];
 };
+__device__ inline int row_scale_row(int M, int wave, int i) { return M <= GEMM_WAVES ? wave : wave + GEMM_WAVES * (i >> 2); }
+__device__ inline int row_scale_part(int M, int lane, int i) { return M <= GEMM_WAVES ? lane + 64 * i : lane + 64 * (i & 3); }
 __device__ inline void row_scale_issue(RowScaleLoads& loads, const Fusion& f, const void* harmless, int M, int wave, int lane) {
-    const bool wanted = f.square_sums && wave < M;
-    const float* src = wanted ? f.square_sums + (size_t)wave * f.n_parts : (const float*)harmless;
-    const int last = wanted ? f.n_parts - 1 : 0;
 #pragma unroll
-    for (int i = 0; i < SCALE_PARTS / 64; ++i) loads.part[i] = src[min(lane + 64 * i, last)];
+    for (int i = 0; i < SCALE_PARTS / 64; ++i) {
+        const int row = row_scale_row(M, wave, i);
+        const bool wanted = f.square_sums && row < M;
+        const float* src = wanted ? f.square_sums + (size_t)row * f.n_parts : (const float*)harmless;
+        loads.part[i] = src[wanted ? min(row_scale_part(M, lane, i), f.n_parts - 1) : 0];
+    }
 }
-// 1 / rms of row `wave` into scale[wave].
+// 1 / rms of the wavefront's row or rows into scale[row].
 __device__ inline void row_scale_finish(const RowScaleLoads& loads, const Fusion& f, int M, int K, int wave, int lane, float* scale) {
-    if (!f.square_sums || wave >= M) return;
-    float sum = 0.f;
+    if (!f.square_sums) return;
+    float sum[2] = {0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < SCALE_PARTS / 64; ++i) sum += lane + 64 * i < f.n_parts ? loads.part[i] : 0.f;
-    sum = wave_sum(sum);
-    if (lane == 0) scale[wave] = rsqrtf(sum / (float)K + f.eps);
+    for (int i = 0; i < SCALE_PARTS / 64; ++i)
+        sum[M <= GEMM_WAVES ? 0 : i >> 2] += row_scale_part(M, lane, i) < f.n_parts ? loads.part[i] : 0.f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int row = wave + GEMM_WAVES * h;
+        if (row >= M || (h && M <= GEMM_WAVES)) continue;
+        const float total = wave_sum(sum[h]);
+        if (lane == 0) scale[row] = rsqrtf(total / (float)K + f.eps);
+    }
 }
 
 // Epilogue of the stream update for one element (m, n) of the result; the 16 lanes that hold
 // the 16 columns of a tile for one m are neighbours, so the sum of squares is four shuffles.
-__device__ inline void stream_update(const Fusion& f, float total, int m, int n, int M, int N, bool own, int tile_index, int tiles) {
+__device__ inline float stream_update(const Fusion& f, float total, int m, int n, int M, int N, bool own) {
     const bool inside = own && m < M && n < N;
     float s = 0.f;
     if (inside) {
@@ -84,7 +96,7 @@ __device__ inline void stream_update(const Fusion& f, float total, int m, int n,
     sq += __shfl_xor(sq, 2, 64);
     sq += __shfl_xor(sq, 4, 64);
     sq += __shfl_xor(sq, 8, 64);
-    if ((threadIdx.x & 15) == 0 && m < M && tile_index < tiles) f.square_sums_out[(size_t)m * tiles + tile_index] = sq;
+    return sq;                              // the tile's sum for row m, in all 16 lanes that hold the row
 }
 
 // One tile of W per workgroup.  GATED: W stacks a gate matrix on an up matrix ([2I, K], gate first)
@@ -96,7 +108,7 @@ template <int MT, typename OutT, bool GATED, int CH>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                       OutT* __restrict__ y, int M, int N, int K, int R, Fusion fusion) {
     __shared__ float partial[GEMM_WAVES][MT][256];
-    __shared__ float row_scale[GEMM_WAVES];
+    __shared__ float row_scale[FUSED_ROWS];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, quad = lane >> 4;
     // R of the tile's 16 rows are this workgroup's own (GATED: 8 gate rows and 8 up rows); the other lanes
@@ -195,7 +207,8 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
             continue;
         }
         if (MT == 1 && sizeof(OutT) == 2 && fusion.resid) {
-            stream_update(fusion, total, m, n, M, N, j < R, blockIdx.x, gridDim.x);
+            const float sq = stream_update(fusion, total, m, n, M, N, j < R);
+            if (j == 0 && m < M) fusion.square_sums_out[(size_t)m * gridDim.x + blockIdx.x] = sq;
             continue;
         }
         if (m < M && j < R && n < N) y[(size_t)m * N + n] = (OutT)total;
@@ -211,7 +224,8 @@ template <typename OutT, bool GATED, int CH>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                            OutT* __restrict__ y, int M, int N, int K, int R, Fusion fusion) {
     __shared__ float partial[GEMM_WAVES][2][256];
-    __shared__ float row_scale[GEMM_WAVES];
+    __shared__ float row_scale[FUSED_ROWS];
+    __shared__ float second_tile_sums[16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, quad = lane >> 4;
     const int half = N / 2;                                        // GATED: rows of the gate matrix
@@ -310,7 +324,11 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_wide_kernel(const
     const int n = n0 + 16 * tile + j;
     const bool own = j < (tile ? own1 : own0);
     if (sizeof(OutT) == 2 && fusion.resid) {
-        stream_update(fusion, total, m, n, M, N, own, 2 * blockIdx.x + tile, 2 * gridDim.x);
+        // One sum of squares per row and workgroup: the second tile's go through LDS to the first tile's threads.
+        const float sq = stream_update(fusion, total, m, n, M, N, own);
+        if (tile && j == 0) second_tile_sums[m] = sq;
+        __syncthreads();
+        if (!tile && j == 0 && m < M) fusion.square_sums_out[(size_t)m * gridDim.x + blockIdx.x] = sq + second_tile_sums[m];
         return;
     }
     if (m < M && own && n < N) y[(size_t)m * N + n] = (OutT)total;
@@ -396,7 +414,7 @@ static void layout(int N, bool gated, int rows, int* workgroups, int* parts) {
     const long total = gated ? N / 2 : N;
     const int r = rows == -1 ? 8 : rows;
     *workgroups = (int)((total + r - 1) / r);
-    *parts = (!gated && rows > 16) ? 2 * *workgroups : *workgroups;
+    *parts = *workgroups;
 }
 
 template <typename OutT, bool GATED>
@@ -431,13 +449,13 @@ static int launch(const bf16_t* x, const bf16_t* w, OutT* y, int M, int N, int K
 static bool fusion_fits(int M, const float* square_sums, int n_parts, const void* resid) {
     if (!square_sums && !resid) return true;
     if (M > FUSED_ROWS) return false;
-    if (square_sums && (n_parts <= 0 || n_parts > SCALE_PARTS)) return false;
+    if (square_sums && (n_parts <= 0 || n_parts > (M <= GEMM_WAVES ? SCALE_PARTS : SCALE_PARTS / 2))) return false;
     return true;
 }
 
 // out_float32: 0 writes bfloat16, 1 writes float32.  rows: rows of W per workgroup, 1 to 32 (more than 16
 // only for M <= 16), or 0 to let the size decide.  square_sums [M, n_parts] (or null) asks for the row scale
-// rsqrt(sum / K + eps), M <= 8.  Refuses (returns -1) what it cannot take.
+// rsqrt(sum / K + eps), M <= 16.  Refuses (returns -1) what it cannot take.
 LSA_EXPORT int lsa_gemm_skinny(int out_float32, const void* x, const void* w, void* y, int M, int N, int K, int rows,
                                const float* square_sums, int n_parts, float eps, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -457,9 +475,9 @@ LSA_EXPORT int lsa_gemm_skinny_parts(int M, int N, int rows) {
     return parts;
 }
 
-// The product as an update of a residual stream that a norm follows (see the top of the file), M <= 8:
+// The product as an update of a residual stream that a norm follows (see the top of the file), M <= 16:
 //   resid_out = round(resid + round(x . w^T [/ rms, if square_sums])), weighted_out = round(resid_out * norm_weight),
-//   square_sums_out [M, lsa_gemm_skinny_parts(M, N, rows)] = sums of resid_out^2 over the columns of each tile.
+//   square_sums_out [M, lsa_gemm_skinny_parts(M, N, rows)] = sums of resid_out^2 over the columns of each workgroup.
 // resid_out may be resid itself.
 LSA_EXPORT int lsa_gemm_skinny_stream(const void* x, const void* w, int M, int N, int K, int rows,
                                       const float* square_sums, int n_parts, float eps,

@@ -15,7 +15,8 @@ from ..parts.attention import group_tiling
 from . import build, library
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
-SKINNY_GEMM_ROWS = 8        # up to this many rows the hand-written weight-streaming product beats the library (measured)
+SKINNY_GEMM_ROWS = 16       # up to this many rows the hand-written weight-streaming products, with the sums, norms and the
+                            # activation between them folded in, beat the library's products plus those kernels (measured)
 
 
 def _code(tensor: torch.Tensor) -> int:
@@ -82,8 +83,8 @@ class HipOps:
         library.preload(self.required_modules(head_dims, dtype))
 
     # -- matrix products -------------------------------------------------------------------
-    FUSED_ROWS = 8          # most rows the few-row product's fused epilogues take
-    SCALE_PARTS = 512       # most partial sums per row its row scale takes
+    FUSED_ROWS = 16         # most rows the few-row product's fused epilogues take
+    SCALE_PARTS = 512       # most partial sums per row its row scale takes (half as many from 9 rows on)
 
     def _few_rows(self, x, weight):
         rows, width = x.shape
@@ -101,7 +102,8 @@ class HipOps:
         return _ptr(square_sums), square_sums.shape[1], float(eps)
 
     def _row_scale_fits(self, row_scale, rows):
-        return row_scale is None or (rows <= self.FUSED_ROWS and 0 < row_scale[0].shape[1] <= self.SCALE_PARTS)
+        most = self.SCALE_PARTS if rows <= 8 else self.SCALE_PARTS // 2
+        return row_scale is None or (rows <= self.FUSED_ROWS and 0 < row_scale[0].shape[1] <= most)
 
     def row_scale_fits(self, x, weight, row_scale) -> bool:
         """Whether the few-row products take ``x`` with this ``row_scale`` (then they do not return None for it)."""
@@ -124,7 +126,7 @@ class HipOps:
 
         ``row_scale = (square_sums [T, P], eps)``: ``x`` is a residual stream already multiplied by a norm's
         weights, ``square_sums`` are partial sums of the stream's squares, and the result rows are divided by the
-        stream's root mean square, so that the result is the product of the normalised stream (up to 8 rows)."""
+        stream's root mean square, so that the result is the product of the normalised stream (up to 16 rows)."""
         rows, width = x.shape
         if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or not self._row_scale_fits(row_scale, rows) \
                 or (rows_per_workgroup > 16 and rows > 16):
@@ -144,7 +146,7 @@ class HipOps:
         ``norm_weight`` follows, in one launch: returns ``(stream, weighted, square_sums)`` with
         ``stream = resid + x @ weight^T`` (a new tensor), ``weighted = stream * norm_weight`` and
         ``square_sums [T, P]`` partial sums of ``stream^2`` (one per tile of the kernel's workgroups), which is what
-        ``row_scale`` of the next product takes.  None if this is no case for it (more than 8 rows, other types)."""
+        ``row_scale`` of the next product takes.  None if this is no case for it (more than 16 rows, other types)."""
         rows, width = x.shape
         n = weight.shape[0]
         if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or rows > self.FUSED_ROWS \

@@ -403,7 +403,7 @@ def test_skinny_gemm(ops, rows, n, k):
             raise RuntimeError("refused")
 
 
-@pytest.mark.parametrize("rows", [1, 5, 8])
+@pytest.mark.parametrize("rows", [1, 5, 8, 9, 16])
 @pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (6144, 1000), (200, 5120), (8192, 64)])
 def test_skinny_gemm_with_row_scale_and_stream_update(ops, rows, n, k):
     """The few-row product with a norm folded in on either side, against the separate kernels' twins:
@@ -448,14 +448,14 @@ def test_skinny_gemm_with_row_scale_and_stream_update(ops, rows, n, k):
         torch.testing.assert_close(got_stream.float(), want_stream.float(), atol=4e-2, rtol=1e-2)
         assert float((got_stream.float() - want_stream.float()).abs().gt(0).float().mean()) < 0.02
         torch.testing.assert_close(got_weighted.float(), (got_stream.float() * next_weight).to(torch.bfloat16).float(), atol=0, rtol=0)
-        assert got_sums.shape[0] == rows and (per == 0 or got_sums.shape[1] == -(-n // per) * (2 if per > 16 else 1))
+        assert got_sums.shape[0] == rows and (per == 0 or got_sums.shape[1] == -(-n // per))
         torch.testing.assert_close(got_sums.sum(1), (got_stream.float() ** 2).sum(1), atol=1e-3, rtol=1e-5)
     # chained: the producer's outputs feed a consumer of width n
     w2 = (torch.randn(72, n, device=DEV) / n ** 0.5).to(torch.bfloat16)
     got_stream, got_weighted, got_sums = ops.linear_into_stream(weighted, w, resid, next_weight, row_scale=(square_sums, eps))
     if n % 8:
         assert ops.linear_few_rows(got_weighted, w2, row_scale=(got_sums, eps)) is None          # widths in steps of 8 only
-    elif got_sums.shape[1] <= ops.SCALE_PARTS:
+    elif got_sums.shape[1] <= (ops.SCALE_PARTS if rows <= 8 else ops.SCALE_PARTS // 2):
         chained = ops.linear_few_rows(got_weighted, w2, out_float32=True, row_scale=(got_sums, eps))
         normed = torch.empty_like(got_stream)
         TorchOps().add_rmsnorm(got_stream.clone(), None, next_weight, eps, normed)
@@ -463,12 +463,17 @@ def test_skinny_gemm_with_row_scale_and_stream_update(ops, rows, n, k):
     else:
         assert ops.linear_few_rows(got_weighted, w2, row_scale=(got_sums, eps)) is None
     # more rows than the fused epilogues take
-    nine = torch.zeros(9, k, device=DEV, dtype=torch.bfloat16)
-    assert ops.linear_into_stream(nine, w, torch.zeros(9, n, device=DEV, dtype=torch.bfloat16), next_weight) is None
-    assert ops.linear_few_rows(nine, w, row_scale=(torch.ones(9, 4, device=DEV), eps)) is None
+    many = torch.zeros(17, k, device=DEV, dtype=torch.bfloat16)
+    saved = ops.skinny_rows
+    try:
+        ops.skinny_rows = 64
+        assert ops.linear_into_stream(many, w, torch.zeros(17, n, device=DEV, dtype=torch.bfloat16), next_weight) is None
+        assert ops.linear_few_rows(many, w, row_scale=(torch.ones(17, 4, device=DEV), eps)) is None
+    finally:
+        ops.skinny_rows = saved
 
 
-@pytest.mark.parametrize("rows", [1, 5, 8])
+@pytest.mark.parametrize("rows", [1, 5, 8, 13, 16])
 @pytest.mark.parametrize("inter, k", [(8, 16), (104, 72), (12288, 4096), (1000, 1000), (264, 5120), (40, 1536), (72, 1792)])
 def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
     print(f"gated product rows {rows} inter {inter} k {k}", flush=True)
@@ -486,4 +491,4 @@ def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
         torch.testing.assert_close(got.float(), expected, atol=2e-2, rtol=2e-2)
         got = ops.linear_gated(x, w, pairs_per_workgroup=per, row_scale=(square_sums, 1e-6))
         torch.testing.assert_close(got.float(), scaled, atol=2e-2, rtol=2e-2)
-    assert ops.linear_gated(torch.zeros(9, k, device=DEV, dtype=torch.bfloat16), w) is None
+    assert ops.linear_gated(torch.zeros(17, k, device=DEV, dtype=torch.bfloat16), w) is None
