@@ -146,28 +146,69 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
 
 constexpr int VT_TOKENS = 64;
 
+// Values of long portions: a workgroup takes 64 consecutive tokens of one KV head through LDS, reads
+// them from the projection in 16-byte pieces and writes them transposed, four slots of one
+// dimension at a time (8 or 16 bytes) where four tokens are neighbours in one page, which is the
+// rule inside a portion; a page's [d][page_size] block is contiguous, so these stores coalesce.
 template <typename T>
 __global__ __launch_bounds__(256) void value_tiles_kernel(
     const T* __restrict__ qkv, T* __restrict__ values, const int* __restrict__ table, int table_stride,
     const int* __restrict__ token_row, const int* __restrict__ positions, int page_size, int n_q, int n_kv, int d, int n_tokens) {
-    extern __shared__ unsigned char tile_bytes[];          // [VT_TOKENS][d + 2] elements of T
+    constexpr int VEC = Elem<T>::kVec;
+    extern __shared__ unsigned char tile_bytes[];          // [VT_TOKENS][d + VEC] elements of T
+    __shared__ long group_base[VT_TOKENS / 4];             // element offset of the group's first slot in `values`, or -1
+    __shared__ unsigned char covered[VT_TOKENS];           // token goes out with its group
     T* tile = reinterpret_cast<T*>(tile_bytes);
     const int token0 = blockIdx.x * VT_TOKENS, kv_head = blockIdx.y;
-    const int pitch = d + 2;
+    const int pitch = d + VEC;
     const int width = (n_q + 2 * n_kv) * d;
-    for (int e = threadIdx.x; e < VT_TOKENS * d; e += 256) {       // rows of the projection: coalesced over the head's d values
-        const int t = e / d, i = e % d;
-        if (token0 + t < n_tokens) tile[t * pitch + i] = qkv[(size_t)(token0 + t) * width + (size_t)(n_q + n_kv + kv_head) * d + i];
+    const int pieces = d / VEC;
+    for (int e = threadIdx.x; e < VT_TOKENS * pieces; e += 256) {
+        const int t = e / pieces, part = e % pieces;
+        if (token0 + t < n_tokens)
+            store_vec16(tile + t * pitch + part * VEC,
+                        load_vec16(qkv + (size_t)(token0 + t) * width + (size_t)(n_q + n_kv + kv_head) * d + part * VEC));
+    }
+    // Four tokens go out together if they are one request's neighbours starting at a position that is a multiple
+    // of four; the groups are laid so that this holds when the tile lies inside one portion.
+    const int shift = (4 - (positions[min(token0, n_tokens - 1)] & 3)) & 3;
+    if (threadIdx.x < VT_TOKENS) covered[threadIdx.x] = 0;
+    __syncthreads();
+    if (threadIdx.x < VT_TOKENS / 4) {
+        const int local = shift + 4 * threadIdx.x, first = token0 + local;
+        long base = -1;
+        if (local + 3 < VT_TOKENS && first + 3 < n_tokens) {
+            const int row = token_row[first], pos = positions[first];
+            bool together = (pos & 3) == 0;
+            for (int r = 1; r < 4; ++r) together = together && token_row[first + r] == row && positions[first + r] == pos + r;
+            const int p = table[(size_t)row * table_stride + pos / page_size];
+            if (together && p >= 0) {
+                base = (((long)p * n_kv + kv_head) * d) * page_size + pos % page_size;
+                for (int r = 0; r < 4; ++r) covered[local + r] = 1;
+            }
+        }
+        group_base[threadIdx.x] = base;
     }
     __syncthreads();
-    const int t = threadIdx.x & (VT_TOKENS - 1);                   // this thread's token: neighbours write neighbouring slots
-    const int token = token0 + t;
-    if (token >= n_tokens) return;
-    const int pos = positions[token];
-    const int p = table[(size_t)token_row[token] * table_stride + pos / page_size];
-    if (p < 0) return;
-    T* dst = values + (((size_t)p * n_kv + kv_head) * d) * page_size + pos % page_size;
-    for (int i = threadIdx.x / VT_TOKENS; i < d; i += 256 / VT_TOKENS) dst[(size_t)i * page_size] = tile[t * pitch + i];
+    for (int e = threadIdx.x; e < (VT_TOKENS / 4) * d; e += 256) {
+        const int g = e & (VT_TOKENS / 4 - 1), i = e / (VT_TOKENS / 4);      // neighbouring threads: neighbouring groups of slots
+        const long base = group_base[g];
+        if (base < 0) continue;
+        T four[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) four[r] = tile[(shift + 4 * g + r) * pitch + i];
+        T* dst = values + base + (size_t)i * page_size;
+        if (sizeof(T) == 2) *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(four);
+        else *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(four);
+    }
+    for (int e = threadIdx.x; e < VT_TOKENS * d; e += 256) {                  // the tokens that are in no such group
+        const int t = e & (VT_TOKENS - 1), i = e / VT_TOKENS;
+        const int token = token0 + t;
+        if (covered[t] || token >= n_tokens) continue;
+        const int pos = positions[token];
+        const int p = table[(size_t)token_row[token] * table_stride + pos / page_size];
+        if (p >= 0) values[(((size_t)p * n_kv + kv_head) * d + i) * page_size + pos % page_size] = tile[t * pitch + i];
+    }
 }
 
 template <typename T>
@@ -188,7 +229,7 @@ static int launch(void* qkv, void* keys, void* values, const int* table, int tab
     int err = (int)hipGetLastError();
     if (err || !tiled_values) return err;
     dim3 vgrid((n_tokens + VT_TOKENS - 1) / VT_TOKENS, n_kv);
-    value_tiles_kernel<T><<<vgrid, 256, VT_TOKENS * (d + 2) * sizeof(T), stream>>>((const T*)qkv, (T*)values, table, table_stride,
+    value_tiles_kernel<T><<<vgrid, 256, VT_TOKENS * (d + Elem<T>::kVec) * sizeof(T), stream>>>((const T*)qkv, (T*)values, table, table_stride,
                                                                                   token_row, positions, page_size, n_q, n_kv, d, n_tokens);
     LSA_LAUNCH_CHECK();
 }

@@ -96,7 +96,8 @@ def make_cache(n_pages, n_kv, page, d, dtype):
 def test_qk_norm_rope_kv_write(ops, dtype, n_q, n_kv, d, page):
     print(f"qk_norm_rope_kv_write {dtype} {n_q}/{n_kv} d{d} page{page}", flush=True)
     torch.manual_seed(d + n_q)
-    lens, starts = ([5, 1, 23], [0, 700, 37]) if d != 128 else ([300, 1, 23], [401, 1, 37])    # portions and decoded tokens; a long portion
+    # portions and decoded tokens; with a long portion the values take the tiled path, at starts that are and are no multiple of four
+    lens, starts = ([5, 1, 23], [0, 700, 37]) if d not in (64, 128) else ([300, 1, 23], [401, 1, 37]) if d == 128 else ([130, 200, 2], [64, 7, 3])
     rows = len(lens)
     n_pages = 200 if page < 500 else 8
     width = max(-(-(s + n) // page) for s, n in zip(starts, lens))
