@@ -156,7 +156,7 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     merges = np.asarray(merges, dtype=np.int32).reshape(-1, 4)
     tiles.sort(key=lambda tile: tile[2] - tile[3])       # most keys first: the long tiles must not start last
     tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 4)
-    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, tiles, per_workgroup)
+    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, tiles, per_workgroup if len(tiles) else 0)
 
 
 class GQAttention(Mixer):

@@ -1,0 +1,106 @@
+"""The host-side work list of the attention kernels: every (token, head) pair of a step is some
+item's or some workgroup tile's, with exactly the keys it may see; split key ranges tile their
+range without gaps; captured steps get arrays whose shape does not depend on the contexts."""
+import random
+
+import numpy as np
+import pytest
+
+from llmserver_amd.parts.attention import (KEY_ALIGN, MAX_SPLITS, MIN_TILES_FOR_WORKGROUPS, build_attention_plan, fixed_split_count,
+                                           group_tiling)
+
+
+def covered_tokens(plan, row_len, row_ctx, group_size, window):
+    """(row, token) -> list of (k_begin, k_end) it is computed against, over items and workgroup tiles."""
+    _, tokens_per_tile, _ = group_tiling(group_size)
+    seen = {}
+    for (row, q0, k_begin, k_end) in plan.items.tolist():
+        for token in range(q0, min(q0 + tokens_per_tile, row_len[row])):
+            seen.setdefault((row, token), []).append((k_begin, k_end))
+    span = plan.tiles_per_workgroup * tokens_per_tile
+    for (row, q0, k_begin, k_end) in plan.tiles.tolist():
+        assert plan.tiles_per_workgroup in (4, 8)
+        for token in range(q0, min(q0 + span, row_len[row])):
+            seen.setdefault((row, token), []).append((k_begin, k_end))
+    return seen
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_every_token_meets_its_keys_exactly_once(seed):
+    rng = random.Random(seed)
+    group_size = rng.choice([1, 2, 4, 5, 8, 16, 20])
+    n_kv = rng.choice([1, 2, 8])
+    window = rng.choice([None, None, 40, 700])
+    rows = rng.randint(1, 9)
+    row_len = [rng.choice([1, 1, 1, 2, 7, 33, 200, 900]) for _ in range(rows)]
+    row_ctx = [n + rng.choice([0, 0, 5, 64, 1000, 5000]) for n in row_len]
+    most = rng.choice([0, 4, 8])
+    plan = build_attention_plan(row_len, row_ctx, group_size, n_kv, window, workgroup_tiles=most)
+    _, tokens_per_tile, _ = group_tiling(group_size)
+    seen = covered_tokens(plan, row_len, row_ctx, group_size, window)
+    for row in range(rows):
+        first_pos = row_ctx[row] - row_len[row]
+        for token in range(row_len[row]):
+            ranges = sorted(seen[(row, token)])
+            # the ranges follow one another without a gap or an overlap ...
+            for (a0, a1), (b0, b1) in zip(ranges, ranges[1:]):
+                assert a1 == b0 or (b0 == b1), (ranges, row, token)
+            lo, hi = ranges[0][0], max(r[1] for r in ranges)
+            # ... and hold every key the token may see: up to itself, from the window's edge (a tile's range is that of
+            # all its tokens, the kernel masks the rest)
+            position = first_pos + token
+            assert hi >= position + 1
+            assert lo <= (0 if window is None else max(0, position - window + 1))
+            if window is None:
+                assert lo == 0
+    # slots: one per split item, consecutive within a merge, none left over
+    slots = plan.item_slot.tolist()
+    used = sorted(s for s in slots if s >= 0)
+    assert used == list(range(plan.n_slots))
+    for (row, q0, first_slot, count) in plan.merges.tolist():
+        members = [i for i, s in enumerate(slots) if first_slot <= s < first_slot + count]
+        assert len(members) == count and count <= MAX_SPLITS
+        assert all(plan.items[i][0] == row and plan.items[i][1] == q0 for i in members)
+        begins = [int(plan.items[i][2]) for i in members]
+        assert all(b % KEY_ALIGN == 0 for b in begins[1:])
+    assert sum(c for *_, c in plan.merges.tolist()) == plan.n_slots
+    # rows with many tiles go to the workgroup kernel when it is offered, and only those
+    tiles_per_row = [-(-n // tokens_per_tile) for n in row_len]
+    rows_in_tiles = {int(r) for r in plan.tiles[:, 0]} if len(plan.tiles) else set()
+    expected = {r for r in range(rows) if most and tiles_per_row[r] >= MIN_TILES_FOR_WORKGROUPS}
+    assert rows_in_tiles == expected
+    keys_of_tiles = [int(k_end - k_begin) for _, _, k_begin, k_end in plan.tiles.tolist()]
+    assert keys_of_tiles == sorted(keys_of_tiles, reverse=True)              # the longest start first
+
+
+def test_captured_steps_get_arrays_of_one_shape():
+    group_size, n_kv = 4, 8
+    rows = 5
+    fixed = fixed_split_count(rows, group_size, n_kv, 4096)
+    shapes = set()
+    for contexts in ([1] * rows, [4096] * rows, [1, 17, 300, 2049, 4000], [33] * rows):
+        plan = build_attention_plan([1] * rows, contexts, group_size, n_kv, None, fixed_splits=fixed)
+        shapes.add((plan.items.shape, plan.item_slot.shape, plan.merges.shape, plan.n_slots, plan.tiles.shape))
+        for (row, q0, k_begin, k_end) in plan.items.tolist():
+            assert 0 <= k_begin <= k_end <= contexts[row]
+        # exactly one item of a row ends at its context and is not empty: the one that takes the new token
+        for row in range(rows):
+            ending = [(b, e) for (r, _, b, e) in plan.items.tolist() if r == row and e == contexts[row] and b < e]
+            assert len(ending) == 1
+    assert len(shapes) == 1
+    assert fixed_split_count(64, group_size, n_kv, 4096) < fixed_split_count(1, group_size, n_kv, 4096)
+
+
+def test_four_or_eight_tiles_per_workgroup():
+    """One short prompt is bounded by its longest workgroup and takes four tiles per workgroup; long rows and many rows
+    keep every compute unit busy and take eight; a kernel that offers only four gets four."""
+    def chosen(lens, ctxs, most=8):
+        return build_attention_plan(lens, ctxs, 4, 8, None, workgroup_tiles=most).tiles_per_workgroup
+    assert chosen([2048], [2048]) == 4
+    assert chosen([1024], [1024]) == 4
+    assert chosen([4096], [4096]) == 8
+    assert chosen([2048], [32768]) == 8
+    assert chosen([512] * 16, [512] * 16) == 8
+    assert chosen([4096], [4096], most=4) == 4
+    assert chosen([1] * 8, [4096] * 8) == 0                                  # no row has enough tiles
+    assert build_attention_plan([4096], [4096], 4, 8, None).tiles_per_workgroup == 0

@@ -18,9 +18,9 @@ def requests_for(case, lengths, seed0=100):
     return {f"q{i}": random_tokens(vocab, n, seed0 + i) for i, n in enumerate(lengths)}, {f"q{i}": (n, seed0 + i) for i, n in enumerate(lengths)}
 
 
-def run(case, steps, max_tokens, tmp_path, page_size=None):
+def run(case, steps, max_tokens, tmp_path, page_size=None, fused=False):
     page = page_size or CASES[case][2]
-    runner = make_runner(model_folder(case), "float32", max_tokens, page, device="cpu", ops=TorchOps())
+    runner = make_runner(model_folder(case), "float32", max_tokens, page, device="cpu", ops=TorchOps(fused=fused))
     report = io.StringIO()
     replay(runner, traces.to_lines(steps).splitlines(), str(tmp_path), report)
     assert report.getvalue().split() == [w for s in steps for w in ("done", str(s["step"]))]
@@ -57,6 +57,23 @@ def test_every_schedule_matches_the_plain_implementation(case, schedule, tmp_pat
     if schedule == "mixed":
         assert sum(lengths) > 2 * budget            # more tokens ran through than the pool holds: pages were used again
     check(case, results, meta)
+
+
+@pytest.mark.parametrize("case", ["A", "B", "C"])
+@pytest.mark.parametrize("schedule", ["tail", "mixed"])
+def test_the_fused_dataflow_matches_the_plain_implementation(case, schedule, tmp_path):
+    """The same with the twins of the fused kernels offered to the parts: projections that add their result to the
+    residual stream and prepare the next norm, projections that apply a prepared norm as a scale of their rows, and
+    single-token steps whose attention normalises, rotates and stores the new token itself."""
+    lengths = (5, 17, 33, 70, 100, 41, 64, 1, 90, 130, 20, 77) if schedule == "mixed" else (70, 33, 100)
+    requests, meta = requests_for(case, lengths)
+    steps = traces.tail_decoded(requests, 32) if schedule == "tail" else traces.mixed(requests, seed=7, budget_tokens=256)
+    results, runner = run(case, steps, traces.peak_tokens(steps), tmp_path, fused=True)
+    check(case, results, meta)
+    calls = runner.ops.fused_calls
+    assert calls["into_stream"] > 0 and calls["row_scale"] > 0 and calls["gated"] > 0
+    if schedule == "tail":
+        assert calls["decode_attention"] > 0
 
 
 def test_a_step_refuses_what_does_not_fit(tmp_path):

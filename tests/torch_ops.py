@@ -13,10 +13,60 @@ from llmserver_amd.parts.attention import group_tiling  # noqa: F401  (kept for 
 
 
 class TorchOps:
+    """``fused=True`` also offers the twins of the fused kernels (sum and norm folded into the few-row products, q/k
+    norm, rotation and cache write inside the attention of single-token steps), for any type and size, so that the
+    parts' fused dataflow runs on the CPU as it does on the GPU."""
     name = "torch"
+    FUSED_ROWS = 16
+
+    def __init__(self, fused: bool = False):
+        self.fuse_stream_updates = fused
+        self.fused = fused
+        self.fused_calls = {"row_scale": 0, "into_stream": 0, "gated": 0, "decode_attention": 0}
 
     def preload(self, head_dims, dtype):
         pass
+
+    # -- twins of the fused few-row products ------------------------------------------------------
+    def row_scale_fits(self, x, weight, row_scale) -> bool:
+        return self.fused and x.shape[1] == weight.shape[1] and 0 < x.shape[0] <= self.FUSED_ROWS
+
+    @staticmethod
+    def _scaled(y, row_scale, width):
+        if row_scale is None:
+            return y
+        square_sums, eps = row_scale
+        return y * torch.rsqrt(square_sums.float().sum(dim=1, keepdim=True) / width + eps)
+
+    def linear_few_rows(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0, row_scale=None):
+        if not self.row_scale_fits(x, weight, row_scale):
+            return None
+        self.fused_calls["row_scale"] += row_scale is not None
+        y = self._scaled(x.float() @ weight.float().t(), row_scale, x.shape[1])
+        return y if (out_float32 or x.dtype == torch.float32) else y.to(x.dtype)
+
+    def linear_into_stream(self, x, weight, resid, norm_weight, rows_per_workgroup=0, row_scale=None):
+        if not self.row_scale_fits(x, weight, row_scale):
+            return None
+        self.fused_calls["into_stream"] += 1
+        y = self._scaled(x.float() @ weight.float().t(), row_scale, x.shape[1]).to(x.dtype)
+        stream = (resid.float() + y.float()).to(resid.dtype)
+        weighted = (stream.float() * norm_weight).to(resid.dtype)
+        squares = stream.float() ** 2
+        parts = torch.stack([squares[:, i::3].sum(dim=1) for i in range(3)], dim=1)      # any split of the row will do
+        return stream, weighted, parts
+
+    def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None):
+        if not self.row_scale_fits(x, gate_up_weight, row_scale):
+            return None
+        self.fused_calls["gated"] += 1
+        gate_up = self._scaled(x.float() @ gate_up_weight.float().t(), row_scale, x.shape[1])
+        inter = gate_up.shape[1] // 2
+        gate, up = gate_up[:, :inter], gate_up[:, inter:]
+        return (gate * torch.sigmoid(gate) * up).to(x.dtype)
+
+    def decode_fusion_fits(self, dtype, head_dim) -> bool:
+        return self.fused
 
     def linear(self, x, weight, out=None, out_float32=False):
         y = (x.float() @ weight.float().t())
@@ -79,9 +129,20 @@ class TorchOps:
         values[pages, :, :, slots] = heads[:, n_q + n_kv:].to(values.dtype)
 
     def paged_attention(self, qkv, out, keys, values, table, row_start, row_len, row_ctx, plan, scale, window, page_size,
-                        n_q, n_kv, head_dim, ctx):
+                        n_q, n_kv, head_dim, ctx, decode_fusion=None):
         """Per request row: gather its keys/values through the block table, one softmax over all
-        keys a query may see (no tiles, no splits)."""
+        keys a query may see (no tiles, no splits).  ``decode_fusion``: the step's rows bring one token each and
+        ``qkv`` is the raw projection, which is left as it is."""
+        if decode_fusion is not None:
+            self.fused_calls["decode_attention"] += 1
+            q_weight, k_weight, eps, cos_sin, write_cache = decode_fusion
+            rows = table.shape[0]
+            assert qkv.shape[0] == rows and all(int(n) == 1 for n in row_len)
+            qkv = qkv.clone()
+            token_row = torch.arange(rows, dtype=torch.int32, device=qkv.device)
+            positions = (row_ctx - 1).to(torch.int32)
+            self.qk_norm_rope_kv_write(qkv, keys, values, table, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
+                                       n_q, n_kv, head_dim, write_cache)
         n = qkv.shape[0]
         q_all = qkv.view(n, n_q + 2 * n_kv, head_dim)[:, :n_q].float()
         group = n_q // n_kv
