@@ -469,11 +469,12 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
 // of one request (SUB tiles each).  They see (almost) the same keys, so each step's 32 keys and values are fetched
 // from the pages once per workgroup into LDS (double-buffered: the global loads of step i+1 are
 // issued before the products of step i and stored to the other buffer afterwards, one barrier a
-// step) and every wavefront reads its MFMA operands from there.  Rows in LDS are padded so that
-// the operand reads of a wavefront spread over the banks.  No key ranges are split here: such
+// step) and every wavefront reads its MFMA operands from there, 16 bytes per lane and read (8-byte
+// reads reach three quarters of the LDS rate at best).  Rows in LDS are padded so that the operand
+// reads of a wavefront spread over the banks.  No key ranges are split here: such
 // rows have many tiles.  `tiles[i]` = {row, first token of the workgroup's tiles, k_begin, k_end}.
 constexpr int K_ROW = D * 2 + 16;                 // bytes of a key row in LDS
-constexpr int V_ROW = 32 * 2 + 8;                 // bytes of a value row (one head dimension, 32 keys)
+constexpr int V_ROW = 32 * 2 + 16;                // bytes of a value row (one head dimension, 32 keys; see store_lds for their order)
 constexpr int K_TILE_BYTES = 32 * K_ROW, V_TILE_BYTES = D * V_ROW;
 // A step is fetched as two halves of 16 keys (with pages of 16 or more keys each half lies in one page):
 // per half, 16-byte pieces of keys (16 keys x D, contiguous in the page) and 8-byte pieces of values (D rows of 4 keys).
@@ -645,7 +646,9 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
                         if (kpos < k_begin || kpos >= k_end) piece[e] = (bf16_t)0.f;
                     }
                 }
-                if (q < V_HALF_PIECES) *reinterpret_cast<bf16x4*>(vl + (q >> 2) * V_ROW + 8 * (4 * h + (q & 3))) = piece;
+                // Keys 4 s .. 4 s + 3 of half h go to bytes 16 s + 8 h: the eight keys that lane quad s of the output
+                // product multiplies (four of each half, as the score product left them) are then 16 contiguous bytes.
+                if (q < V_HALF_PIECES) *reinterpret_cast<bf16x4*>(vl + (q >> 2) * V_ROW + 16 * (q & 3) + 8 * h) = piece;
             }
         }
     };
@@ -712,14 +715,7 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
         }
 #pragma unroll
         for (int c = 0; c < ND; ++c) {
-            const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vl + (16 * c + col) * V_ROW + 8 * quad);
-            const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vl + (16 * c + col) * V_ROW + 32 + 8 * quad);
-            bf16x8 vf;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                vf[r] = lo4[r];
-                vf[4 + r] = hi4[r];
-            }
+            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vl + (16 * c + col) * V_ROW + 16 * quad);
 #pragma unroll
             for (int u = 0; u < SUB; ++u) acc[u][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], acc[u][c], 0, 0, 0);
         }
