@@ -24,6 +24,35 @@ def test_greedy_generation_matches_the_plain_implementation(case):
     assert agree >= 20, (got_bf16, expected)             # bfloat16 may leave the greedy path where two logits nearly tie
 
 
+@pytest.mark.parametrize("case", ["A", "B", "C"])
+@pytest.mark.parametrize("rows", [5, 12, 16, 24])
+def test_wide_decode_steps_match_the_plain_implementation(case, rows):
+    """One step that decodes a token for each of 5, 12, 16 or 24 requests at once (bfloat16): up to 16 rows the
+    few-row products carry the sums and norms between them in their epilogues (one row per wavefront up to 8, two
+    beyond), 24 rows go through the library's products and the separate kernels; every row must give the plain
+    implementation's logits for its own sequence."""
+    import numpy as np
+    from helpers import plain_logits
+    from llmserver_amd.cache import CacheManager
+    from llmserver_amd.engine import ModelRunner, StepEntry, load_model
+    print(f"wide decode step {case} {rows} rows", flush=True)
+    raw, _, page = CASES[case]
+    model = load_model(model_folder(case), "cuda", "bfloat16")
+    cache = CacheManager(model.cache_specs(), page, 400, device="cuda", dtype=model.dtype)
+    runner = ModelRunner(model, cache, use_graphs=False)
+    lengths = [37, 5, 64, 2, 90, 16, 17, 33, 3, 70, 48, 9, 4, 81, 40, 7, 66, 21, 12, 55, 30, 8, 19, 44][:rows]
+    tokens = {f"r{i}": random_tokens(raw["vocab_size"], n, 300 + i) for i, n in enumerate(lengths)}
+    for rid, sequence in tokens.items():
+        cache.open(rid)
+        runner.step([StepEntry(rid, sequence[:-1], [])])
+    logits = runner.step([StepEntry(rid, sequence[-1:], [0]) for rid, sequence in tokens.items()]).float().cpu().numpy()
+    for i, n in enumerate(lengths):
+        expected = plain_logits(case, n, 300 + i)[n - 1].numpy()
+        error = float(np.abs(logits[i] - expected).max())
+        assert error <= 0.02 * max(1.0, float(np.abs(expected).max())), (i, n, error)
+    cache.check_invariants()
+
+
 def test_small_budget_and_few_pages_give_the_same_tokens():
     """Chunked prefill beside decodes under a token budget of 32, and a pool so small that requests
     are preempted and recomputed, must not change greedy output (float32)."""

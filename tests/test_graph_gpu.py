@@ -10,10 +10,10 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("case, n_live", [("A", 3), ("B", 3), ("B", 12)])
+@pytest.mark.parametrize("case, n_live", [("A", 3), ("B", 3), ("B", 12), ("B", 24)])
 def test_replayed_steps_equal_eager_steps(case, n_live, dtype):
-    """Three rows keep the products in the hand-written few-row kernel; twelve rows put the
-    library's products inside the captured graph."""
+    """Three and twelve rows keep the products in the hand-written few-row kernels (one and two rows per
+    wavefront in their fused epilogues); twenty-four rows put the library's products inside the captured graph."""
     from llmserver_amd.cache import CacheManager
     from llmserver_amd.engine import ModelRunner, StepEntry, load_model
     print(f"graph replay {case} {n_live} rows {dtype}", flush=True)
@@ -21,9 +21,9 @@ def test_replayed_steps_equal_eager_steps(case, n_live, dtype):
     model = load_model(model_folder(case), "cuda", dtype)
     runners = []
     for use_graphs in (True, False):
-        cache = CacheManager(model.cache_specs(), page, 200, device="cuda", dtype=model.dtype)
+        cache = CacheManager(model.cache_specs(), page, 500, device="cuda", dtype=model.dtype)
         runners.append(ModelRunner(model, cache, use_graphs=use_graphs))
-    lengths = [37, 5, 64, 1, 90, 16, 17, 33, 2, 70, 48, 9][:n_live]
+    lengths = [37, 5, 64, 1, 90, 16, 17, 33, 2, 70, 48, 9, 3, 81, 40, 7, 66, 21, 12, 55, 30, 8, 19, 44][:n_live]
     prompts = {f"r{i}": random_tokens(raw["vocab_size"], n, 1 + i) for i, n in enumerate(lengths)}
     feed = {rid: random_tokens(raw["vocab_size"], 80, 10 + i) for i, rid in enumerate(prompts)}
     for runner in runners:
