@@ -689,10 +689,17 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
                     tile_max[u] = fmaxf(tile_max[u], v);
                 }
         }
+        // The value operands are asked for now, so that they arrive while the softmax runs, and the output products
+        // of the first tile are issued before the softmax of the second: the MFMA pipe works on them meanwhile.
+        // (With one tile per wavefront there is nothing to overlap them with; they are read where they are used.)
+        bf16x8 vf[SUB > 1 ? ND : 1];
+        if (SUB > 1) {
+#pragma unroll
+            for (int c = 0; c < ND; ++c) vf[c] = *reinterpret_cast<const bf16x8*>(vl + (16 * c + col) * V_ROW + 16 * quad);
+        }
         // The running maximum of a pair only moves when some key of this step beats it, which
         // soon becomes rare: then the exchange between the lanes of a pair and the rescaling of
         // the accumulators are skipped (the result is the same, the maximum being unchanged).
-        bf16x8 pf[SUB];
 #pragma unroll
         for (int u = 0; u < SUB; ++u) {
             if (__any(tile_max[u] > run_max[u])) {
@@ -706,18 +713,18 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
                 for (int c = 0; c < ND; ++c) acc[u][c] *= alpha;
             }
             const float shift = run_max[u] == NEG_INF ? 0.f : -run_max[u] * scale_log2;
+            bf16x8 pf;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[u][e], scale_log2, shift));
                 run_sum[u] += p;
-                pf[u][e] = (bf16_t)p;
+                pf[e] = (bf16_t)p;
             }
-        }
 #pragma unroll
-        for (int c = 0; c < ND; ++c) {
-            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vl + (16 * c + col) * V_ROW + 16 * quad);
-#pragma unroll
-            for (int u = 0; u < SUB; ++u) acc[u][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], acc[u][c], 0, 0, 0);
+            for (int c = 0; c < ND; ++c) {
+                const bf16x8 value = SUB > 1 ? vf[SUB > 1 ? c : 0] : *reinterpret_cast<const bf16x8*>(vl + (16 * c + col) * V_ROW + 16 * quad);
+                acc[u][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(value, pf, acc[u][c], 0, 0, 0);
+            }
         }
     };
     auto compute = [&](int buf, int kt) {

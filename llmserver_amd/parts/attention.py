@@ -74,9 +74,9 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
     """4 or ``most`` tiles per workgroup of the prompt-portion kernel, whichever the step's rows finish sooner with.
 
     A workgroup walks its keys in steps of 32.  With all compute units busy, eight tiles per workgroup get more out of
-    every step (measured on Qwen3-8B shapes: 2.9 ns a step against 2 x 2.13 ns for the same tokens in two workgroups
+    every step (measured on Qwen3-8B shapes: 2.75 ns a step against 2 x 2.0 ns for the same tokens in two workgroups
     of four; setting up and draining a workgroup costs about 8 steps more), but a step of theirs takes longer
-    (1.52 against 1.4 us), and the workgroup with the most steps bounds the launch from below: one short prompt
+    (1.40 against 1.37 us), and the workgroup with the most steps bounds the launch from below: one short prompt
     finishes sooner with four, long rows and many rows with eight."""
     if most <= 4:
         return most
@@ -94,7 +94,7 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
             total += int(steps.sum()) + 8 * len(steps)
             longest = max(longest, int(steps.max()))
         return max(total * heads * ns_per_step * 1e-3, longest * us_per_step_alone)
-    return most if estimate(most, 2.9, 1.52) < estimate(4, 2.13, 1.4) else 4
+    return most if estimate(most, 2.75, 1.40) < estimate(4, 2.0, 1.37) else 4
 
 
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
