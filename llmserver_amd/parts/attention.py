@@ -30,7 +30,7 @@ from .linear import Linear
 TILE_ROWS = 16          # rows of (token, group head) pairs one wavefront handles (MFMA N dimension)
 KEY_ALIGN = 32          # key ranges of split items start at multiples of this
 MAX_SPLITS = 64
-MIN_KEYS_PER_SPLIT = 256
+MIN_KEYS_PER_SPLIT = 64     # shorter key ranges than this are not worth a wavefront of their own (measured at batch 1 to 8)
 TARGET_WAVES = 1024     # wavefronts wanted in flight on 256 CUs (measured: more and shorter items cost more in the merge than they gain)
 
 
