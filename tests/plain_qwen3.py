@@ -91,13 +91,14 @@ def causal_attention(q, k, v, scale, window=None):
     return torch.matmul(torch.softmax(scores, dim=-1), v)
 
 
-def attention_block(x, tensors, prefix, config, positions, window=None, kv_store=None, kv_from=None):
+def attention_block(x, tensors, prefix, config, positions, window=None, kv_store=None, kv_from=None, cos_sin=None):
     """Projections, per-head q/k norm before the rotation, rotation, attention, output projection
     (/root/reference/utils/attention.py:119-128, 155-159, 299-300).
 
     ``kv_store`` (a dict) receives this layer's rotated keys and values under ``prefix``;
     ``kv_from`` names a prefix whose stored keys and values are used instead of this layer's own
-    (the tests' toy arrangement in which one layer reads another layer's cache)."""
+    (the tests' toy arrangement in which one layer reads another layer's cache).  ``cos_sin`` replaces the
+    rotation's cosines and sines (the tests' toy position encodings)."""
     n_q, n_kv, d = config["num_attention_heads"], config["num_key_value_heads"], head_dim_of(config)
     seq = x.shape[0]
 
@@ -111,7 +112,7 @@ def attention_block(x, tensors, prefix, config, positions, window=None, kv_store
     v = project("v_proj").view(seq, n_kv, d).permute(1, 0, 2)
     q = rms_norm(q, tensors[f"{prefix}.q_norm.weight"], config["rms_norm_eps"])
     k = rms_norm(k, tensors[f"{prefix}.k_norm.weight"], config["rms_norm_eps"])
-    cos, sin = rope_cos_sin(positions, d, rope_theta_of(config), x.dtype)
+    cos, sin = cos_sin if cos_sin is not None else rope_cos_sin(positions, d, rope_theta_of(config), x.dtype)
     q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
     if kv_store is not None:
         if kv_from is not None:

@@ -1,5 +1,7 @@
 """Generality of the parts, shown with toys that live in this file only: a mixer with state of its
-own, layers with different windows, a layer run twice, a layer that reads another layer's cache.
+own, a feed-forward that routes every token to one of several experts, another position encoding
+and layers without any, layers with different windows, a layer run twice, a layer that reads
+another layer's cache.
 Each toy is registered as an architecture, written as a random model folder, loaded and stepped
 through the framework's own step function in different cuts, without a change to the framework.
 The CPU variants use the torch twins of the kernels, the GPU variants the HIP kernels."""
@@ -17,8 +19,8 @@ from llmserver_amd.cache import CacheManager
 from llmserver_amd.config import ModelConfig, field, register_architecture
 from llmserver_amd.engine import ModelRunner, StepEntry, load_model
 from llmserver_amd.models.decoder import DecoderModel, LayerCall
-from llmserver_amd.parts import (MATRIX, GatedMLP, GQAttention, Linear, Mixer, ParamSpec, PreNormBlock, RMSNorm,
-                                 RotaryPosition, StateSpec, TokenEmbedding)
+from llmserver_amd.parts import (MATRIX, FeedForward, GatedMLP, GQAttention, Linear, Mixer, NoPosition, ParamSpec, PositionEncoding,
+                                 PreNormBlock, RMSNorm, RotaryPosition, StateSpec, TokenEmbedding)
 from llmserver_amd.weights import RandomInit, write_random_model
 from torch_ops import TorchOps
 
@@ -51,6 +53,66 @@ class RunningMeanMixer(Mixer):
         return out
 
 
+# ----------------------------------------------------------------------------- a feed-forward with routing
+class TopOneExperts(FeedForward):
+    """out = p_e(x) * expert_e(x) for the expert e with the largest router probability p (softmax of the router's
+    32-bit logits).  Every expert runs on every token and the others are masked out: wasteful, but free of host
+    decisions, so a step with this feed-forward can still be captured into a graph."""
+
+    def __init__(self, width, intermediate, n_experts):
+        self.router = Linear(width, ("router",), (n_experts,), out_float32=True)
+        self.experts = [GatedMLP(width, intermediate) for _ in range(n_experts)]
+
+    def param_specs(self):
+        specs = dict(self.router.param_specs())
+        for index, expert in enumerate(self.experts):
+            specs.update({f"experts.{index}.{name}": spec for name, spec in expert.param_specs().items()})
+        return specs
+
+    def assign(self, name, tensor):
+        if name.startswith("router."):
+            self.router.assign(name, tensor)
+        else:
+            _, index, rest = name.split(".", 2)
+            self.experts[int(index)].assign(rest, tensor)
+
+    def finalize(self):
+        self.router.finalize()
+        for expert in self.experts:
+            expert.finalize()
+
+    def forward(self, x, ctx):
+        probabilities = torch.softmax(self.router.forward(x, ctx).float(), dim=-1)
+        top, chosen = probabilities.max(dim=-1)
+        out = torch.zeros_like(x, dtype=torch.float32)
+        for index, expert in enumerate(self.experts):
+            weight = torch.where(chosen == index, top, torch.zeros_like(top))[:, None]
+            out += weight * expert.forward(x, ctx).float()
+        return out.to(x.dtype)
+
+
+# ----------------------------------------------------------------------------- another position encoding
+class HarmonicPosition(PositionEncoding):
+    """A rotate-half rotation whose pair i turns by position / (i + 1)^1.5: only the table of inverse
+    frequencies differs from the framework's own encoding, the kernels take any such table."""
+
+    def __init__(self, rotary_dim):
+        self.rotary_dim = rotary_dim
+        self._tables = {}
+
+    def inverse_frequencies(self):
+        return (torch.arange(1, self.rotary_dim // 2 + 1, dtype=torch.float32)) ** -1.5
+
+    def rotary_table(self, device):
+        # made once per device: a step that is being captured into a graph must not copy from the host
+        if str(device) not in self._tables:
+            self._tables[str(device)] = self.inverse_frequencies().to(device)
+        return self._tables[str(device)]
+
+    def cos_sin(self, ctx):
+        return ctx.computed(("harmonic", id(self)), lambda: ctx.ops.rotary_table(ctx.positions, self.rotary_table(ctx.device)))
+
+
 @dataclasses.dataclass(frozen=True)
 class ToyConfig(ModelConfig):
     MODEL_TYPE: ClassVar[str] = "toy_parts"
@@ -64,6 +126,8 @@ class ToyConfig(ModelConfig):
     rope_theta: float = field("rope_theta", float)
     layer_kinds: object = field("layer_kinds", object)       # per block: "mean", or an attention window (0 = all keys)
     layer_order: object = field("layer_order", object)       # per call: [block, cache, writes]
+    ffn_experts: object = field("ffn_experts", object, None)        # per block: 0 = dense, n = top-one of n experts
+    position_kinds: object = field("position_kinds", object, None)  # per block: "rope", "harmonic" or "none"
     tie_word_embeddings: bool = field("tie_word_embeddings", bool, False)
 
     @property
@@ -72,16 +136,20 @@ class ToyConfig(ModelConfig):
 
 
 def build_toy(config: ToyConfig) -> DecoderModel:
-    position = RotaryPosition(config.head_dim, config.rope_theta)
+    positions = {"rope": RotaryPosition(config.head_dim, config.rope_theta), "harmonic": HarmonicPosition(config.head_dim),
+                 "none": NoPosition()}
     blocks = []
-    for kind in config.layer_kinds:
+    for index, kind in enumerate(config.layer_kinds):
         if kind == "mean":
             mixer = RunningMeanMixer(config.hidden_size)
         else:
+            position = positions[config.position_kinds[index] if config.position_kinds else "rope"]
             mixer = GQAttention(config.hidden_size, config.num_attention_heads, config.num_key_value_heads, config.head_dim,
                                 position, qk_norm_eps=config.rms_norm_eps, window=kind or None)
+        n_experts = config.ffn_experts[index] if config.ffn_experts else 0
+        ffn = TopOneExperts(config.hidden_size, config.intermediate_size, n_experts) if n_experts else GatedMLP(config.hidden_size, config.intermediate_size)
         blocks.append(PreNormBlock(RMSNorm(config.hidden_size, config.rms_norm_eps), mixer,
-                                   RMSNorm(config.hidden_size, config.rms_norm_eps), GatedMLP(config.hidden_size, config.intermediate_size)))
+                                   RMSNorm(config.hidden_size, config.rms_norm_eps), ffn))
     order = [LayerCall(b, c, bool(w)) for b, c, w in config.layer_order]
     head = Linear(config.hidden_size, ("lm_head",), (config.vocab_size,), out_float32=True)
     return DecoderModel(config, TokenEmbedding(config.vocab_size, config.hidden_size), blocks,
@@ -99,7 +167,12 @@ TOYS = {
     "windows": dict(BASE, layer_kinds=[0, 9, 20, 0, 9], layer_order=[[i, i, 1] for i in range(5)]),
     # block 1 runs twice (shared weights, a cache for each run); the last call reads the cache block 0 wrote
     "order": dict(BASE, layer_kinds=[0, 0, 0], layer_order=[[0, 0, 1], [1, 1, 1], [1, 2, 1], [2, 0, 0]]),
+    # a dense feed-forward, top-one of three experts, top-one of two
+    "experts": dict(BASE, layer_kinds=[0, 0, 0], layer_order=[[i, i, 1] for i in range(3)], ffn_experts=[0, 3, 2]),
+    # the framework's rotation, another table of frequencies, no rotation at all
+    "positions": dict(BASE, layer_kinds=[0, 0, 0], layer_order=[[i, i, 1] for i in range(3)], position_kinds=["rope", "harmonic", "none"]),
 }
+DISCONTINUOUS = {"experts"}       # a router's choice can flip under bfloat16 rounding: compared in float32 only
 
 
 def plain_toy(raw, tensors, tokens):
@@ -120,12 +193,30 @@ def plain_toy(raw, tensors, tokens):
         else:
             slot = f"cache{cache}"
             local = {}
+            position_kind = raw["position_kinds"][block] if raw.get("position_kinds") else "rope"
+            cos_sin = None
+            if position_kind != "rope":
+                pairs = raw["head_dim"] // 2
+                rates = torch.arange(1, pairs + 1, dtype=h.dtype) ** -1.5 if position_kind == "harmonic" else torch.zeros(pairs, dtype=h.dtype)
+                angles = positions.to(h.dtype)[:, None] * torch.cat([rates, rates])[None, :]
+                cos_sin = (torch.cos(angles), torch.sin(angles))
             mixed = plain.attention_block(normed, tensors, f"{prefix}.self_attn", config, positions, kind or None,
-                                          kv_store=local if writes else stored, kv_from=None if writes else slot)
+                                          kv_store=local if writes else stored, kv_from=None if writes else slot, cos_sin=cos_sin)
             if writes:
                 stored[slot] = local[f"{prefix}.self_attn"]
         h = h + mixed
-        h = h + plain.swiglu_mlp(plain.rms_norm(h, tensors[f"{prefix}.post_attention_layernorm.weight"], eps), tensors, f"{prefix}.mlp")
+        normed = plain.rms_norm(h, tensors[f"{prefix}.post_attention_layernorm.weight"], eps)
+        n_experts = raw["ffn_experts"][block] if raw.get("ffn_experts") else 0
+        if n_experts:
+            probabilities = torch.softmax(normed @ tensors[f"{prefix}.mlp.router.weight"].T, dim=-1)
+            top, chosen = probabilities.max(dim=-1)
+            update = torch.zeros_like(h)
+            for expert in range(n_experts):
+                rows = chosen == expert
+                update[rows] = top[rows, None] * plain.swiglu_mlp(normed[rows], tensors, f"{prefix}.mlp.experts.{expert}")
+            h = h + update
+        else:
+            h = h + plain.swiglu_mlp(normed, tensors, f"{prefix}.mlp")
     return plain.rms_norm(h, tensors["model.norm.weight"], eps) @ tensors["lm_head.weight"].T
 
 
@@ -187,5 +278,7 @@ def test_toy_on_cpu(name):
 @pytest.mark.parametrize("name", sorted(TOYS))
 def test_toy_on_gpu(name, dtype, tol):
     print(f"toy {name} {dtype}", flush=True)
+    if name in DISCONTINUOUS and dtype != "float32":
+        pytest.skip("a router's choice can flip under bfloat16 rounding; this toy is compared in float32")
     from llmserver_amd.kernels import default_ops
     run_toy(name, "cuda", dtype, default_ops(), tol)
