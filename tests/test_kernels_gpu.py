@@ -405,7 +405,7 @@ def test_skinny_gemm(ops, rows, n, k):
 
 
 @pytest.mark.parametrize("rows", [1, 5, 8, 9, 16])
-@pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (6144, 1000), (200, 5120), (8192, 64)])
+@pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (6144, 1000), (200, 5120), (8192, 64), (5120, 512), (2048, 256)])
 def test_skinny_gemm_with_row_scale_and_stream_update(ops, rows, n, k):
     """The few-row product with a norm folded in on either side, against the separate kernels' twins:
     as a consumer it reads the stream times the norm's weights and divides its rows by the stream's rms,
