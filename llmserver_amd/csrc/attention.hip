@@ -785,13 +785,18 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
 // Merge the partial slots of a tile: out = sum_s w_s acc_s / sum_s w_s l_s, w_s = exp(m_s - max m).
 struct Merge { int row, q0, first_slot, n_slots; };
 
-__global__ __launch_bounds__(128) void merge_kernel(
+constexpr int MERGE_WAVES = 4;
+
+__global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
     elem_t* __restrict__ out, const int* __restrict__ row_start, const int* __restrict__ row_len,
     const Merge* __restrict__ merges, const float* __restrict__ part_acc, const float* __restrict__ part_ml, Geometry g) {
-    // One block per (tile, KV head, pair).  First the slots' weights (a thread per slot), then
-    // the weighted sum (a thread per output dimension, slots unrolled so their loads overlap).
+    // One block per (tile, KV head, pair).  First the slots' weights (a thread per slot), then the weighted sum:
+    // wavefront v takes slots v, v + 4, ... (four loads in flight each, so 64 slots are four trips to memory, not
+    // sixteen), a lane two neighbouring output dimensions, and the wavefronts' sums meet in LDS.
+    constexpr int PAIRS = D / 2, PER_LANE = (PAIRS + 63) / 64;
     __shared__ float weight[64];
     __shared__ float inv_total;
+    __shared__ float2 wave_total[MERGE_WAVES - 1][PAIRS];
     const Merge m = merges[blockIdx.x];
     const int col = blockIdx.z;
     const int kv_head = blockIdx.y / g.gtiles, gtile = blockIdx.y % g.gtiles;
@@ -799,8 +804,9 @@ __global__ __launch_bounds__(128) void merge_kernel(
     if (pair_token >= g.tokens_per_tile || m.q0 + pair_token >= row_len[m.row] || pair_head_in_group >= g.group) return;
     const size_t stride = (size_t)gridDim.y * 16;                       // pairs per slot
     const size_t base = ((size_t)m.first_slot * gridDim.y + blockIdx.y) * 16 + col;
-    if (threadIdx.x < 64) {
-        const int s = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (wave == 0) {
+        const int s = lane;
         float mx = NEG_INF, sum = 0.f;
         if (s < m.n_slots) {
             mx = part_ml[(base + s * stride) * 2];
@@ -812,20 +818,66 @@ __global__ __launch_bounds__(128) void merge_kernel(
         const float total = wave_sum(w * sum);
         if (s == 0) inv_total = total > 0.f ? 1.f / total : 0.f;
     }
+    // The partial results do not depend on the weights: their first loads are issued before the barrier.
+    const float* acc = part_acc + base * D;
+    float2 total[PER_LANE];
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) total[i] = make_float2(0.f, 0.f);
+    auto slot_values = [&](int s, int i) {
+        const int pair = min(lane + 64 * i, PAIRS - 1);
+        return *reinterpret_cast<const float2*>(acc + (size_t)min(s, m.n_slots - 1) * stride * D + 2 * pair);
+    };
+    float2 first[PER_LANE][4];
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) first[i][j] = slot_values(wave + MERGE_WAVES * j, i);
     __syncthreads();
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int s = wave + MERGE_WAVES * j;
+            const float w = s < m.n_slots ? weight[s] : 0.f;
+            total[i].x += w * first[i][j].x;
+            total[i].y += w * first[i][j].y;
+        }
+    for (int s0 = wave + 4 * MERGE_WAVES; s0 < m.n_slots; s0 += 4 * MERGE_WAVES) {
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) {
+            float2 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = slot_values(s0 + MERGE_WAVES * j, i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int s = s0 + MERGE_WAVES * j;
+                const float w = s < m.n_slots ? weight[s] : 0.f;
+                total[i].x += w * v[j].x;
+                total[i].y += w * v[j].y;
+            }
+        }
+    }
+    if (wave) {
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i)
+            if (lane + 64 * i < PAIRS) wave_total[wave - 1][lane + 64 * i] = total[i];
+    }
+    __syncthreads();
+    if (wave) return;
     const int head = kv_head * g.group + pair_head_in_group;
     elem_t* o = out + ((size_t)(row_start[m.row] + m.q0 + pair_token) * g.n_q + head) * D;
-    const float* acc = part_acc + base * D;
-    for (int dim = threadIdx.x; dim < D; dim += blockDim.x) {
-        float total = 0.f;
-        int s = 0;
-        for (; s + 4 <= m.n_slots; s += 4) {
-            const float a0 = acc[(size_t)(s + 0) * stride * D + dim], a1 = acc[(size_t)(s + 1) * stride * D + dim];
-            const float a2 = acc[(size_t)(s + 2) * stride * D + dim], a3 = acc[(size_t)(s + 3) * stride * D + dim];
-            total += weight[s] * a0 + weight[s + 1] * a1 + weight[s + 2] * a2 + weight[s + 3] * a3;
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) {
+        const int pair = lane + 64 * i;
+        if (pair >= PAIRS) continue;
+        float2 sum = total[i];
+#pragma unroll
+        for (int v = 0; v < MERGE_WAVES - 1; ++v) {
+            sum.x += wave_total[v][pair].x;
+            sum.y += wave_total[v][pair].y;
         }
-        for (; s < m.n_slots; ++s) total += weight[s] * acc[(size_t)s * stride * D + dim];
-        o[dim] = (elem_t)(total * inv_total);
+        o[2 * pair] = (elem_t)(sum.x * inv_total);
+        o[2 * pair + 1] = (elem_t)(sum.y * inv_total);
     }
 }
 
@@ -872,7 +924,7 @@ LSA_EXPORT int lsa_paged_attention(
     int err = (int)hipGetLastError();
     if (err || n_merges <= 0) return err;
     dim3 mgrid(n_merges, n_kv * gtiles, 16);
-    merge_kernel<<<mgrid, 128, 0, stream>>>((elem_t*)out, row_start, row_len, (const Merge*)merges, part_acc, part_ml, g);
+    merge_kernel<<<mgrid, MERGE_WAVES * 64, 0, stream>>>((elem_t*)out, row_start, row_len, (const Merge*)merges, part_acc, part_ml, g);
     LSA_LAUNCH_CHECK();
 }
 
