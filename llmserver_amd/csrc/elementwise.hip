@@ -36,25 +36,83 @@ __global__ void embedding_kernel(const T* __restrict__ table, const int* __restr
 // out = s * rsqrt(mean(s^2) + eps) * w, computed from the rounded s.
 // rows == nullptr: every token row t: resid[t] = s, out[t] = norm.
 // rows != nullptr: out[i] = norm of row rows[i]; resid is not written.
+// The update of a row comes as `d` (values of the row's type) or as `parts` partial sums in float32 (`sums`, the
+// same element of each `sums_stride` elements apart), which are added up and rounded to the row's type first.
+struct PartialSums {
+    const float* sums;
+    int parts;
+    size_t stride;
+};
+
 template <typename T, int V>
-__device__ inline void load_sum(const T* __restrict__ x, const T* __restrict__ d, int i, float (&s)[V]) {
+__device__ inline void load_sum(const T* __restrict__ x, const T* __restrict__ d, const PartialSums& p, size_t row_offset, int i,
+                                float (&s)[V]) {
+    float update[V];
+    const bool any = d || p.sums;
+    if (p.sums) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) update[k] = 0.f;
+        const float* src = p.sums + row_offset + i;
+        if (V % 4 == 0) {
+            // Four parts' loads are issued together: the parts are read in a quarter of the trips to memory.
+            constexpr int Q = V % 4 == 0 ? V / 4 : 1;
+            int part = 0;
+            for (; part + 4 <= p.parts; part += 4, src += 4 * p.stride) {
+                float4 v[4][Q];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int k = 0; k < Q; ++k) v[j][k] = *reinterpret_cast<const float4*>(src + j * p.stride + 4 * k);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int k = 0; k < Q; ++k) {
+                        update[4 * k] += v[j][k].x;
+                        update[4 * k + 1] += v[j][k].y;
+                        update[4 * k + 2] += v[j][k].z;
+                        update[4 * k + 3] += v[j][k].w;
+                    }
+            }
+            for (; part < p.parts; ++part, src += p.stride) {
+#pragma unroll
+                for (int k = 0; k < Q; ++k) {
+                    const float4 v = *reinterpret_cast<const float4*>(src + 4 * k);
+                    update[4 * k] += v.x;
+                    update[4 * k + 1] += v.y;
+                    update[4 * k + 2] += v.z;
+                    update[4 * k + 3] += v.w;
+                }
+            }
+        } else {
+            for (int part = 0; part < p.parts; ++part, src += p.stride) {
+#pragma unroll
+                for (int k = 0; k < V; ++k) update[k] += src[k];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < V; ++k) update[k] = Elem<T>::round(update[k]);
+    }
     if (V > 1) {
-        Vec16<T> a = load_vec16(x + i);
+        Vec16<T> a = load_vec16(x + row_offset + i);
 #pragma unroll
         for (int k = 0; k < V; ++k) s[k] = (float)a.v[k];
         if (d) {
-            Vec16<T> b = load_vec16(d + i);
+            Vec16<T> b = load_vec16(d + row_offset + i);
 #pragma unroll
-            for (int k = 0; k < V; ++k) s[k] = Elem<T>::round(s[k] + (float)b.v[k]);
+            for (int k = 0; k < V; ++k) update[k] = (float)b.v[k];
         }
     } else {
-        s[0] = (float)x[i];
-        if (d) s[0] = Elem<T>::round(s[0] + (float)d[i]);
+        s[0] = (float)x[row_offset + i];
+        if (d) update[0] = (float)d[row_offset + i];
+    }
+    if (any) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) s[k] = Elem<T>::round(s[k] + update[k]);
     }
 }
 
 template <typename T, int V>
-__global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid, const T* __restrict__ delta,
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid, const T* __restrict__ delta, PartialSums partial,
                                                           const float* __restrict__ weight, float eps,
                                                           T* __restrict__ out, const int* __restrict__ rows, int width) {
     // The first CACHE vectors of a thread stay in registers between the two passes (a row of up
@@ -62,9 +120,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
     constexpr int CACHE = 4;
     __shared__ float scratch[16];
     const int src_row = rows ? rows[blockIdx.x] : blockIdx.x;
-    T* x = resid + (size_t)src_row * width;
-    const T* d = delta ? delta + (size_t)src_row * width : nullptr;
+    const size_t row_offset = (size_t)src_row * width;
+    T* x = resid + row_offset;
     T* y = out + (size_t)blockIdx.x * width;
+    const bool updated = delta || partial.sums;
     const int stride = blockDim.x * V;
     float kept[CACHE][V];
     float sq = 0.f;
@@ -72,14 +131,14 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
     for (int c = 0; c < CACHE; ++c) {
         const int i = threadIdx.x * V + c * stride;
         if (i < width) {
-            load_sum<T, V>(x, d, i, kept[c]);
+            load_sum<T, V>(resid, delta, partial, row_offset, i, kept[c]);
 #pragma unroll
             for (int k = 0; k < V; ++k) sq += kept[c][k] * kept[c][k];
         }
     }
     for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
         float s[V];
-        load_sum<T, V>(x, d, i, s);
+        load_sum<T, V>(resid, delta, partial, row_offset, i, s);
 #pragma unroll
         for (int k = 0; k < V; ++k) sq += s[k] * s[k];
     }
@@ -93,10 +152,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
                 r.v[k] = (T)s[k];
                 o.v[k] = (T)(s[k] * rstd * weight[i + k]);
             }
-            if (d && !rows) store_vec16(x + i, r);
+            if (updated && !rows) store_vec16(x + i, r);
             store_vec16(y + i, o);
         } else {
-            if (d && !rows) x[i] = (T)s[0];
+            if (updated && !rows) x[i] = (T)s[0];
             y[i] = (T)(s[0] * rstd * weight[i]);
         }
     };
@@ -107,7 +166,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
     }
     for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
         float s[V];
-        load_sum<T, V>(x, d, i, s);
+        load_sum<T, V>(resid, delta, partial, row_offset, i, s);
         emit(i, s);
     }
 }
@@ -155,13 +214,14 @@ static int launch_embedding(const void* table, const int* ids, void* out, int n_
 }
 
 template <typename T>
-static int launch_add_rmsnorm(void* resid, const void* delta, const float* weight, float eps, void* out, const int* rows,
-                              int n_out, int width, hipStream_t stream) {
+static int launch_add_rmsnorm(void* resid, const void* delta, PartialSums partial, const float* weight, float eps, void* out,
+                              const int* rows, int n_out, int width, hipStream_t stream) {
     if (n_out <= 0) return 0;
+    if (delta && partial.sums) return -1;
     if (width % Elem<T>::kVec == 0)
-        add_rmsnorm_kernel<T, Elem<T>::kVec><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, weight, eps, (T*)out, rows, width);
+        add_rmsnorm_kernel<T, Elem<T>::kVec><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, partial, weight, eps, (T*)out, rows, width);
     else
-        add_rmsnorm_kernel<T, 1><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, weight, eps, (T*)out, rows, width);
+        add_rmsnorm_kernel<T, 1><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, partial, weight, eps, (T*)out, rows, width);
     LSA_LAUNCH_CHECK();
 }
 
@@ -194,8 +254,19 @@ LSA_EXPORT int lsa_embedding(int dtype, const void* table, const int* ids, void*
 }
 LSA_EXPORT int lsa_add_rmsnorm(int dtype, void* resid, const void* delta, const float* weight, float eps, void* out,
                                const int* rows, int n_out, int width, hipStream_t stream) {
-    return dtype ? launch_add_rmsnorm<bf16_t>(resid, delta, weight, eps, out, rows, n_out, width, stream)
-                 : launch_add_rmsnorm<float>(resid, delta, weight, eps, out, rows, n_out, width, stream);
+    const PartialSums none = {nullptr, 0, 0};
+    return dtype ? launch_add_rmsnorm<bf16_t>(resid, delta, none, weight, eps, out, rows, n_out, width, stream)
+                 : launch_add_rmsnorm<float>(resid, delta, none, weight, eps, out, rows, n_out, width, stream);
+}
+// The same with the update given as `parts` partial sums in float32, [parts, rows of resid, width]: they are added
+// up and rounded to the stream's type, as a product that had not been split would have been, then added to the stream.
+LSA_EXPORT int lsa_add_rmsnorm_partial_sums(int dtype, void* resid, const float* sums, int parts, long part_stride,
+                                            const float* weight, float eps, void* out, const int* rows, int n_out, int width,
+                                            hipStream_t stream) {
+    if (!sums || parts <= 0 || part_stride < 0) return -1;
+    const PartialSums partial = {sums, parts, (size_t)part_stride};
+    return dtype ? launch_add_rmsnorm<bf16_t>(resid, nullptr, partial, weight, eps, out, rows, n_out, width, stream)
+                 : launch_add_rmsnorm<float>(resid, nullptr, partial, weight, eps, out, rows, n_out, width, stream);
 }
 LSA_EXPORT int lsa_swiglu(int dtype, const void* gate_up, void* out, int n_tokens, int inter, hipStream_t stream) {
     return dtype ? launch_swiglu<bf16_t>(gate_up, out, n_tokens, inter, stream)

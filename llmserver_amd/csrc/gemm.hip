@@ -361,6 +361,131 @@ static int compute_units() {
     return units;
 }
 
+// ------------------------------------------------------------------------------------------
+// 17 to 64 rows of activations.  Every slice of X is now as large as four tiles of W, so a workgroup
+// whose wavefronts split K (each loading its own slice of X) would move several times more X than W.
+// Here the eight wavefronts of a workgroup take eight different tiles of W (128 rows) over the
+// same range of K instead, and share that range of X through LDS, 512 columns at a time; the
+// ranges of K are spread over workgroups (grid y) so that the chip is filled, and every workgroup
+// writes its partial sums in float32, [split, M, N].  Adding them up is left to whoever reads the
+// result next (the residual sum and norm that follow take partial sums), which costs no launch.
+constexpr int SPLIT_TILE_ROWS = 16 * GEMM_WAVES;       // rows of W per workgroup
+constexpr int SPLIT_SLAB = 512;                         // columns of X staged at a time
+constexpr int SPLIT_PITCH = SPLIT_SLAB * 2 + 16;        // bytes per staged row: 16 rows apart are 64 banks apart
+constexpr int SPLIT_CHUNK = 8;                          // k steps of W whose loads are issued together
+
+template <int MT>
+__global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                     float* __restrict__ partial, int M, int N, int K, int k_range) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char staged[];      // [2][16 MT][SPLIT_PITCH]
+    constexpr int BUFFER = 16 * MT * SPLIT_PITCH;
+    constexpr int PIECES = 16 * MT * (SPLIT_SLAB / 8) / (GEMM_WAVES * 64);      // 16-byte pieces of a slab per thread
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, quad = lane >> 4;
+    const int n0 = blockIdx.x * SPLIT_TILE_ROWS + 16 * wave;
+    const int k_first = blockIdx.y * k_range, k_last = min(K, k_first + k_range);
+    const bf16_t* wp = w + (size_t)min(n0 + col, N - 1) * K + 8 * quad;
+    const int k_safe = K - 8;
+    f32x4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    struct Chunk { bf16x8 a[SPLIT_CHUNK]; };
+    auto load_chunk = [&](Chunk& c, int k0) {
+#pragma unroll
+        for (int u = 0; u < SPLIT_CHUNK; ++u) c.a[u] = *reinterpret_cast<const bf16x8*>(wp + min(k0 + 32 * u + 8 * quad, k_safe) - 8 * quad);
+    };
+    auto multiply_chunk = [&](const Chunk& c, int k0, const unsigned char* slab, int k_in_slab) {
+#pragma unroll
+        for (int u = 0; u < SPLIT_CHUNK; ++u) {
+            bf16x8 a = c.a[u];
+            if (k0 + 32 * u + 8 * quad >= k_last) a = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const bf16x8 b = *reinterpret_cast<const bf16x8*>(slab + (16 * t + col) * SPLIT_PITCH + 2 * (k_in_slab + 32 * u + 8 * quad));
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+            }
+        }
+    };
+    // A slab of X: rows beyond M and columns beyond K are staged as zeros (their loads read a valid address).
+    struct Slab { bf16x8 piece[PIECES]; };
+    auto load_slab = [&](Slab& r, int k0) {
+#pragma unroll
+        for (int j = 0; j < PIECES; ++j) {
+            const int e = tid + GEMM_WAVES * 64 * j, m = e / (SPLIT_SLAB / 8), k = k0 + 8 * (e % (SPLIT_SLAB / 8));
+            r.piece[j] = *reinterpret_cast<const bf16x8*>(x + (size_t)min(m, M - 1) * K + min(k, k_safe));
+        }
+    };
+    auto store_slab = [&](const Slab& r, int k0, unsigned char* slab) {
+#pragma unroll
+        for (int j = 0; j < PIECES; ++j) {
+            const int e = tid + GEMM_WAVES * 64 * j, m = e / (SPLIT_SLAB / 8), piece = e % (SPLIT_SLAB / 8);
+            bf16x8 v = r.piece[j];
+            if (m >= M || k0 + 8 * piece >= K) v = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+            *reinterpret_cast<bf16x8*>(slab + m * SPLIT_PITCH + 16 * piece) = v;
+        }
+    };
+    if (k_first < k_last) {
+        constexpr int HALF = 32 * SPLIT_CHUNK;          // a slab is two chunks of W
+        Chunk p, q;
+        Slab next;
+        // Loads are issued in the order in which they are waited for: X of a slab before the W it meets.
+        load_slab(next, k_first);
+        load_chunk(p, k_first);
+        load_chunk(q, k_first + HALF);
+        store_slab(next, k_first, staged);
+        __syncthreads();
+        int buffer = 0, k0 = k_first;
+        // While a slab is multiplied, the next one travels through registers to the other buffer (which every
+        // wavefront has finished reading before the barrier that ended the previous round) and the W it will
+        // meet is requested, a chunk as soon as the registers of one are free.  The last slab requests nothing.
+        for (; k0 + SPLIT_SLAB < k_last; k0 += SPLIT_SLAB, buffer ^= 1) {
+            load_slab(next, k0 + SPLIT_SLAB);
+            multiply_chunk(p, k0, staged + buffer * BUFFER, 0);
+            load_chunk(p, k0 + SPLIT_SLAB);
+            multiply_chunk(q, k0 + HALF, staged + buffer * BUFFER, HALF);
+            load_chunk(q, k0 + SPLIT_SLAB + HALF);
+            store_slab(next, k0 + SPLIT_SLAB, staged + (buffer ^ 1) * BUFFER);
+            __syncthreads();
+        }
+        multiply_chunk(p, k0, staged + buffer * BUFFER, 0);
+        multiply_chunk(q, k0 + HALF, staged + buffer * BUFFER, HALF);
+    }
+    // Lane (col, quad) holds Y[16 t + col][n0 + 4 quad .. + 4].
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = 16 * t + col, n = n0 + 4 * quad;
+        if (m >= M) continue;
+        float* dst = partial + ((size_t)blockIdx.y * M + m) * N + n;
+        if (n + 3 < N && N % 4 == 0) {
+            *reinterpret_cast<f32x4*>(dst) = acc[t];
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < N) dst[r] = acc[t][r];
+        }
+    }
+}
+
+// Columns of X per workgroup (a multiple of 256) for a size: the one with which the compute units, working
+// through the workgroups in rounds, are done soonest; a round costs its columns plus a fixed part.
+static int split_range(int N, int K) {
+    const long tiles = (N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS;
+    const int units = compute_units();
+    const int whole = (K + 255) / 256 * 256;
+    long best_cost = -1;
+    int best = whole;
+    for (int range = whole; range >= 256; range -= 256) {
+        const long splits = (K + range - 1) / range;
+        const long cost = (tiles * splits + units - 1) / units * (range + 512);
+        if (best_cost < 0 || cost < best_cost) {       // ties: the larger range, fewer partial sums
+            best_cost = cost;
+            best = range;
+        }
+    }
+    return best;
+}
+
+
 // Rows of W per workgroup.  The compute units work through the workgroups in rounds, a round takes
 // as long as its workgroups have rows (plus a fixed part), and a round that is not full costs as
 // much as a full one: so the best size is the one with the smallest rounds * (rows + fixed part).
@@ -503,4 +628,36 @@ LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* h
     const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr};
     return launch<bf16_t, true>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)hidden, M, 2 * I, K, choose_rows(M, 2 * I, true, rows),
                                 fusion, stream);
+}
+
+// Partial sums that lsa_gemm_split writes for a size (the first dimension of its result), or -1 if it does not
+// take the size: 17 <= M <= 64, K a multiple of 8.
+LSA_EXPORT int lsa_gemm_split_parts(int M, int N, int K) {
+    if (M <= 16 || M > 64 || N <= 0 || K < 8 || K % 8 != 0) return -1;
+    const int range = split_range(N, K);
+    return (K + range - 1) / range;
+}
+
+// partial [lsa_gemm_split_parts(M, N, K), M, N] float32: sums over ranges of K of x [M, K] . w [N, K]^T (bfloat16);
+// their sum over the first dimension is the product.
+LSA_EXPORT int lsa_gemm_split(const void* x, const void* w, float* partial, int M, int N, int K, hipStream_t stream) {
+    if (lsa_gemm_split_parts(M, N, K) < 0 || !x || !w || !partial) return -1;
+    const int range = split_range(N, K);
+    const dim3 grid((N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS, (K + range - 1) / range), block(GEMM_WAVES * 64);
+#define LSA_SPLIT(MT)                                                                                                          \
+    {                                                                                                                          \
+        static bool sized = false;                                                                                             \
+        constexpr int bytes = 2 * 16 * MT * SPLIT_PITCH;                                                                       \
+        if (!sized) {                                                                                                          \
+            const hipError_t e = hipFuncSetAttribute((const void*)gemm_split_kernel<MT>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
+            if (e != hipSuccess) return (int)e;                                                                                \
+            sized = true;                                                                                                      \
+        }                                                                                                                      \
+        gemm_split_kernel<MT><<<grid, block, bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, partial, M, N, K, range);    \
+    }
+    if (M <= 32) LSA_SPLIT(2)
+    else if (M <= 48) LSA_SPLIT(3)
+    else LSA_SPLIT(4)
+#undef LSA_SPLIT
+    LSA_LAUNCH_CHECK();
 }

@@ -11,6 +11,7 @@ _P = c_void_p
 _SIGNATURES = {
     "lsa_embedding": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
     "lsa_add_rmsnorm": [c_int, _P, _P, _P, c_float, _P, _P, c_int, c_int, _P],
+    "lsa_add_rmsnorm_partial_sums": [c_int, _P, _P, c_int, c_long, _P, c_float, _P, _P, c_int, c_int, _P],
     "lsa_swiglu": [c_int, _P, _P, c_int, c_int, _P],
     "lsa_add_bias": [c_int, _P, _P, c_int, c_int, _P],
     "lsa_qk_norm_rope_kv_write": [c_int, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int,
@@ -27,6 +28,8 @@ _SIGNATURES = {
     "lsa_gemm_skinny_parts": [c_int, c_int, c_int],
     "lsa_gemm_skinny_stream": [_P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P, _P, _P, _P, _P, _P],
     "lsa_gemm_skinny_gated": [_P, _P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P],
+    "lsa_gemm_split_parts": [c_int, c_int, c_int],
+    "lsa_gemm_split": [_P, _P, _P, c_int, c_int, c_int, _P],
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

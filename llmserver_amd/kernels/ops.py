@@ -71,6 +71,8 @@ class HipOps:
         # Whether projections may fold the residual sum and the norm between two few-row products into their
         # epilogues (see linear_into_stream); off, every such sum and norm is a kernel of its own.
         self.fuse_stream_updates = True
+        # Whether projections whose result is added to the residual stream may leave it as partial sums at 17 to 64 rows.
+        self.split_products = True
 
     @staticmethod
     def required_modules(head_dims, dtype):
@@ -141,6 +143,25 @@ class HipOps:
                                              int(rows_per_workgroup), sums, parts, eps, _stream()), "gemm_skinny")
         return out
 
+    SPLIT_ROWS = 64         # most rows the product that leaves partial sums takes (it starts above the few-row kernels')
+
+    def linear_partial_sums(self, x, weight):
+        """``x @ weight^T`` for 17 to 64 rows as float32 partial sums ``[parts, T, out]`` over ranges of the inner
+        dimension (their sum is the product), or None if this is no case for it.  Whoever adds the result to the
+        residual stream adds the parts up (:meth:`add_rmsnorm` takes them)."""
+        rows, width = x.shape
+        if not (self.skinny_rows < rows <= self.SPLIT_ROWS) or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
+                or x.shape[1] != weight.shape[1] or not self.split_products:
+            return None
+        parts = self._gemm.lsa_gemm_split_parts(rows, weight.shape[0], width)
+        if parts < 2:           # refused, or so many rows of the weight that nothing is split: the library is as fast
+            return None
+        _check(x, "x", torch.bfloat16)
+        _check(weight, "weight", torch.bfloat16)
+        out = torch.empty((parts, rows, weight.shape[0]), device=x.device, dtype=torch.float32)
+        _launched(self._gemm.lsa_gemm_split(_ptr(x), _ptr(weight), _ptr(out), rows, weight.shape[0], width, _stream()), "gemm_split")
+        return out
+
     def linear_into_stream(self, x, weight, resid, norm_weight, rows_per_workgroup=0, row_scale=None):
         """The few-row product as an update of the residual stream ``resid [T, out]`` that a norm with weights
         ``norm_weight`` follows, in one launch: returns ``(stream, weighted, square_sums)`` with
@@ -198,15 +219,23 @@ class HipOps:
                                                   table.shape[0], _stream()), "embedding")
 
     def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None):
+        """``resid += delta`` (unless ``rows`` selects), ``out = rmsnorm(resid) * weight``.  ``delta``: None, a tensor
+        like ``resid``, or float32 partial sums ``[parts, T, width]`` of one (see :meth:`linear_partial_sums`)."""
         n_tokens, width = resid.shape
         _check(resid, "resid")
         _check(weight, "weight", torch.float32, (width,))
-        if delta is not None:
-            _check(delta, "delta", resid.dtype, (n_tokens, width))
         n_out = n_tokens if rows is None else rows.shape[0]
         _check(out, "out", resid.dtype, (n_out, width))
         if rows is not None:
             _check(rows, "rows", torch.int32, (n_out,))
+        if delta is not None and delta.dim() == 3:
+            _check(delta, "delta", torch.float32, (delta.shape[0], n_tokens, width))
+            _launched(self._elementwise.lsa_add_rmsnorm_partial_sums(
+                _code(resid), _ptr(resid), _ptr(delta), delta.shape[0], n_tokens * width, _ptr(weight), float(eps), _ptr(out),
+                _ptr(rows), n_out, width, _stream()), "add_rmsnorm")
+            return
+        if delta is not None:
+            _check(delta, "delta", resid.dtype, (n_tokens, width))
         _launched(self._elementwise.lsa_add_rmsnorm(_code(resid), _ptr(resid), _ptr(delta), _ptr(weight), float(eps),
                                                     _ptr(out), _ptr(rows), n_out, width, _stream()), "add_rmsnorm")
 

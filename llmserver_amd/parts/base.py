@@ -64,6 +64,8 @@ class Norm(Part):
     ``add_norm(resid, delta, ctx, rows=None)`` computes ``s = resid + delta`` in 32-bit (``delta``
     may be None), stores ``s`` back into ``resid`` and returns ``norm(s)``; with ``rows`` (int32
     device tensor) only those token rows are normalised and returned, ``resid`` is left alone.
+    A norm with ``weight`` and ``eps`` attributes (an RMSNorm) may be handed ``delta`` as float32
+    partial sums ``[parts, T, H]`` by a projection that was told this norm follows it.
     """
 
     def add_norm(self, resid, delta, ctx, rows=None):
@@ -74,13 +76,14 @@ class StreamUpdate:
     """What a part may return instead of a plain update of the residual stream, when its last
     projection has already added the update and prepared the norm that follows.
 
-    ``resid [T, H]`` is the stream with the update added, ``weighted [T, H] = resid * norm.weight``,
-    ``square_sums [T, P]`` float32 partial sums of ``resid^2`` over P parts of each row, ``norm`` the
-    norm they were prepared for.  A projection that reads ``weighted`` and divides its result rows
-    by ``sqrt(sum(square_sums) / H + eps)`` has multiplied the normalised stream."""
+    ``resid [T, H]`` is the stream with the update added, ``norm`` the norm that was prepared, in one of two ways.
+    Either ``weighted [T, H] = resid * norm.weight`` and ``square_sums [T, P]``, float32 partial sums of
+    ``resid^2`` over P parts of each row: a projection that reads ``weighted`` and divides its result rows by
+    ``sqrt(sum(square_sums) / H + eps)`` has multiplied the normalised stream.  Or ``normed [T, H]``, the norm's
+    result itself (the update came as partial sums, and the kernel that added them up went on to normalise)."""
 
-    def __init__(self, norm: "Norm", resid, weighted, square_sums):
-        self.norm, self.resid, self.weighted, self.square_sums = norm, resid, weighted, square_sums
+    def __init__(self, norm: "Norm", resid, weighted=None, square_sums=None, normed=None):
+        self.norm, self.resid, self.weighted, self.square_sums, self.normed = norm, resid, weighted, square_sums, normed
 
 
 class PendingNorm:
@@ -99,7 +102,7 @@ class PendingNorm:
                 self.prepared = delta
             resid, delta = delta.resid, None
         self.norm, self.resid, self.delta, self.ctx = norm, resid, delta, ctx
-        self._done = None
+        self._done = self.prepared.normed if self.prepared is not None else None
 
     def tensor(self):
         if self._done is None:
@@ -109,7 +112,7 @@ class PendingNorm:
 
     def row_scale(self):
         """``(weighted stream, (square_sums, eps))`` if a projection may apply the norm as a row scale, else None."""
-        if self.prepared is None or self._done is not None or not hasattr(self.norm, "eps"):
+        if self.prepared is None or self.prepared.weighted is None or self._done is not None or not hasattr(self.norm, "eps"):
             return None
         return self.prepared.weighted, (self.prepared.square_sums, self.norm.eps)
 

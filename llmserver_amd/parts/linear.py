@@ -63,7 +63,8 @@ class Linear(Part):
 
     def forward(self, x, ctx, out=None, sink=None):
         """``x`` is a tensor or a :class:`PendingNorm`.  With ``sink`` (a :class:`ResidualSink`) the result may
-        come back as a :class:`StreamUpdate`: already added to the residual stream, the following norm prepared."""
+        come back as a :class:`StreamUpdate`: already added to the residual stream, the following norm prepared
+        or carried out."""
         ops = ctx.ops
         fused = getattr(ops, "fuse_stream_updates", False)
         row_scale = None
@@ -78,6 +79,13 @@ class Linear(Part):
             done = ops.linear_into_stream(x, self.weight, sink.stream(), sink.norm.weight, row_scale=row_scale)
             if done is not None:
                 return StreamUpdate(sink.norm, *done)
+            # More rows: the product may leave its result as partial sums, which the kernel of the sum and the
+            # norm adds up on its way.
+            partial_sums = getattr(ops, "linear_partial_sums", None)
+            sums = partial_sums(x, self.weight) if partial_sums is not None and row_scale is None else None
+            if sums is not None:
+                stream = sink.stream()
+                return StreamUpdate(sink.norm, stream, normed=sink.norm.add_norm(stream, sums, ctx))
         if row_scale is not None:
             y = ops.linear_few_rows(x, self.weight, out=out, out_float32=self.out_float32, row_scale=row_scale)
         else:

@@ -404,6 +404,49 @@ def test_skinny_gemm(ops, rows, n, k):
             raise RuntimeError("refused")
 
 
+@pytest.mark.parametrize("rows", [17, 31, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (2050, 1000), (200, 5128), (8192, 64), (5120, 520), (127, 264)])
+def test_product_in_partial_sums(ops, rows, n, k):
+    """The product for 17 to 64 rows, which leaves partial sums over ranges of the inner dimension, against a float64
+    product of the same bfloat16 values: one range and many, ranges that end inside a staged slab, sizes that are no
+    multiple of the tiles.  Then the kernel that adds them up, adds the result to a residual stream and normalises,
+    against its twin."""
+    print(f"product in partial sums rows {rows} n {n} k {k}", flush=True)
+    torch.manual_seed(rows * n + k)
+    x = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(n, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
+    expected = (x.double() @ w.double().t()).float()
+    parts = ops._gemm.lsa_gemm_split_parts(rows, n, k)
+    assert parts >= 1
+    sums = torch.full((parts, rows, n), float("nan"), device=DEV)                          # every element must be written
+    assert ops._gemm.lsa_gemm_split(x.data_ptr(), w.data_ptr(), sums.data_ptr(), rows, n, k, None) == 0
+    torch.testing.assert_close(sums.sum(0), expected, atol=2e-4, rtol=1e-4)
+    offered = ops.linear_partial_sums(x, w)
+    assert (offered is None) == (parts < 2)                                               # nothing to split: left to the library
+    if offered is not None:
+        assert torch.equal(offered, sums)
+    for refused in (16, 65):
+        assert ops._gemm.lsa_gemm_split_parts(refused, n, k) == -1
+    assert ops._gemm.lsa_gemm_split_parts(rows, n, k + 4) == -1
+    resid = (2 * torch.randn(rows, n, device=DEV)).to(torch.bfloat16)
+    weight = 1 + 0.2 * torch.randn(n, device=DEV)
+    got_x, ref_x = resid.clone(), resid.clone()
+    got, ref = torch.empty_like(resid), torch.empty_like(resid)
+    ops.add_rmsnorm(got_x, sums, weight, 1e-5, got)
+    TorchOps().add_rmsnorm(ref_x, sums, weight, 1e-5, ref)
+    # the parts are added up in another order than the twin's: a sum on a rounding boundary may differ by one step
+    assert float((got_x.float() - ref_x.float()).abs().gt(0).float().mean()) < 0.01
+    torch.testing.assert_close(got_x.float(), ref_x.float(), atol=4e-2, rtol=1e-2)
+    close(got, ref, torch.bfloat16)
+    picked = torch.tensor([rows - 1, 0, 3, 3], device=DEV, dtype=torch.int32)
+    got_x = resid.clone()
+    got, ref = (torch.empty(4, n, device=DEV, dtype=torch.bfloat16) for _ in range(2))
+    ops.add_rmsnorm(got_x, sums, weight, 1e-5, got, picked)
+    TorchOps().add_rmsnorm(resid.clone(), sums, weight, 1e-5, ref, picked)
+    assert torch.equal(got_x, resid)
+    close(got, ref, torch.bfloat16)
+
+
 @pytest.mark.parametrize("rows", [1, 5, 8, 9, 16])
 @pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (6144, 1000), (200, 5120), (8192, 64), (5120, 512), (2048, 256)])
 def test_skinny_gemm_with_row_scale_and_stream_update(ops, rows, n, k):

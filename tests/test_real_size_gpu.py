@@ -1,7 +1,9 @@
-"""One decoder layer at the real sizes of Qwen3-8B (width 4096, 32/8 heads of 128, intermediate
+"""Two decoder layers at the real sizes of Qwen3-8B (width 4096, 32/8 heads of 128, intermediate
 12288, vocabulary 151936, tied head to keep the folder small) against the plain implementation:
 whole, in portions and token by token, in float32 and in bfloat16.  At these sizes a
-reduced-precision matrix mode on the 32-bit path would show at once."""
+reduced-precision matrix mode on the 32-bit path would show at once, and the products that depend
+on the size run as in serving: the portion of 40 tokens leaves the results of both projections
+into the residual stream as partial sums (two layers, so that the feed-forward's has a norm after it)."""
 import numpy as np
 import pytest
 import torch
@@ -13,7 +15,7 @@ from llmserver_amd.weights import RandomInit, write_random_model
 
 pytestmark = pytest.mark.gpu
 
-REAL = dict(model_type="qwen3", num_hidden_layers=1, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+REAL = dict(model_type="qwen3", num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
             head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
             attention_bias=False, tie_word_embeddings=True)
 

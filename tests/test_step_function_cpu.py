@@ -72,6 +72,7 @@ def test_the_fused_dataflow_matches_the_plain_implementation(case, schedule, tmp
     check(case, results, meta)
     calls = runner.ops.fused_calls
     assert calls["into_stream"] > 0 and calls["row_scale"] > 0 and calls["gated"] > 0
+    assert calls["partial_sums"] > 0
     if schedule == "tail":
         assert calls["decode_attention"] > 0
 

@@ -22,7 +22,7 @@ class TorchOps:
     def __init__(self, fused: bool = False):
         self.fuse_stream_updates = fused
         self.fused = fused
-        self.fused_calls = {"row_scale": 0, "into_stream": 0, "gated": 0, "decode_attention": 0}
+        self.fused_calls = {"row_scale": 0, "into_stream": 0, "gated": 0, "decode_attention": 0, "partial_sums": 0}
 
     def preload(self, head_dims, dtype):
         pass
@@ -65,6 +65,13 @@ class TorchOps:
         gate, up = gate_up[:, :inter], gate_up[:, inter:]
         return (gate * torch.sigmoid(gate) * up).to(x.dtype)
 
+    def linear_partial_sums(self, x, weight):
+        if not self.fused or not 16 < x.shape[0] <= 64:
+            return None
+        self.fused_calls["partial_sums"] += 1
+        bounds = [0, x.shape[1] // 3, x.shape[1] // 2, x.shape[1]]                      # any split of the inner dimension
+        return torch.stack([x[:, a:b].float() @ weight[:, a:b].float().t() for a, b in zip(bounds, bounds[1:])])
+
     def decode_fusion_fits(self, dtype, head_dim) -> bool:
         return self.fused
 
@@ -80,6 +87,8 @@ class TorchOps:
         out.copy_(table[token_ids.long()])
 
     def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None):
+        if delta is not None and delta.dim() == 3:                                       # partial sums of the update
+            delta = delta.sum(dim=0).to(resid.dtype)
         if rows is None:
             total = resid.float()
             if delta is not None:
