@@ -41,7 +41,13 @@ def _ptr(tensor):
     return None if tensor is None else tensor.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """Handle of torch's current stream on the current device (asked for at every launch: the fast way if torch has it)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -73,6 +79,7 @@ class HipOps:
         self.fuse_stream_updates = True
         # Whether projections whose result is added to the residual stream may leave it as partial sums at 17 to 64 rows.
         self.split_products = True
+        self._split_parts = {}      # (rows, out, in) -> partial sums the split product writes for that size
 
     @staticmethod
     def required_modules(head_dims, dtype):
@@ -153,7 +160,10 @@ class HipOps:
         if not (self.skinny_rows < rows <= self.SPLIT_ROWS) or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
                 or x.shape[1] != weight.shape[1] or not self.split_products:
             return None
-        parts = self._gemm.lsa_gemm_split_parts(rows, weight.shape[0], width)
+        size = (rows, weight.shape[0], width)
+        parts = self._split_parts.get(size)
+        if parts is None:
+            parts = self._split_parts[size] = self._gemm.lsa_gemm_split_parts(*size)
         if parts < 2:           # refused, or so many rows of the weight that nothing is split: the library is as fast
             return None
         _check(x, "x", torch.bfloat16)
