@@ -362,24 +362,26 @@ static int compute_units() {
 }
 
 // ------------------------------------------------------------------------------------------
-// 17 to 64 rows of activations.  Every slice of X is now as large as four tiles of W, so a workgroup
-// whose wavefronts split K (each loading its own slice of X) would move several times more X than W.
-// Here the eight wavefronts of a workgroup take eight different tiles of W (128 rows) over the
-// same range of K instead, and share that range of X through LDS, 512 columns at a time; the
-// ranges of K are spread over workgroups (grid y) so that the chip is filled, and every workgroup
-// writes its partial sums in float32, [split, M, N].  Adding them up is left to whoever reads the
-// result next (the residual sum and norm that follow take partial sums), which costs no launch.
+// 17 to 128 rows of activations.  Every slice of X is now as large as several tiles of W, so a
+// workgroup whose wavefronts split K (each loading its own slice of X) would move several times
+// more X than W.  Here the eight wavefronts of a workgroup take eight different tiles of W (128
+// rows) over the same range of K instead, and share that range of X through LDS, a slab of 512 or
+// 256 columns at a time; the ranges of K are spread over workgroups so that the chip is filled,
+// and every workgroup writes its partial sums in float32, [split, M, N].  Adding them up is left
+// to whoever reads the result next (the residual sum and norm that follow take partial sums),
+// which costs no launch.
 constexpr int SPLIT_TILE_ROWS = 16 * GEMM_WAVES;       // rows of W per workgroup
-constexpr int SPLIT_SLAB = 512;                         // columns of X staged at a time
-constexpr int SPLIT_PITCH = SPLIT_SLAB * 2 + 16;        // bytes per staged row: 16 rows apart are 64 banks apart
-constexpr int SPLIT_CHUNK = 8;                          // k steps of W whose loads are issued together
+constexpr int SPLIT_MOST_ROWS = 128;                    // most rows of X
 
-template <int MT>
+// SLAB: columns of X staged at a time (512 up to 64 rows, 256 beyond: two slabs have to fit into LDS).
+template <int MT, int SLAB>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                      float* __restrict__ partial, int M, int N, int K, int k_range) {
+    constexpr int SPLIT_PITCH = SLAB * 2 + 16;          // bytes per staged row: 16 rows apart are 64 banks apart
+    constexpr int SPLIT_CHUNK = SLAB / 64;              // k steps of W whose loads are issued together: half a slab
     extern __shared__ __attribute__((aligned(16))) unsigned char staged[];      // [2][16 MT][SPLIT_PITCH]
     constexpr int BUFFER = 16 * MT * SPLIT_PITCH;
-    constexpr int PIECES = 16 * MT * (SPLIT_SLAB / 8) / (GEMM_WAVES * 64);      // 16-byte pieces of a slab per thread
+    constexpr int PIECES = 16 * MT * (SLAB / 8) / (GEMM_WAVES * 64);      // 16-byte pieces of a slab per thread
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, quad = lane >> 4;
     const int n0 = blockIdx.x * SPLIT_TILE_ROWS + 16 * wave;
     const int k_first = blockIdx.y * k_range, k_last = min(K, k_first + k_range);
@@ -411,14 +413,14 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_
     auto load_slab = [&](Slab& r, int k0) {
 #pragma unroll
         for (int j = 0; j < PIECES; ++j) {
-            const int e = tid + GEMM_WAVES * 64 * j, m = e / (SPLIT_SLAB / 8), k = k0 + 8 * (e % (SPLIT_SLAB / 8));
+            const int e = tid + GEMM_WAVES * 64 * j, m = e / (SLAB / 8), k = k0 + 8 * (e % (SLAB / 8));
             r.piece[j] = *reinterpret_cast<const bf16x8*>(x + (size_t)min(m, M - 1) * K + min(k, k_safe));
         }
     };
     auto store_slab = [&](const Slab& r, int k0, unsigned char* slab) {
 #pragma unroll
         for (int j = 0; j < PIECES; ++j) {
-            const int e = tid + GEMM_WAVES * 64 * j, m = e / (SPLIT_SLAB / 8), piece = e % (SPLIT_SLAB / 8);
+            const int e = tid + GEMM_WAVES * 64 * j, m = e / (SLAB / 8), piece = e % (SLAB / 8);
             bf16x8 v = r.piece[j];
             if (m >= M || k0 + 8 * piece >= K) v = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
             *reinterpret_cast<bf16x8*>(slab + m * SPLIT_PITCH + 16 * piece) = v;
@@ -438,13 +440,13 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_
         // While a slab is multiplied, the next one travels through registers to the other buffer (which every
         // wavefront has finished reading before the barrier that ended the previous round) and the W it will
         // meet is requested, a chunk as soon as the registers of one are free.  The last slab requests nothing.
-        for (; k0 + SPLIT_SLAB < k_last; k0 += SPLIT_SLAB, buffer ^= 1) {
-            load_slab(next, k0 + SPLIT_SLAB);
+        for (; k0 + SLAB < k_last; k0 += SLAB, buffer ^= 1) {
+            load_slab(next, k0 + SLAB);
             multiply_chunk(p, k0, staged + buffer * BUFFER, 0);
-            load_chunk(p, k0 + SPLIT_SLAB);
+            load_chunk(p, k0 + SLAB);
             multiply_chunk(q, k0 + HALF, staged + buffer * BUFFER, HALF);
-            load_chunk(q, k0 + SPLIT_SLAB + HALF);
-            store_slab(next, k0 + SPLIT_SLAB, staged + (buffer ^ 1) * BUFFER);
+            load_chunk(q, k0 + SLAB + HALF);
+            store_slab(next, k0 + SLAB, staged + (buffer ^ 1) * BUFFER);
             __syncthreads();
         }
         multiply_chunk(p, k0, staged + buffer * BUFFER, 0);
@@ -631,9 +633,9 @@ LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* h
 }
 
 // Partial sums that lsa_gemm_split writes for a size (the first dimension of its result), or -1 if it does not
-// take the size: 17 <= M <= 64, K a multiple of 8.
+// take the size: 17 <= M <= 128, K a multiple of 8.
 LSA_EXPORT int lsa_gemm_split_parts(int M, int N, int K) {
-    if (M <= 16 || M > 64 || N <= 0 || K < 8 || K % 8 != 0) return -1;
+    if (M <= 16 || M > SPLIT_MOST_ROWS || N <= 0 || K < 8 || K % 8 != 0) return -1;
     const int range = split_range(N, K);
     return (K + range - 1) / range;
 }
@@ -644,20 +646,24 @@ LSA_EXPORT int lsa_gemm_split(const void* x, const void* w, float* partial, int 
     if (lsa_gemm_split_parts(M, N, K) < 0 || !x || !w || !partial) return -1;
     const int range = split_range(N, K);
     const dim3 grid((N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS, (K + range - 1) / range), block(GEMM_WAVES * 64);
-#define LSA_SPLIT(MT)                                                                                                          \
+#define LSA_SPLIT(MT, SLAB)                                                                                                    \
     {                                                                                                                          \
         static bool sized = false;                                                                                             \
-        constexpr int bytes = 2 * 16 * MT * SPLIT_PITCH;                                                                       \
+        constexpr int bytes = 2 * 16 * MT * (2 * SLAB + 16);                                                                   \
         if (!sized) {                                                                                                          \
-            const hipError_t e = hipFuncSetAttribute((const void*)gemm_split_kernel<MT>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
+            const hipError_t e = hipFuncSetAttribute((const void*)gemm_split_kernel<MT, SLAB>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
             if (e != hipSuccess) return (int)e;                                                                                \
             sized = true;                                                                                                      \
         }                                                                                                                      \
-        gemm_split_kernel<MT><<<grid, block, bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, partial, M, N, K, range);    \
+        gemm_split_kernel<MT, SLAB><<<grid, block, bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, partial, M, N, K, range); \
     }
-    if (M <= 32) LSA_SPLIT(2)
-    else if (M <= 48) LSA_SPLIT(3)
-    else LSA_SPLIT(4)
+    // Slabs of 512 columns where two of them fit into LDS and the range is made of whole ones (a slab is loaded whole).
+    const bool wide = range % 512 == 0;
+    if (M <= 32) { if (wide) LSA_SPLIT(2, 512) else LSA_SPLIT(2, 256) }
+    else if (M <= 48) { if (wide) LSA_SPLIT(3, 512) else LSA_SPLIT(3, 256) }
+    else if (M <= 64) { if (wide) LSA_SPLIT(4, 512) else LSA_SPLIT(4, 256) }
+    else if (M <= 96) LSA_SPLIT(6, 256)
+    else LSA_SPLIT(8, 256)
 #undef LSA_SPLIT
     LSA_LAUNCH_CHECK();
 }

@@ -77,7 +77,7 @@ class HipOps:
         # Whether projections may fold the residual sum and the norm between two few-row products into their
         # epilogues (see linear_into_stream); off, every such sum and norm is a kernel of its own.
         self.fuse_stream_updates = True
-        # Whether projections whose result is added to the residual stream may leave it as partial sums at 17 to 64 rows.
+        # Whether projections whose result is added to the residual stream may leave it as partial sums at 17 to 128 rows.
         self.split_products = True
         self._split_parts = {}      # (rows, out, in) -> partial sums the split product writes for that size
 
@@ -150,10 +150,10 @@ class HipOps:
                                              int(rows_per_workgroup), sums, parts, eps, _stream()), "gemm_skinny")
         return out
 
-    SPLIT_ROWS = 64         # most rows the product that leaves partial sums takes (it starts above the few-row kernels')
+    SPLIT_ROWS = 128        # most rows the product that leaves partial sums takes (it starts above the few-row kernels')
 
     def linear_partial_sums(self, x, weight):
-        """``x @ weight^T`` for 17 to 64 rows as float32 partial sums ``[parts, T, out]`` over ranges of the inner
+        """``x @ weight^T`` for 17 to 128 rows as float32 partial sums ``[parts, T, out]`` over ranges of the inner
         dimension (their sum is the product), or None if this is no case for it.  Whoever adds the result to the
         residual stream adds the parts up (:meth:`add_rmsnorm` takes them)."""
         rows, width = x.shape

@@ -404,10 +404,10 @@ def test_skinny_gemm(ops, rows, n, k):
             raise RuntimeError("refused")
 
 
-@pytest.mark.parametrize("rows", [17, 31, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("rows", [17, 32, 33, 48, 49, 64, 65, 96, 97, 128])
 @pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (2050, 1000), (200, 5128), (8192, 64), (5120, 520), (127, 264)])
 def test_product_in_partial_sums(ops, rows, n, k):
-    """The product for 17 to 64 rows, which leaves partial sums over ranges of the inner dimension, against a float64
+    """The product for 17 to 128 rows, which leaves partial sums over ranges of the inner dimension, against a float64
     product of the same bfloat16 values: one range and many, ranges that end inside a staged slab, sizes that are no
     multiple of the tiles.  Then the kernel that adds them up, adds the result to a residual stream and normalises,
     against its twin."""
@@ -425,7 +425,7 @@ def test_product_in_partial_sums(ops, rows, n, k):
     assert (offered is None) == (parts < 2)                                               # nothing to split: left to the library
     if offered is not None:
         assert torch.equal(offered, sums)
-    for refused in (16, 65):
+    for refused in (16, 129):
         assert ops._gemm.lsa_gemm_split_parts(refused, n, k) == -1
     assert ops._gemm.lsa_gemm_split_parts(rows, n, k + 4) == -1
     resid = (2 * torch.randn(rows, n, device=DEV)).to(torch.bfloat16)

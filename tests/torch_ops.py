@@ -66,7 +66,7 @@ class TorchOps:
         return (gate * torch.sigmoid(gate) * up).to(x.dtype)
 
     def linear_partial_sums(self, x, weight):
-        if not self.fused or not 16 < x.shape[0] <= 64:
+        if not self.fused or not 16 < x.shape[0] <= 128:
             return None
         self.fused_calls["partial_sums"] += 1
         bounds = [0, x.shape[1] // 3, x.shape[1] // 2, x.shape[1]]                      # any split of the inner dimension
