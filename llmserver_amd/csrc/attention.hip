@@ -785,14 +785,15 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
 // Merge the partial slots of a tile: out = sum_s w_s acc_s / sum_s w_s l_s, w_s = exp(m_s - max m).
 struct Merge { int row, q0, first_slot, n_slots; };
 
-constexpr int MERGE_WAVES = 4;
+constexpr int MERGE_WAVES = 4;         // at most; the launch brings as many as the merges' slots can use
 
 __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
     elem_t* __restrict__ out, const int* __restrict__ row_start, const int* __restrict__ row_len,
     const Merge* __restrict__ merges, const float* __restrict__ part_acc, const float* __restrict__ part_ml, Geometry g) {
     // One block per (tile, KV head, pair).  First the slots' weights (a thread per slot), then the weighted sum:
-    // wavefront v takes slots v, v + 4, ... (four loads in flight each, so 64 slots are four trips to memory, not
-    // sixteen), a lane two neighbouring output dimensions, and the wavefronts' sums meet in LDS.
+    // with W wavefronts in the block, wavefront v takes slots v, v + W, ... (four loads in flight each, so 64 slots
+    // are four trips to memory for four wavefronts, not sixteen), a lane two neighbouring output dimensions, and the
+    // wavefronts' sums meet in LDS.
     constexpr int PAIRS = D / 2, PER_LANE = (PAIRS + 63) / 64;
     __shared__ float weight[64];
     __shared__ float inv_total;
@@ -804,7 +805,7 @@ __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
     if (pair_token >= g.tokens_per_tile || m.q0 + pair_token >= row_len[m.row] || pair_head_in_group >= g.group) return;
     const size_t stride = (size_t)gridDim.y * 16;                       // pairs per slot
     const size_t base = ((size_t)m.first_slot * gridDim.y + blockIdx.y) * 16 + col;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     if (wave == 0) {
         const int s = lane;
         float mx = NEG_INF, sum = 0.f;
@@ -831,26 +832,26 @@ __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
 #pragma unroll
     for (int i = 0; i < PER_LANE; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) first[i][j] = slot_values(wave + MERGE_WAVES * j, i);
+        for (int j = 0; j < 4; ++j) first[i][j] = slot_values(wave + waves * j, i);
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < PER_LANE; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int s = wave + MERGE_WAVES * j;
+            const int s = wave + waves * j;
             const float w = s < m.n_slots ? weight[s] : 0.f;
             total[i].x += w * first[i][j].x;
             total[i].y += w * first[i][j].y;
         }
-    for (int s0 = wave + 4 * MERGE_WAVES; s0 < m.n_slots; s0 += 4 * MERGE_WAVES) {
+    for (int s0 = wave + 4 * waves; s0 < m.n_slots; s0 += 4 * waves) {
 #pragma unroll
         for (int i = 0; i < PER_LANE; ++i) {
             float2 v[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = slot_values(s0 + MERGE_WAVES * j, i);
+            for (int j = 0; j < 4; ++j) v[j] = slot_values(s0 + waves * j, i);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int s = s0 + MERGE_WAVES * j;
+                const int s = s0 + waves * j;
                 const float w = s < m.n_slots ? weight[s] : 0.f;
                 total[i].x += w * v[j].x;
                 total[i].y += w * v[j].y;
@@ -872,7 +873,7 @@ __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
         if (pair >= PAIRS) continue;
         float2 sum = total[i];
 #pragma unroll
-        for (int v = 0; v < MERGE_WAVES - 1; ++v) {
+        for (int v = 0; v < waves - 1; ++v) {
             sum.x += wave_total[v][pair].x;
             sum.y += wave_total[v][pair].y;
         }
@@ -884,8 +885,8 @@ __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
 LSA_EXPORT int lsa_paged_attention(
     const void* q, long q_token_stride, void* out, const void* keys, const void* values, const int* table, int table_stride,
     const int* row_start, const int* row_len, const int* row_ctx, const void* items, const int* item_slot, int n_items,
-    const void* merges, int n_merges, float* part_acc, float* part_ml, const void* tiles, int n_tiles, float scale, int window,
-    int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
+    const void* merges, int n_merges, int n_slots, float* part_acc, float* part_ml, const void* tiles, int n_tiles, float scale,
+    int window, int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
     int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, int tiles_per_workgroup,
     hipStream_t stream) {
     if (n_items <= 0 && n_tiles <= 0) return 0;
@@ -924,7 +925,10 @@ LSA_EXPORT int lsa_paged_attention(
     int err = (int)hipGetLastError();
     if (err || n_merges <= 0) return err;
     dim3 mgrid(n_merges, n_kv * gtiles, 16);
-    merge_kernel<<<mgrid, MERGE_WAVES * 64, 0, stream>>>((elem_t*)out, row_start, row_len, (const Merge*)merges, part_acc, part_ml, g);
+    // A wavefront for every four slots of an average merge (the slots of a step's merges differ little).
+    const int wanted_waves = (n_slots / n_merges + 3) / 4;
+    const int merge_waves = wanted_waves < 1 ? 1 : wanted_waves > MERGE_WAVES ? MERGE_WAVES : wanted_waves;
+    merge_kernel<<<mgrid, merge_waves * 64, 0, stream>>>((elem_t*)out, row_start, row_len, (const Merge*)merges, part_acc, part_ml, g);
     LSA_LAUNCH_CHECK();
 }
 
