@@ -1,7 +1,9 @@
-// Weight-streaming matrix product for a few rows of activations (decode steps):
-//   Y[M, N] = X[M, K] . W[N, K]^T,  bfloat16 inputs, 32-bit accumulation, M <= 64.
+// Weight-streaming matrix products for a few rows of activations (decode steps, short portions):
+//   Y[M, N] = X[M, K] . W[N, K]^T,  bfloat16 inputs, 32-bit accumulation.
 // With so few rows the product is bound by reading W once from HBM, so the kernels are built
-// around that stream: a workgroup owns 16 (or 32) consecutive rows of W; its eight wavefronts
+// around that stream.  Two families: the one below for up to 16 rows (it runs up to 64, but is
+// beaten there), and further down one for 17 to 128 rows that leaves partial sums.
+// In the first, a workgroup owns 16 (or 32) consecutive rows of W; its eight wavefronts
 // split K between them, each streams its slice of the rows with 16-byte loads issued many at a
 // time, multiplies it with the matching slice of X (which stays in cache) on 16x16x32 MFMAs, and
 // the eight partial tiles are added through LDS and rounded once.
