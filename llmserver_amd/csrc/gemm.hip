@@ -648,14 +648,17 @@ LSA_EXPORT int lsa_gemm_split(const void* x, const void* w, float* partial, int 
     if (lsa_gemm_split_parts(M, N, K) < 0 || !x || !w || !partial) return -1;
     const int range = split_range(N, K);
     const dim3 grid((N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS, (K + range - 1) / range), block(GEMM_WAVES * 64);
+    // More LDS than a kernel gets by default: asked for once per kernel and device.
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -1;
 #define LSA_SPLIT(MT, SLAB)                                                                                                    \
     {                                                                                                                          \
-        static bool sized = false;                                                                                             \
+        static bool sized[64] = {};                                                                                            \
         constexpr int bytes = 2 * 16 * MT * (2 * SLAB + 16);                                                                   \
-        if (!sized) {                                                                                                          \
+        if (!sized[device]) {                                                                                                  \
             const hipError_t e = hipFuncSetAttribute((const void*)gemm_split_kernel<MT, SLAB>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
             if (e != hipSuccess) return (int)e;                                                                                \
-            sized = true;                                                                                                      \
+            sized[device] = true;                                                                                              \
         }                                                                                                                      \
         gemm_split_kernel<MT, SLAB><<<grid, block, bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, partial, M, N, K, range); \
     }
