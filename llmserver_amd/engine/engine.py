@@ -256,6 +256,36 @@ class Engine:
             self.preempt_request(victim)
 
     # -- one step ----------------------------------------------------------------------------
+    def warmup_graphs(self, batch_sizes=None) -> int:
+        """Capture the decode graph of these numbers of rows (default: every power of two up to ``max_batch_size``, and
+        that) before serving, so that the first steps of those sizes do not pay for it; an idle engine only.  Returns how
+        many graphs are held afterwards (/root/reference/utils/engine.py:150-161).  The graphs serve contexts up to the
+        first width of the block table; longer ones are captured when they are reached."""
+        if not self.runner.use_graphs or self.active_requests:
+            return 0
+        most = self.scheduler.max_batch_size
+        if batch_sizes is None:
+            batch_sizes = sorted({min(most, 1 << i) for i in range(most.bit_length() + 1)})
+        try:
+            for rows in batch_sizes:
+                if not 0 < rows <= most or rows > self.kv_cache.available_pages()[0]:
+                    continue
+                names = [f"warmup-{i}" for i in range(rows)]
+                try:
+                    for name in names:
+                        self.kv_cache.open(name)
+                    self.runner.step([StepEntry(name, [0], [0]) for name in names])      # one token each: the captured kind of step
+                finally:
+                    for name in names:
+                        if name in self.kv_cache.requests:
+                            self.kv_cache.close(name)
+        except Exception as error:               # as the reference: serving goes on, graphs are captured on first use
+            import warnings
+            warnings.warn(f"graph warm-up failed ({error!r}); graphs will be captured on first use")
+            self.runner.drop_graphs()
+            return 0
+        return self.runner.graph_count()
+
     def run_scheduled(self, out) -> None:
         """Turn the plan into one flat batch, run it, sample, and move every request on."""
         entries, sampled = [], []

@@ -147,6 +147,12 @@ class ModelRunner:
         self.graph_replays += 1
         return captured.logits
 
+    def graph_count(self) -> int:
+        return len(self._graphs)
+
+    def drop_graphs(self) -> None:
+        self._graphs.clear()
+
     @torch.inference_mode()
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run one step; returns float32 logits ``[wanted, vocab]`` in the order of the entries and their ``want``.

@@ -74,6 +74,30 @@ def test_small_budget_and_few_pages_give_the_same_tokens():
     assert min(tight.kv_cache.available_pages()) == 27
 
 
+def test_graphs_captured_ahead_change_nothing():
+    """Decode graphs captured before serving: all pages come back, and generation gives the tokens it gives without
+    (greedy, bfloat16, several requests at once so that the captured sizes are met)."""
+    from llmserver_amd import Engine, load_model
+    print("graphs captured ahead", flush=True)
+    case = "A"
+    raw, _, page = CASES[case]
+    prompts = [random_tokens(raw["vocab_size"], n, 80 + i) for i, n in enumerate((5, 17, 33, 9))]
+    model = load_model(model_folder(case), "cuda", "bfloat16")
+    def engine():
+        return Engine(model, None, max_new_tokens=10, max_batch_size=4, max_num_batched_tokens=64, kv_cache_num_blocks=40,
+                      kv_cache_block_size=page, ignore_eos=True)
+    plain_run = engine().generate(prompts)
+    warmed = engine()
+    assert warmed.warmup_graphs() == 3                                   # 1, 2 and 4 rows
+    assert min(warmed.kv_cache.available_pages()) == 40 and not warmed.kv_cache.requests
+    replays = warmed.runner.graph_replays
+    assert warmed.generate(prompts) == plain_run
+    assert warmed.runner.graph_replays > replays and warmed.runner.graph_count() == 3     # no further capture was needed
+    warmed.add_request(None, prompt_token_ids=[1, 2, 3])
+    assert warmed.warmup_graphs() == 0                                   # not while requests are live
+    warmed.kv_cache.check_invariants()
+
+
 def test_temperature_sampling_is_seeded_per_request():
     """Workload of tiny configuration B: temperature 0.8 with a fixed seed; a request's tokens do not
     depend on what shares its batch or on the token budget."""
