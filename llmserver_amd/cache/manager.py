@@ -36,13 +36,23 @@ class LayerCacheView:
     state: Optional[torch.Tensor] = None     # [slots, *shape] for a mixer with per-request state
 
 
+SCRATCH_PAGES = 16      # pages of storage beyond every pool (see CacheGroup.scratch_page)
+
+
 class CacheGroup:
     def __init__(self, index: int, spec: PagedKVSpec, caches: List[int], num_pages: int, page_size: int):
         self.index, self.spec, self.caches = index, spec, caches
         self.pool = PagePool(num_pages, page_size)
         self.page_size = page_size
-        self.keys = None     # [len(caches), pages, kv_heads, page_size, head_dim]
-        self.values = None   # [len(caches), pages, kv_heads, head_dim, page_size]
+        self.keys = None     # [len(caches), pages + SCRATCH_PAGES, kv_heads, page_size, head_dim]
+        self.values = None   # [len(caches), pages + SCRATCH_PAGES, kv_heads, head_dim, page_size]
+
+    def scratch_page(self, index: int) -> int:
+        """One of the pages behind the pool's, which no request ever holds: rows that a step adds to fill a captured
+        shape write there (each its own page), and nobody reads them."""
+        if not 0 <= index < SCRATCH_PAGES:
+            raise ValueError(f"scratch pages are 0..{SCRATCH_PAGES - 1}, asked for {index}")
+        return self.pool.num_pages + index
 
     def first_needed_block(self, num_computed: int) -> int:
         """First logical block a query at position >= num_computed can still see."""
@@ -96,7 +106,7 @@ class CacheManager:
     def _allocate_storage(self):
         for group in self.groups:
             spec, n = group.spec, len(group.caches)
-            pages = group.pool.num_pages
+            pages = group.pool.num_pages + SCRATCH_PAGES
             group.keys = torch.zeros((n, pages, spec.n_kv_heads, self.page_size, spec.head_dim), device=self.device, dtype=self.dtype)
             group.values = torch.zeros((n, pages, spec.n_kv_heads, spec.head_dim, self.page_size), device=self.device, dtype=self.dtype)
         for cache, spec in self.state_specs.items():

@@ -28,7 +28,7 @@ from .batch import StepEntry
 from .request import (STREAM_END, CompletedRequest, Request, RequestFinishReason, RequestStatus, SamplingParams,
                       TokenStream)
 from .scheduler import Scheduler
-from .step import ModelRunner
+from .step import ModelRunner, padded_rows
 
 
 def _read_generation_config(model) -> dict:
@@ -257,15 +257,16 @@ class Engine:
 
     # -- one step ----------------------------------------------------------------------------
     def warmup_graphs(self, batch_sizes=None) -> int:
-        """Capture the decode graph of these numbers of rows (default: every power of two up to ``max_batch_size``, and
-        that) before serving, so that the first steps of those sizes do not pay for it; an idle engine only.  Returns how
-        many graphs are held afterwards (/root/reference/utils/engine.py:150-161).  The graphs serve contexts up to the
-        first width of the block table; longer ones are captured when they are reached."""
+        """Capture the decode graphs of these numbers of rows (default: every size that decoding steps of up to
+        ``max_batch_size`` rows are filled up to) before serving, so that the first steps of those sizes do not pay for
+        it; an idle engine only.  Returns how many graphs are held afterwards
+        (/root/reference/utils/engine.py:150-161).  The graphs serve contexts up to the first width of the block
+        table; longer ones are captured when they are reached."""
         if not self.runner.use_graphs or self.active_requests:
             return 0
         most = self.scheduler.max_batch_size
         if batch_sizes is None:
-            batch_sizes = sorted({min(most, 1 << i) for i in range(most.bit_length() + 1)})
+            batch_sizes = sorted({min(most, padded_rows(rows)) for rows in range(1, most + 1)})
         try:
             for rows in batch_sizes:
                 if not 0 < rows <= most or rows > self.kv_cache.available_pages()[0]:

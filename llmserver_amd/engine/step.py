@@ -8,7 +8,8 @@ one pass, and one code path serves generation, the benchmark and trace replay.
 
 A step that brings one token per request is launch-bound, so it is captured once into a HIP
 graph per (rows, block-table width, wanted rows) and replayed afterwards: the kernels read
-everything that changes from the staged arrays, whose addresses and shapes stay the same.  The
+everything that changes from the staged arrays, whose addresses and shapes stay the same.  Decoding
+steps are filled up with rows of nobody's to one of a few sizes, so that few graphs serve every batch.  The
 reference replays its decode pass from a CUDA graph in the same way
 (/root/reference/utils/cuda_graph.py:51-99).
 """
@@ -25,7 +26,17 @@ from ..cache.manager import CacheManager
 from .batch import Staging, StepContext, StepEntry
 
 TABLE_WIDTH_STEP = 64      # captured steps serve block tables up to the next multiple of this many pages
-MAX_GRAPHS = 12
+MAX_GRAPHS = 24
+
+
+def padded_rows(rows: int) -> int:
+    """The number of rows a captured step of ``rows`` single tokens runs with: the next of 1, 2, 3, 4, 6, 8, ..., 16,
+    20, 24, ..., 32, 40, 48, ..., 64, 80, 96, ...  (at most a quarter more, never 16 more), so that requests that
+    come and go do not ask for a graph of every size."""
+    if rows <= 4:
+        return rows
+    step = 2 if rows <= 16 else 4 if rows <= 32 else 8 if rows <= 64 else 16
+    return -(-rows // step) * step
 
 
 class _CapturedStep:
@@ -51,8 +62,10 @@ class ModelRunner:
         self.graph_replays = 0
 
     def build_context(self, entries: Sequence[StepEntry], staging: Optional[Staging] = None,
-                      table_width: Optional[int] = None) -> StepContext:
-        """Check the entries against the cache, allocate their pages, lay out the flat batch."""
+                      table_width: Optional[int] = None, filler_rows: int = 0) -> StepContext:
+        """Check the entries against the cache, allocate their pages, lay out the flat batch.  ``filler_rows`` more rows
+        follow the entries', each a first token of nobody's on a scratch page of its own, its logits wanted: they
+        bring a step of single tokens to the shape of a captured one."""
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
@@ -85,16 +98,27 @@ class ModelRunner:
             token_row.extend([row] * len(tokens))
         for entry, ctx_len in zip(entries, row_ctx):
             self.cache.ensure(entry.request_id, ctx_len)
+        for filler in range(filler_rows):
+            logit_idx.append(len(token_ids))
+            row_start.append(len(token_ids))
+            row_len.append(1)
+            row_ctx.append(1)
+            token_row.append(len(entries) + filler)
+            token_ids.append(0)
+            positions.append(0)
         tables = []
         for group in self.cache.groups:
             width = max(1, max(len(self.cache.record(rid).tables[group.index]) for rid in request_ids))
             if table_width is not None:
                 width = table_width
-            table = np.full((len(entries), width), -1, dtype=np.int32)
+            table = np.full((len(entries) + filler_rows, width), -1, dtype=np.int32)
             for row, rid in enumerate(request_ids):
                 pages = self.cache.record(rid).tables[group.index]
                 table[row, :len(pages)] = pages
+            for filler in range(filler_rows):
+                table[len(entries) + filler, 0] = group.scratch_page(filler)
             tables.append(table)
+        request_ids = request_ids + [None] * filler_rows
         slots = None
         if self.cache.state_specs:
             slots = np.asarray([self.cache.record(rid).state_slot for rid in request_ids], dtype=np.int32)
@@ -116,12 +140,16 @@ class ModelRunner:
                 return None
             blocks = max(blocks, -(-(record.num_computed + 1) // self.cache.page_size))
         width = -(-blocks // TABLE_WIDTH_STEP) * TABLE_WIDTH_STEP
-        return (len(entries), width, sum(len(entry.want) for entry in entries))
+        rows, wanted = len(entries), sum(len(entry.want) for entry in entries)
+        if all(len(entry.want) == 1 for entry in entries):
+            rows = wanted = padded_rows(rows)          # decoding: filled up to one of a few sizes
+        return (rows, width, wanted)
 
     def _step_captured(self, entries, key) -> torch.Tensor:
         captured = self._graphs.get(key)
         staging = captured.staging if captured is not None else Staging(self.device, capacity=4096)
-        ctx = self.build_context(entries, staging=staging, table_width=key[1])
+        ctx = self.build_context(entries, staging=staging, table_width=key[1], filler_rows=key[0] - len(entries))
+        wanted = sum(len(entry.want) for entry in entries)           # the fillers' logits come last and are dropped
         ctx.static_max_keys = key[1] * self.cache.page_size
         self.model.prepare(ctx)
         if captured is None:
@@ -137,15 +165,15 @@ class ModelRunner:
             self._graphs[key] = _CapturedStep(graph, static_logits, ctx.layout, staging)
             while len(self._graphs) > MAX_GRAPHS:
                 self._graphs.popitem(last=False)
-            return logits
+            return logits[:wanted]
         self._graphs.move_to_end(key)
         ctx.upload()
         if ctx.layout != captured.layout:
             warnings.warn("a captured step met arrays of another shape; running it eagerly")
-            return self.model.forward(ctx, self.cache)
+            return self.model.forward(ctx, self.cache)[:wanted]
         captured.graph.replay()
         self.graph_replays += 1
-        return captured.logits
+        return captured.logits[:wanted]
 
     def graph_count(self) -> int:
         return len(self._graphs)

@@ -88,11 +88,11 @@ def test_graphs_captured_ahead_change_nothing():
                       kv_cache_block_size=page, ignore_eos=True)
     plain_run = engine().generate(prompts)
     warmed = engine()
-    assert warmed.warmup_graphs() == 3                                   # 1, 2 and 4 rows
+    assert warmed.warmup_graphs() == 4                                   # 1, 2, 3 and 4 rows
     assert min(warmed.kv_cache.available_pages()) == 40 and not warmed.kv_cache.requests
     replays = warmed.runner.graph_replays
     assert warmed.generate(prompts) == plain_run
-    assert warmed.runner.graph_replays > replays and warmed.runner.graph_count() == 3     # no further capture was needed
+    assert warmed.runner.graph_replays > replays and warmed.runner.graph_count() == 4     # no further capture was needed
     warmed.add_request(None, prompt_token_ids=[1, 2, 3])
     assert warmed.warmup_graphs() == 0                                   # not while requests are live
     warmed.kv_cache.check_invariants()

@@ -10,10 +10,12 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("case, n_live", [("A", 3), ("B", 3), ("B", 12), ("B", 24)])
+@pytest.mark.parametrize("case, n_live", [("A", 3), ("B", 3), ("B", 5), ("B", 12), ("B", 21), ("B", 24)])
 def test_replayed_steps_equal_eager_steps(case, n_live, dtype):
     """Three and twelve rows keep the products in the hand-written few-row kernels (one and two rows per
-    wavefront in their fused epilogues); twenty-four rows put the library's products inside the captured graph."""
+    wavefront in their fused epilogues); twenty-four rows put the library's products inside the captured graph; five
+    and twenty-one rows are filled up to six and twenty-four with rows of nobody's (and, every ninth turn, three and
+    eleven to three and twelve)."""
     from llmserver_amd.cache import CacheManager
     from llmserver_amd.engine import ModelRunner, StepEntry, load_model
     print(f"graph replay {case} {n_live} rows {dtype}", flush=True)
@@ -43,6 +45,7 @@ def test_replayed_steps_equal_eager_steps(case, n_live, dtype):
                 runner.step([StepEntry("tmp", random_tokens(raw["vocab_size"], 23, turn), [22])])
                 runner.cache.close("tmp")
     assert runners[0].graph_replays >= 60 and runners[1].graph_replays == 0
+    assert runners[0].graph_count() <= 3, list(runners[0]._graphs)     # both numbers of rows, and the prompt of one token
     assert worst <= (1e-5 if dtype == "float32" else 2e-2), worst
     for runner in runners:
         runner.cache.check_invariants()

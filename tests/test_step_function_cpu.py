@@ -97,3 +97,28 @@ def test_a_step_refuses_what_does_not_fit(tmp_path):
     assert runner.cache.record("a").num_computed == 0 and runner.cache.available_pages() == [4]
     out = runner.step([StepEntry("a", [1, 2, 3], [])])
     assert out.shape == (0, 256) and runner.cache.record("a").num_computed == 3
+
+
+def test_filler_rows_of_a_captured_shape(tmp_path):
+    """Decoding steps are filled up to one of a few numbers of rows; the rows added are first tokens of nobody's, each
+    on a scratch page of its own behind the pool, and the requests' own rows and pages are what they were."""
+    from llmserver_amd.engine import StepEntry
+    from llmserver_amd.engine.step import padded_rows
+    sizes = [padded_rows(rows) for rows in range(1, 200)]
+    assert all(rows <= size < rows + 16 and size <= max(rows + 1, rows * 5 // 4) for rows, size in zip(range(1, 200), sizes))
+    assert sizes == sorted(sizes) and len(set(sizes[:64])) == 18 and all(padded_rows(size) == size for size in sizes)
+    runner = make_runner(model_folder("A"), "float32", 256, 16, device="cpu", ops=TorchOps())
+    for name, n in (("a", 5), ("b", 20)):
+        runner.cache.open(name)
+        runner.step([StepEntry(name, list(range(1, n + 1)), [])])
+    entries = [StepEntry("a", [7], [0]), StepEntry("b", [9], [0])]
+    plain = runner.build_context(entries)
+    filled = runner.build_context(entries, filler_rows=3)
+    pool_pages = runner.cache.groups[0].pool.num_pages
+    assert filled.n_rows == 5 and filled.n_tokens == 5 and filled.n_out == 5
+    assert list(filled.h_row_ctx) == [6, 21, 1, 1, 1] and list(filled.h_row_len) == [1] * 5
+    table = filled.h_tables[0]
+    assert (table[:2, :plain.h_tables[0].shape[1]] == plain.h_tables[0]).all()
+    assert list(table[2:, 0]) == [pool_pages, pool_pages + 1, pool_pages + 2] and (table[2:, 1:] == -1).all()
+    assert runner.cache.groups[0].keys.shape[1] > pool_pages + 2
+    runner.cache.check_invariants()
