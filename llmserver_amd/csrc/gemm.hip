@@ -376,18 +376,22 @@ constexpr int SPLIT_TILE_ROWS = 16 * GEMM_WAVES;       // rows of W per workgrou
 constexpr int SPLIT_MOST_ROWS = 128;                    // most rows of X
 
 // SLAB: columns of X staged at a time (512 up to 64 rows, 256 beyond: two slabs have to fit into LDS).
-template <int MT, int SLAB>
+// GATED: W stacks a gate matrix on an up matrix ([N, K], gate rows first) and the result wanted is
+// silu(x . gate^T) * (x . up^T) in bfloat16, [M, N / 2]: four wavefronts take 64 gate rows, the other four the up rows
+// that belong to them, and the two halves meet in the epilogue; one range of K only (nothing is left to add up).
+template <int MT, int SLAB, bool GATED>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                                     float* __restrict__ partial, int M, int N, int K, int k_range) {
+                                                                     void* __restrict__ out, int M, int N, int K, int k_range) {
     constexpr int SPLIT_PITCH = SLAB * 2 + 16;          // bytes per staged row: 16 rows apart are 64 banks apart
     constexpr int SPLIT_CHUNK = SLAB / 64;              // k steps of W whose loads are issued together: half a slab
     extern __shared__ __attribute__((aligned(16))) unsigned char staged[];      // [2][16 MT][SPLIT_PITCH]
     constexpr int BUFFER = 16 * MT * SPLIT_PITCH;
     constexpr int PIECES = 16 * MT * (SLAB / 8) / (GEMM_WAVES * 64);      // 16-byte pieces of a slab per thread
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, quad = lane >> 4;
-    const int n0 = blockIdx.x * SPLIT_TILE_ROWS + 16 * wave;
+    const int n0 = GATED ? blockIdx.x * (SPLIT_TILE_ROWS / 2) + 16 * (wave & 3) : blockIdx.x * SPLIT_TILE_ROWS + 16 * wave;
     const int k_first = blockIdx.y * k_range, k_last = min(K, k_first + k_range);
-    const bf16_t* wp = w + (size_t)min(n0 + col, N - 1) * K + 8 * quad;
+    const int w_row = GATED ? (wave < 4 ? min(n0 + col, N / 2 - 1) : N / 2 + min(n0 + col, N / 2 - 1)) : min(n0 + col, N - 1);
+    const bf16_t* wp = w + (size_t)w_row * K + 8 * quad;
     const int k_safe = K - 8;
     f32x4 acc[MT];
 #pragma unroll
@@ -455,6 +459,32 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_
         multiply_chunk(q, k0 + HALF, staged + buffer * BUFFER, HALF);
     }
     // Lane (col, quad) holds Y[16 t + col][n0 + 4 quad .. + 4].
+    if (GATED) {
+        // The up halves go through LDS (the staged X is done with) to the wavefronts that hold their gate halves.
+        const int half = N / 2;
+        __syncthreads();
+        f32x4* exchange = reinterpret_cast<f32x4*>(staged);            // [4 wavefronts][MT][64 lanes]
+        if (wave >= 4) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) exchange[((wave - 4) * MT + t) * 64 + lane] = acc[t];
+        }
+        __syncthreads();
+        if (wave >= 4) return;
+        bf16_t* hidden = reinterpret_cast<bf16_t*>(out);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int m = 16 * t + col, n = n0 + 4 * quad;
+            const f32x4 up = exchange[(wave * MT + t) * 64 + lane];
+            if (m >= M) continue;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float gate = acc[t][r];
+                if (n + r < half) hidden[(size_t)m * half + n + r] = (bf16_t)(gate / (1.f + expf(-gate)) * up[r]);
+            }
+        }
+        return;
+    }
+    float* partial = reinterpret_cast<float*>(out);
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int m = 16 * t + col, n = n0 + 4 * quad;
@@ -470,10 +500,9 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_
     }
 }
 
-// Columns of X per workgroup (a multiple of 256) for a size: the one with which the compute units, working
+// Columns of X per workgroup (a multiple of 256) for `tiles` workgroups per range of K: the one with which the compute units, working
 // through the workgroups in rounds, are done soonest; a round costs its columns plus a fixed part.
-static int split_range(int N, int K) {
-    const long tiles = (N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS;
+static int split_range(long tiles, int K) {
     const int units = compute_units();
     const int whole = (K + 255) / 256 * 256;
     long best_cost = -1;
@@ -638,7 +667,7 @@ LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* h
 // take the size: 17 <= M <= 128, K a multiple of 8.
 LSA_EXPORT int lsa_gemm_split_parts(int M, int N, int K) {
     if (M <= 16 || M > SPLIT_MOST_ROWS || N <= 0 || K < 8 || K % 8 != 0) return -1;
-    const int range = split_range(N, K);
+    const int range = split_range((N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS, K);
     return (K + range - 1) / range;
 }
 
@@ -646,29 +675,55 @@ LSA_EXPORT int lsa_gemm_split_parts(int M, int N, int K) {
 // their sum over the first dimension is the product.
 LSA_EXPORT int lsa_gemm_split(const void* x, const void* w, float* partial, int M, int N, int K, hipStream_t stream) {
     if (lsa_gemm_split_parts(M, N, K) < 0 || !x || !w || !partial) return -1;
-    const int range = split_range(N, K);
+    const int range = split_range((N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS, K);
     const dim3 grid((N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS, (K + range - 1) / range), block(GEMM_WAVES * 64);
     // More LDS than a kernel gets by default: asked for once per kernel and device.
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -1;
-#define LSA_SPLIT(MT, SLAB)                                                                                                    \
+#define LSA_SPLIT(MT, SLAB, GATED)                                                                                             \
     {                                                                                                                          \
         static bool sized[64] = {};                                                                                            \
         constexpr int bytes = 2 * 16 * MT * (2 * SLAB + 16);                                                                   \
         if (!sized[device]) {                                                                                                  \
-            const hipError_t e = hipFuncSetAttribute((const void*)gemm_split_kernel<MT, SLAB>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); \
+            const hipError_t e = hipFuncSetAttribute((const void*)gemm_split_kernel<MT, SLAB, GATED>,                          \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, bytes);                       \
             if (e != hipSuccess) return (int)e;                                                                                \
             sized[device] = true;                                                                                              \
         }                                                                                                                      \
-        gemm_split_kernel<MT, SLAB><<<grid, block, bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, partial, M, N, K, range); \
+        gemm_split_kernel<MT, SLAB, GATED><<<grid, block, bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, range); \
     }
     // Slabs of 512 columns where two of them fit into LDS and the range is made of whole ones (a slab is loaded whole).
     const bool wide = range % 512 == 0;
-    if (M <= 32) { if (wide) LSA_SPLIT(2, 512) else LSA_SPLIT(2, 256) }
-    else if (M <= 48) { if (wide) LSA_SPLIT(3, 512) else LSA_SPLIT(3, 256) }
-    else if (M <= 64) { if (wide) LSA_SPLIT(4, 512) else LSA_SPLIT(4, 256) }
-    else if (M <= 96) LSA_SPLIT(6, 256)
-    else LSA_SPLIT(8, 256)
+    void* out = partial;
+    if (M <= 32) { if (wide) LSA_SPLIT(2, 512, false) else LSA_SPLIT(2, 256, false) }
+    else if (M <= 48) { if (wide) LSA_SPLIT(3, 512, false) else LSA_SPLIT(3, 256, false) }
+    else if (M <= 64) { if (wide) LSA_SPLIT(4, 512, false) else LSA_SPLIT(4, 256, false) }
+    else if (M <= 96) LSA_SPLIT(6, 256, false)
+    else LSA_SPLIT(8, 256, false)
+    LSA_LAUNCH_CHECK();
+}
+
+constexpr int SPLIT_GATED_MOST_ROWS = 32;     // beyond, the library's product and the activation kernel are faster (measured)
+
+// Whether lsa_gemm_split_gated takes a size: 17 <= M <= 32, K a multiple of 8, and so many pairs of a gate and an up
+// row that one range of K per workgroup fills the chip in one round (with ranges to add up there is no result to
+// activate; with more rounds than one the library is faster: measured 118 against 104 us at 400 workgroups).
+LSA_EXPORT int lsa_gemm_split_gated_fits(int M, int I, int K) {
+    if (M <= 16 || M > SPLIT_GATED_MOST_ROWS || I <= 0 || K < 8 || K % 8 != 0) return 0;
+    const long tiles = (I + SPLIT_TILE_ROWS / 2 - 1) / (SPLIT_TILE_ROWS / 2);
+    return tiles <= compute_units() && split_range(tiles, K) >= K ? 1 : 0;
+}
+
+// hidden [M, I] = silu(x . gate^T) * (x . up^T) in bfloat16, gate_up [2 I, K] with the gate rows first.
+LSA_EXPORT int lsa_gemm_split_gated(const void* x, const void* w, void* hidden, int M, int I, int K, hipStream_t stream) {
+    if (!lsa_gemm_split_gated_fits(M, I, K) || !x || !w || !hidden) return -1;
+    const int N = 2 * I, range = (K + 255) / 256 * 256;
+    const dim3 grid((I + SPLIT_TILE_ROWS / 2 - 1) / (SPLIT_TILE_ROWS / 2), 1), block(GEMM_WAVES * 64);
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -1;
+    void* out = hidden;
+    const bool wide = range % 512 == 0;
+    if (wide) LSA_SPLIT(2, 512, true) else LSA_SPLIT(2, 256, true)
 #undef LSA_SPLIT
     LSA_LAUNCH_CHECK();
 }

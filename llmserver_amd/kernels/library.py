@@ -30,6 +30,8 @@ _SIGNATURES = {
     "lsa_gemm_skinny_gated": [_P, _P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P],
     "lsa_gemm_split_parts": [c_int, c_int, c_int],
     "lsa_gemm_split": [_P, _P, _P, c_int, c_int, c_int, _P],
+    "lsa_gemm_split_gated_fits": [c_int, c_int, c_int],
+    "lsa_gemm_split_gated": [_P, _P, _P, c_int, c_int, c_int, _P],
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

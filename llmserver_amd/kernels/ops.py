@@ -206,6 +206,8 @@ class HipOps:
         ``row_scale`` as in :meth:`linear_few_rows`."""
         rows, width = x.shape
         inter = gate_up_weight.shape[0] // 2
+        if rows > self.skinny_rows:
+            return self._linear_gated_beyond_few_rows(x, gate_up_weight) if row_scale is None and pairs_per_workgroup == 0 else None
         if not self._few_rows(x, gate_up_weight) or inter % 8 or gate_up_weight.shape[1] != width or rows > 16 \
                 or not self._row_scale_fits(row_scale, rows):
             return None
@@ -215,6 +217,26 @@ class HipOps:
         sums, parts, eps = self._row_scale_args(row_scale, rows)
         _launched(self._gemm.lsa_gemm_skinny_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, int(pairs_per_workgroup), sums, parts,
                                                    eps, _stream()), "gemm_skinny_gated")
+        return out
+
+    def _linear_gated_beyond_few_rows(self, x, gate_up_weight):
+        """The same for 17 to 32 rows where the weight has so many rows that one workgroup can take the whole inner
+        dimension (the kernel of :meth:`linear_partial_sums` with the activation in its epilogue), else None."""
+        rows, width = x.shape
+        inter = gate_up_weight.shape[0] // 2
+        if x.dtype != torch.bfloat16 or gate_up_weight.dtype != torch.bfloat16 or gate_up_weight.shape[1] != width \
+                or gate_up_weight.shape[0] % 2 or not self.split_products:
+            return None
+        size = ("gated", rows, inter, width)
+        fits = self._split_parts.get(size)
+        if fits is None:
+            fits = self._split_parts[size] = self._gemm.lsa_gemm_split_gated_fits(rows, inter, width)
+        if not fits:
+            return None
+        _check(x, "x", torch.bfloat16)
+        _check(gate_up_weight, "gate_up_weight", torch.bfloat16)
+        out = torch.empty((rows, inter), device=x.device, dtype=torch.bfloat16)
+        _launched(self._gemm.lsa_gemm_split_gated(_ptr(x), _ptr(gate_up_weight), _ptr(out), rows, inter, width, _stream()), "gemm_split_gated")
         return out
 
     # -- hand-written kernels ----------------------------------------------------------------

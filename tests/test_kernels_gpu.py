@@ -535,4 +535,27 @@ def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
         torch.testing.assert_close(got.float(), expected, atol=2e-2, rtol=2e-2)
         got = ops.linear_gated(x, w, pairs_per_workgroup=per, row_scale=(square_sums, 1e-6))
         torch.testing.assert_close(got.float(), scaled, atol=2e-2, rtol=2e-2)
-    assert ops.linear_gated(torch.zeros(17, k, device=DEV, dtype=torch.bfloat16), w) is None
+    assert ops.linear_gated(torch.zeros(17, k, device=DEV, dtype=torch.bfloat16), w, row_scale=(torch.ones(17, 4, device=DEV), 1e-6)) is None
+
+
+@pytest.mark.parametrize("rows", [17, 24, 32, 33])
+@pytest.mark.parametrize("inter, k", [(12288, 4096), (9000, 264), (10001, 72), (16384, 1000), (20000, 1000), (8192, 512), (1000, 1000)])
+def test_gated_product_beyond_few_rows(ops, rows, inter, k):
+    """17 to 32 rows: the product that shares the activations through LDS, with the activation in its epilogue, where
+    the weight has rows enough for one workgroup to take the whole inner dimension, and not more than one round of
+    workgroups; elsewhere it is not offered."""
+    print(f"gated product beyond few rows {rows} inter {inter} k {k}", flush=True)
+    torch.manual_seed(rows + inter + k)
+    x = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
+    got = ops.linear_gated(x, w)
+    offered = bool(ops._gemm.lsa_gemm_split_gated_fits(rows, inter, k))
+    assert offered == (rows <= 32 and 8192 < inter <= 16384)      # tiles of 64 pairs: more than half the compute units, not more than all
+    assert (got is not None) == offered
+    if got is not None:
+        gate_up = x.double() @ w.double().t()
+        expected = (torch.nn.functional.silu(gate_up[:, :inter]) * gate_up[:, inter:]).float()
+        assert got.shape == (rows, inter) and got.dtype == torch.bfloat16
+        torch.testing.assert_close(got.float(), expected, atol=2e-2, rtol=2e-2)
+    assert ops.linear_gated(torch.zeros(49, k, device=DEV, dtype=torch.bfloat16), w) is None
+    assert ops._gemm.lsa_gemm_split_gated(x.data_ptr(), w.data_ptr(), x.data_ptr(), 16, inter, k, None) == -1

@@ -57,7 +57,8 @@ class TorchOps:
         return stream, weighted, parts
 
     def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None):
-        if not self.row_scale_fits(x, gate_up_weight, row_scale):
+        beyond = self.fused and row_scale is None and 16 < x.shape[0] <= 32            # the kernel for more rows has no row scale
+        if not beyond and not self.row_scale_fits(x, gate_up_weight, row_scale):
             return None
         self.fused_calls["gated"] += 1
         gate_up = self._scaled(x.float() @ gate_up_weight.float().t(), row_scale, x.shape[1])
