@@ -80,6 +80,13 @@ class HipOps:
         # Whether projections whose result is added to the residual stream may leave it as partial sums at 17 to 128 rows.
         self.split_products = True
         self._split_parts = {}      # (rows, out, in) -> partial sums the split product writes for that size
+        # The few-row products win on most shapes but not on all (on Qwen3-32B's gate/up the library is a third faster):
+        # the first time a size is met outside a graph capture, the few-row kernel is timed against the library's
+        # product plus the kernels it would have absorbed, and the faster is kept for that size.
+        self.choose_by_measurement = True
+        self._library_faster = {}   # (kind, rows, out, in, scaled, float32 result) -> bool
+        self._flush = None
+        self._replay_overhead = None
 
     @staticmethod
     def required_modules(head_dims, dtype):
@@ -99,6 +106,88 @@ class HipOps:
         rows, width = x.shape
         return x.dtype == torch.bfloat16 and 0 < rows <= self.skinny_rows and width % 8 == 0 and width >= 8 \
             and weight.dtype == torch.bfloat16
+
+    LIBRARY_MARGIN = 0.93       # the library replaces a few-row kernel only if it takes less than this share of its time
+
+    def _median_time(self, run, repeats=5):
+        """Milliseconds of ``run()``, replayed from a graph of its own (several launches then follow one another as
+        they do in a captured step, with no host between them), weights cold (a buffer larger than the caches is
+        read before every replay)."""
+        if self._flush is None:
+            self._flush = torch.zeros(96 << 20, device="cuda", dtype=torch.int32)
+        run()                                             # loads what the first call of a kernel loads
+        current = torch.cuda.current_stream()
+        side = torch.cuda.Stream()
+        side.wait_stream(current)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            graph.capture_begin()
+            run()
+            graph.capture_end()
+        current.wait_stream(side)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        times = []
+        for _ in range(repeats):
+            self._flush.sum()
+            start.record()
+            graph.replay()
+            end.record()
+            end.synchronize()
+            times.append(start.elapsed_time(end))
+        return sorted(times)[repeats // 2]
+
+    def _replay_cost(self):
+        """What a replay takes between its events beside its kernels (milliseconds): a replay of next to nothing."""
+        if self._replay_overhead is None:
+            cell = torch.zeros(1, device="cuda")
+            self._replay_overhead = self._median_time(lambda: cell.zero_(), repeats=7)
+        return self._replay_overhead
+
+    def library_is_faster(self, kind, x, weight, scaled=False, out_float32=False) -> bool:
+        """Whether, for these sizes, the library's product (with a norm kernel before it if ``scaled``, and the
+        activation kernel after it if ``kind`` is "gated") beats the few-row kernel that does it all; measured once."""
+        if not self.choose_by_measurement:
+            return False
+        rows, width = x.shape
+        key = (kind, rows, weight.shape[0], width, bool(scaled), bool(out_float32))
+        known = self._library_faster.get(key)
+        if known is not None:
+            return known
+        if torch.cuda.is_current_stream_capturing():
+            return False                                  # nothing can be timed while a graph is recorded
+        sums = torch.ones((rows, 16), device=x.device, dtype=torch.float32) if scaled else None
+        row_scale = (sums, 1e-6) if scaled else None
+        stream = torch.zeros_like(x) if scaled else None
+        norm_weight = torch.ones(width, device=x.device, dtype=torch.float32) if scaled else None
+        normed = torch.empty_like(x) if scaled else None
+        saved, self.choose_by_measurement = self.choose_by_measurement, False
+        try:
+            if kind == "gated":
+                hidden = torch.empty((rows, weight.shape[0] // 2), device=x.device, dtype=x.dtype)
+
+                def few():
+                    return self.linear_gated(x, weight, row_scale=row_scale)
+
+                def library():
+                    if scaled:
+                        self.add_rmsnorm(stream, None, norm_weight, 1e-6, normed)
+                    self.swiglu(torch.mm(x, weight.t()), hidden)
+            else:
+                def few():
+                    return self.linear_few_rows(x, weight, out_float32=out_float32, row_scale=row_scale)
+
+                def library():
+                    if scaled:
+                        self.add_rmsnorm(stream, None, norm_weight, 1e-6, normed)
+                    return torch.mm(x, weight.t(), out_dtype=torch.float32) if out_float32 else torch.mm(x, weight.t())
+            if few() is None:
+                return False                              # no case for the few-row kernel: nothing to choose
+            overhead = self._replay_cost()
+            faster = self._median_time(library) - overhead < self.LIBRARY_MARGIN * (self._median_time(few) - overhead)
+        finally:
+            self.choose_by_measurement = saved
+        self._library_faster[key] = faster
+        return faster
 
     def _row_scale_args(self, row_scale, rows):
         """``row_scale = (square_sums [rows, P] float32, eps)`` or None -> kernel arguments."""
@@ -123,7 +212,7 @@ class HipOps:
         fixes the few-row kernel's share of the weight per workgroup (1 to 32; 0 lets the size decide)."""
         if x.shape[1] != weight.shape[1]:
             raise ValueError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
-        if self._few_rows(x, weight):
+        if self._few_rows(x, weight) and (rows_per_workgroup or not self.library_is_faster("plain", x, weight, False, out_float32)):
             # Few rows: the product is a stream over the weights; the hand-written kernel reads them once at HBM rate.
             return self.linear_few_rows(x, weight, out=out, out_float32=out_float32, rows_per_workgroup=rows_per_workgroup)
         if out_float32 and x.dtype != torch.float32:
@@ -210,6 +299,8 @@ class HipOps:
             return self._linear_gated_beyond_few_rows(x, gate_up_weight) if row_scale is None and pairs_per_workgroup == 0 else None
         if not self._few_rows(x, gate_up_weight) or inter % 8 or gate_up_weight.shape[1] != width or rows > 16 \
                 or not self._row_scale_fits(row_scale, rows):
+            return None
+        if pairs_per_workgroup == 0 and self.library_is_faster("gated", x, gate_up_weight, row_scale is not None):
             return None
         _check(x, "x", torch.bfloat16)
         _check(gate_up_weight, "gate_up_weight", torch.bfloat16)

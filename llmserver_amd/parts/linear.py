@@ -70,7 +70,9 @@ class Linear(Part):
         row_scale = None
         if isinstance(x, PendingNorm):
             scaled = x.row_scale() if fused else None
-            if scaled is not None and ops.row_scale_fits(scaled[0], self.weight, scaled[1]):
+            library_is_faster = getattr(ops, "library_is_faster", None)
+            if scaled is not None and ops.row_scale_fits(scaled[0], self.weight, scaled[1]) and not (
+                    library_is_faster is not None and library_is_faster("plain", scaled[0], self.weight, True, self.out_float32)):
                 x, row_scale = scaled            # the norm becomes a scale of the product's rows
             else:
                 x = x.tensor()
