@@ -664,9 +664,10 @@ LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* h
 }
 
 // Partial sums that lsa_gemm_split writes for a size (the first dimension of its result), or -1 if it does not
-// take the size: 17 <= M <= 128, K a multiple of 8.
+// take the size: M <= 128 (it is made for 17 and more, but on some shapes it beats the few-row kernel from 9 on),
+// K a multiple of 8.
 LSA_EXPORT int lsa_gemm_split_parts(int M, int N, int K) {
-    if (M <= 16 || M > SPLIT_MOST_ROWS || N <= 0 || K < 8 || K % 8 != 0) return -1;
+    if (M < 1 || M > SPLIT_MOST_ROWS || N <= 0 || K < 8 || K % 8 != 0) return -1;
     const int range = split_range((N + SPLIT_TILE_ROWS - 1) / SPLIT_TILE_ROWS, K);
     return (K + range - 1) / range;
 }

@@ -189,6 +189,40 @@ class HipOps:
         self._library_faster[key] = faster
         return faster
 
+    def partial_sums_are_faster(self, x, weight) -> bool:
+        """For a projection of few rows into the residual stream: whether the product in partial sums plus the kernel
+        that adds them up and normalises beats the few-row kernel that does it all (long inner dimensions at 9 to 16
+        rows, where every workgroup of the few-row kernel moves as many activations as weights); measured once."""
+        rows, width = x.shape
+        if not self.choose_by_measurement or not self.split_products or not self.fuse_stream_updates \
+                or not 8 < rows <= self.skinny_rows or not self._few_rows(x, weight):
+            return False
+        key = ("stream", rows, weight.shape[0], width, False, False)
+        known = self._library_faster.get(key)
+        if known is not None:
+            return known
+        if torch.cuda.is_current_stream_capturing():
+            return False
+        resid = torch.zeros((rows, weight.shape[0]), device=x.device, dtype=x.dtype)
+        norm_weight = torch.ones(weight.shape[0], device=x.device, dtype=torch.float32)
+        normed = torch.empty_like(resid)
+        saved, self.choose_by_measurement = self.choose_by_measurement, False
+        try:
+            def few():
+                return self.linear_into_stream(x, weight, resid, norm_weight)
+
+            def split():
+                self.add_rmsnorm(resid, self.linear_partial_sums(x, weight, few_rows_too=True), norm_weight, 1e-6, normed)
+            if few() is None or self.linear_partial_sums(x, weight, few_rows_too=True) is None:
+                faster = False
+            else:
+                overhead = self._replay_cost()
+                faster = self._median_time(split) - overhead < self.LIBRARY_MARGIN * (self._median_time(few) - overhead)
+        finally:
+            self.choose_by_measurement = saved
+        self._library_faster[key] = faster
+        return faster
+
     def _row_scale_args(self, row_scale, rows):
         """``row_scale = (square_sums [rows, P] float32, eps)`` or None -> kernel arguments."""
         if row_scale is None:
@@ -241,12 +275,12 @@ class HipOps:
 
     SPLIT_ROWS = 128        # most rows the product that leaves partial sums takes (it starts above the few-row kernels')
 
-    def linear_partial_sums(self, x, weight):
-        """``x @ weight^T`` for 17 to 128 rows as float32 partial sums ``[parts, T, out]`` over ranges of the inner
-        dimension (their sum is the product), or None if this is no case for it.  Whoever adds the result to the
-        residual stream adds the parts up (:meth:`add_rmsnorm` takes them)."""
+    def linear_partial_sums(self, x, weight, few_rows_too=False):
+        """``x @ weight^T`` for 17 to 128 rows (fewer if ``few_rows_too``) as float32 partial sums ``[parts, T, out]``
+        over ranges of the inner dimension (their sum is the product), or None if this is no case for it.  Whoever
+        adds the result to the residual stream adds the parts up (:meth:`add_rmsnorm` takes them)."""
         rows, width = x.shape
-        if not (self.skinny_rows < rows <= self.SPLIT_ROWS) or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
+        if not ((0 if few_rows_too else self.skinny_rows) < rows <= self.SPLIT_ROWS) or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
                 or x.shape[1] != weight.shape[1] or not self.split_products:
             return None
         size = (rows, weight.shape[0], width)

@@ -78,13 +78,18 @@ class Linear(Part):
                 x = x.tensor()
         if sink is not None and fused and self.bias is None and not self.out_float32 \
                 and getattr(sink.norm, "weight", None) is not None and hasattr(sink.norm, "eps"):
-            done = ops.linear_into_stream(x, self.weight, sink.stream(), sink.norm.weight, row_scale=row_scale)
-            if done is not None:
-                return StreamUpdate(sink.norm, *done)
-            # More rows: the product may leave its result as partial sums, which the kernel of the sum and the
-            # norm adds up on its way.
+            # The product may leave its result as partial sums, which the kernel of the sum and the norm adds up on
+            # its way: that is the way of 17 rows and more, and of fewer where it has been measured to be faster.
             partial_sums = getattr(ops, "linear_partial_sums", None)
-            sums = partial_sums(x, self.weight) if partial_sums is not None and row_scale is None else None
+            split_few_rows = partial_sums is not None and row_scale is None and getattr(ops, "partial_sums_are_faster", None) is not None \
+                and ops.partial_sums_are_faster(x, self.weight)
+            if not split_few_rows:
+                done = ops.linear_into_stream(x, self.weight, sink.stream(), sink.norm.weight, row_scale=row_scale)
+                if done is not None:
+                    return StreamUpdate(sink.norm, *done)
+            sums = None
+            if partial_sums is not None and row_scale is None:
+                sums = partial_sums(x, self.weight, few_rows_too=True) if split_few_rows else partial_sums(x, self.weight)
             if sums is not None:
                 stream = sink.stream()
                 return StreamUpdate(sink.norm, stream, normed=sink.norm.add_norm(stream, sums, ctx))

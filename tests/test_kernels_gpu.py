@@ -409,7 +409,7 @@ def test_skinny_gemm(ops, rows, n, k):
             raise RuntimeError("refused")
 
 
-@pytest.mark.parametrize("rows", [17, 32, 33, 48, 49, 64, 65, 96, 97, 128])
+@pytest.mark.parametrize("rows", [9, 16, 17, 32, 33, 48, 49, 64, 65, 96, 97, 128])
 @pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (2050, 1000), (200, 5128), (8192, 64), (5120, 520), (127, 264)])
 def test_product_in_partial_sums(ops, rows, n, k):
     """The product for 17 to 128 rows, which leaves partial sums over ranges of the inner dimension, against a float64
@@ -426,11 +426,11 @@ def test_product_in_partial_sums(ops, rows, n, k):
     sums = torch.full((parts, rows, n), float("nan"), device=DEV)                          # every element must be written
     assert ops._gemm.lsa_gemm_split(x.data_ptr(), w.data_ptr(), sums.data_ptr(), rows, n, k, None) == 0
     torch.testing.assert_close(sums.sum(0), expected, atol=2e-4, rtol=1e-4)
-    offered = ops.linear_partial_sums(x, w)
+    offered = ops.linear_partial_sums(x, w, few_rows_too=True)
     assert (offered is None) == (parts < 2)                                               # nothing to split: left to the library
     if offered is not None:
         assert torch.equal(offered, sums)
-    for refused in (16, 129):
+    for refused in (0, 129):
         assert ops._gemm.lsa_gemm_split_parts(refused, n, k) == -1
     assert ops._gemm.lsa_gemm_split_parts(rows, n, k + 4) == -1
     resid = (2 * torch.randn(rows, n, device=DEV)).to(torch.bfloat16)

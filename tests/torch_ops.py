@@ -66,8 +66,8 @@ class TorchOps:
         gate, up = gate_up[:, :inter], gate_up[:, inter:]
         return (gate * torch.sigmoid(gate) * up).to(x.dtype)
 
-    def linear_partial_sums(self, x, weight):
-        if not self.fused or not 16 < x.shape[0] <= 128:
+    def linear_partial_sums(self, x, weight, few_rows_too=False):
+        if not self.fused or not (0 if few_rows_too else 16) < x.shape[0] <= 128:
             return None
         self.fused_calls["partial_sums"] += 1
         bounds = [0, x.shape[1] // 3, x.shape[1] // 2, x.shape[1]]                      # any split of the inner dimension
