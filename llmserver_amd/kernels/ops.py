@@ -122,8 +122,10 @@ class HipOps:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(side):
             graph.capture_begin()
-            run()
-            graph.capture_end()
+            try:
+                run()
+            finally:
+                graph.capture_end()                       # whatever happened, the stream must not stay in capture
         current.wait_stream(side)
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         times = []
@@ -135,6 +137,16 @@ class HipOps:
             end.synchronize()
             times.append(start.elapsed_time(end))
         return sorted(times)[repeats // 2]
+
+    def _second_is_faster(self, first, second) -> bool:
+        """Times both; a measurement that fails (something that cannot be recorded into a graph) keeps the first."""
+        try:
+            overhead = self._replay_cost()
+            return self._median_time(second) - overhead < self.LIBRARY_MARGIN * (self._median_time(first) - overhead)
+        except RuntimeError as error:
+            import warnings
+            warnings.warn(f"timing two ways of a product failed ({error!r}); keeping the few-row kernel")
+            return False
 
     def _replay_cost(self):
         """What a replay takes between its events beside its kernels (milliseconds): a replay of next to nothing."""
@@ -182,8 +194,7 @@ class HipOps:
                     return torch.mm(x, weight.t(), out_dtype=torch.float32) if out_float32 else torch.mm(x, weight.t())
             if few() is None:
                 return False                              # no case for the few-row kernel: nothing to choose
-            overhead = self._replay_cost()
-            faster = self._median_time(library) - overhead < self.LIBRARY_MARGIN * (self._median_time(few) - overhead)
+            faster = self._second_is_faster(few, library)
         finally:
             self.choose_by_measurement = saved
         self._library_faster[key] = faster
@@ -216,8 +227,7 @@ class HipOps:
             if few() is None or self.linear_partial_sums(x, weight, few_rows_too=True) is None:
                 faster = False
             else:
-                overhead = self._replay_cost()
-                faster = self._median_time(split) - overhead < self.LIBRARY_MARGIN * (self._median_time(few) - overhead)
+                faster = self._second_is_faster(few, split)
         finally:
             self.choose_by_measurement = saved
         self._library_faster[key] = faster
