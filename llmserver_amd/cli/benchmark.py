@@ -32,6 +32,8 @@ RANDOM_CONFIGS = {
                        intermediate_size=6144, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=True),
     "qwen3-8b": dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
                      intermediate_size=12288, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
+    "qwen3-14b": dict(num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, head_dim=128,
+                      intermediate_size=17408, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
     "qwen3-32b": dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
                       intermediate_size=25600, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
 }
