@@ -786,6 +786,7 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
 struct Merge { int row, q0, first_slot, n_slots; };
 
 constexpr int MERGE_WAVES = 4;         // at most; the launch brings as many as the merges' slots can use
+constexpr int MERGE_MOST_SLOTS = 128;  // key ranges one tile may be split into (two slots' weights per lane of a wavefront)
 
 __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
     elem_t* __restrict__ out, const int* __restrict__ row_start, const int* __restrict__ row_len,
@@ -795,7 +796,7 @@ __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
     // are four trips to memory for four wavefronts, not sixteen), a lane two neighbouring output dimensions, and the
     // wavefronts' sums meet in LDS.
     constexpr int PAIRS = D / 2, PER_LANE = (PAIRS + 63) / 64;
-    __shared__ float weight[64];
+    __shared__ float weight[MERGE_MOST_SLOTS];
     __shared__ float inv_total;
     __shared__ float2 wave_total[MERGE_WAVES - 1][PAIRS];
     const Merge m = merges[blockIdx.x];
@@ -807,17 +808,29 @@ __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
     const size_t base = ((size_t)m.first_slot * gridDim.y + blockIdx.y) * 16 + col;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     if (wave == 0) {
-        const int s = lane;
-        float mx = NEG_INF, sum = 0.f;
-        if (s < m.n_slots) {
-            mx = part_ml[(base + s * stride) * 2];
-            sum = part_ml[(base + s * stride) * 2 + 1];
+        float mx[MERGE_MOST_SLOTS / 64], sum[MERGE_MOST_SLOTS / 64];
+        float top = NEG_INF;
+#pragma unroll
+        for (int i = 0; i < MERGE_MOST_SLOTS / 64; ++i) {
+            const int s = lane + 64 * i;
+            mx[i] = NEG_INF;
+            sum[i] = 0.f;
+            if (s < m.n_slots) {
+                mx[i] = part_ml[(base + s * stride) * 2];
+                sum[i] = part_ml[(base + s * stride) * 2 + 1];
+            }
+            top = fmaxf(top, mx[i]);
         }
-        const float top = wave_max(mx);
-        const float w = mx == NEG_INF ? 0.f : expf(mx - top);
-        weight[s] = w;
-        const float total = wave_sum(w * sum);
-        if (s == 0) inv_total = total > 0.f ? 1.f / total : 0.f;
+        top = wave_max(top);
+        float weighted = 0.f;
+#pragma unroll
+        for (int i = 0; i < MERGE_MOST_SLOTS / 64; ++i) {
+            const float w = mx[i] == NEG_INF ? 0.f : expf(mx[i] - top);
+            weight[lane + 64 * i] = w;
+            weighted += w * sum[i];
+        }
+        const float total = wave_sum(weighted);
+        if (lane == 0) inv_total = total > 0.f ? 1.f / total : 0.f;
     }
     // The partial results do not depend on the weights: their first loads are issued before the barrier.
     const float* acc = part_acc + base * D;
@@ -941,5 +954,7 @@ LSA_EXPORT int lsa_attention_workgroup_tiles() {
     return 0;
 #endif
 }
+// Most key ranges a tile's keys may be split into (the merge takes no more slots per tile).
+LSA_EXPORT int lsa_attention_most_splits() { return MERGE_MOST_SLOTS; }
 LSA_EXPORT int lsa_attention_head_dim() { return D; }
 LSA_EXPORT int lsa_attention_is_bf16() { return LSA_BF16; }

@@ -22,6 +22,7 @@ _SIGNATURES = {
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, c_int,
                             c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, _P],
     "lsa_attention_workgroup_tiles": [],
+    "lsa_attention_most_splits": [],
     "lsa_attention_head_dim": [],
     "lsa_attention_is_bf16": [],
     "lsa_gemm_skinny": [c_int, _P, _P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P],

@@ -528,6 +528,8 @@ class HipOps:
                 _check(cos_sin, "cos_sin", torch.float32, (n, head_dim))
             fusion_mode = 3 if write_cache else 1
         lib = self._attention_library(qkv.dtype, head_dim)
+        if plan.get("most_splits", 0) > lib.lsa_attention_most_splits():
+            raise ValueError(f"the plan splits a tile's keys into {plan['most_splits']} ranges, the merge kernel takes {lib.lsa_attention_most_splits()}")
         _launched(lib.lsa_paged_attention(
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(row_start),
             _ptr(row_len), _ptr(row_ctx), _ptr(plan["items"]), _ptr(plan["item_slot"]), n_items, _ptr(plan["merges"]),

@@ -29,7 +29,7 @@ from .linear import Linear
 
 TILE_ROWS = 16          # rows of (token, group head) pairs one wavefront handles (MFMA N dimension)
 KEY_ALIGN = 32          # key ranges of split items start at multiples of this
-MAX_SPLITS = 64
+MAX_SPLITS = 128        # key ranges per tile (the merge kernel's limit, which the kernel namespace checks)
 MIN_KEYS_PER_SPLIT = 64     # shorter key ranges than this are not worth a wavefront of their own (measured at batch 1 to 8)
 TARGET_WAVES = 1024     # wavefronts wanted in flight on 256 CUs (measured: more and shorter items cost more in the merge than they gain)
 
@@ -224,6 +224,7 @@ class GQAttention(Mixer):
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
             "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),
             "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup,
+            "most_splits": int(plan.merges[:, 3].max()) if len(plan.merges) else 0,
         })
 
     def forward(self, x, ctx, cache, sink=None):

@@ -300,6 +300,10 @@ def test_attention_long_context_splits_and_needle(ops, dtype):
     assert float(ref[0, :128].float().mean()) > 5.0             # the far key won: its value (10) dominates the first head
     attention_case(ops, dtype, 8, 2, 128, 16, [1, 3], [2049, 1500], seed=3, target_waves=1)      # same, unsplit
     attention_case(ops, dtype, 4, 4, 64, 16, [600], [600], seed=4, target_waves=10 ** 6)         # a whole prompt, split to the limit
+    plan, ref = attention_case(ops, dtype, 4, 1, 64, 16, [1], [16384], seed=5)                   # one token behind 16,383: 128 key ranges
+    assert int(plan.merges[:, 3].max()) == 128 and float(ref[0, :64].float().mean()) > 5.0
+    plan, _ = attention_case(ops, dtype, 4, 1, 64, 16, [1], [8300], seed=6)                      # 87 ranges: more than one wavefront has lanes
+    assert 64 < int(plan.merges[:, 3].max()) < 128
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
