@@ -44,12 +44,12 @@ struct PartialSums {
     size_t stride;
 };
 
-template <typename T, int V>
+template <typename T, int V, bool PARTIAL>
 __device__ inline void load_sum(const T* __restrict__ x, const T* __restrict__ d, const PartialSums& p, size_t row_offset, int i,
                                 float (&s)[V]) {
     float update[V];
-    const bool any = d || p.sums;
-    if (p.sums) {
+    const bool any = PARTIAL || d;
+    if (PARTIAL) {
 #pragma unroll
         for (int k = 0; k < V; ++k) update[k] = 0.f;
         const float* src = p.sums + row_offset + i;
@@ -96,14 +96,14 @@ __device__ inline void load_sum(const T* __restrict__ x, const T* __restrict__ d
         Vec16<T> a = load_vec16(x + row_offset + i);
 #pragma unroll
         for (int k = 0; k < V; ++k) s[k] = (float)a.v[k];
-        if (d) {
+        if (!PARTIAL && d) {
             Vec16<T> b = load_vec16(d + row_offset + i);
 #pragma unroll
             for (int k = 0; k < V; ++k) update[k] = (float)b.v[k];
         }
     } else {
         s[0] = (float)x[row_offset + i];
-        if (d) update[0] = (float)d[row_offset + i];
+        if (!PARTIAL && d) update[0] = (float)d[row_offset + i];
     }
     if (any) {
 #pragma unroll
@@ -111,7 +111,8 @@ __device__ inline void load_sum(const T* __restrict__ x, const T* __restrict__ d
     }
 }
 
-template <typename T, int V>
+// PARTIAL: the update comes as partial sums (a kernel of its own, so that the plain one keeps its registers).
+template <typename T, int V, bool PARTIAL>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid, const T* __restrict__ delta, PartialSums partial,
                                                           const float* __restrict__ weight, float eps,
                                                           T* __restrict__ out, const int* __restrict__ rows, int width) {
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
     const size_t row_offset = (size_t)src_row * width;
     T* x = resid + row_offset;
     T* y = out + (size_t)blockIdx.x * width;
-    const bool updated = delta || partial.sums;
+    const bool updated = PARTIAL || delta;
     const int stride = blockDim.x * V;
     float kept[CACHE][V];
     float sq = 0.f;
@@ -131,14 +132,14 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
     for (int c = 0; c < CACHE; ++c) {
         const int i = threadIdx.x * V + c * stride;
         if (i < width) {
-            load_sum<T, V>(resid, delta, partial, row_offset, i, kept[c]);
+            load_sum<T, V, PARTIAL>(resid, delta, partial, row_offset, i, kept[c]);
 #pragma unroll
             for (int k = 0; k < V; ++k) sq += kept[c][k] * kept[c][k];
         }
     }
     for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
         float s[V];
-        load_sum<T, V>(resid, delta, partial, row_offset, i, s);
+        load_sum<T, V, PARTIAL>(resid, delta, partial, row_offset, i, s);
 #pragma unroll
         for (int k = 0; k < V; ++k) sq += s[k] * s[k];
     }
@@ -166,7 +167,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(T* __restrict__ resid,
     }
     for (int i = threadIdx.x * V + CACHE * stride; i < width; i += stride) {
         float s[V];
-        load_sum<T, V>(resid, delta, partial, row_offset, i, s);
+        load_sum<T, V, PARTIAL>(resid, delta, partial, row_offset, i, s);
         emit(i, s);
     }
 }
@@ -218,10 +219,17 @@ static int launch_add_rmsnorm(void* resid, const void* delta, PartialSums partia
                               const int* rows, int n_out, int width, hipStream_t stream) {
     if (n_out <= 0) return 0;
     if (delta && partial.sums) return -1;
-    if (width % Elem<T>::kVec == 0)
-        add_rmsnorm_kernel<T, Elem<T>::kVec><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, partial, weight, eps, (T*)out, rows, width);
-    else
-        add_rmsnorm_kernel<T, 1><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, partial, weight, eps, (T*)out, rows, width);
+#define LSA_ADD_RMSNORM(V, PARTIAL) \
+    add_rmsnorm_kernel<T, V, PARTIAL><<<n_out, 256, 0, stream>>>((T*)resid, (const T*)delta, partial, weight, eps, (T*)out, rows, width)
+    const bool vectors = width % Elem<T>::kVec == 0;
+    if (partial.sums) {
+        if (vectors) LSA_ADD_RMSNORM(Elem<T>::kVec, true);
+        else LSA_ADD_RMSNORM(1, true);
+    } else {
+        if (vectors) LSA_ADD_RMSNORM(Elem<T>::kVec, false);
+        else LSA_ADD_RMSNORM(1, false);
+    }
+#undef LSA_ADD_RMSNORM
     LSA_LAUNCH_CHECK();
 }
 
