@@ -707,12 +707,12 @@ LSA_EXPORT int lsa_gemm_split(const void* x, const void* w, float* partial, int 
 constexpr int SPLIT_GATED_MOST_ROWS = 32;     // beyond, the library's product and the activation kernel are faster (measured)
 
 // Whether lsa_gemm_split_gated takes a size: 17 <= M <= 32, K a multiple of 8, and so many pairs of a gate and an up
-// row that one range of K per workgroup fills the chip in one round (with ranges to add up there is no result to
-// activate; with more rounds than one the library is faster: measured 118 against 104 us at 400 workgroups).
+// row that one range of K per workgroup fills the chip (with ranges to add up there is no result to activate).
+// Whether it is the faster way is for the caller to measure: with more rounds of workgroups than one the library
+// has been seen to win (118 against 104 us at 400 workgroups).
 LSA_EXPORT int lsa_gemm_split_gated_fits(int M, int I, int K) {
     if (M <= 16 || M > SPLIT_GATED_MOST_ROWS || I <= 0 || K < 8 || K % 8 != 0) return 0;
-    const long tiles = (I + SPLIT_TILE_ROWS / 2 - 1) / (SPLIT_TILE_ROWS / 2);
-    return tiles <= compute_units() && split_range(tiles, K) >= K ? 1 : 0;
+    return split_range((I + SPLIT_TILE_ROWS / 2 - 1) / (SPLIT_TILE_ROWS / 2), K) >= K ? 1 : 0;
 }
 
 // hidden [M, I] = silu(x . gate^T) * (x . up^T) in bfloat16, gate_up [2 I, K] with the gate rows first.

@@ -157,11 +157,15 @@ class HipOps:
 
     def library_is_faster(self, kind, x, weight, scaled=False, out_float32=False) -> bool:
         """Whether, for these sizes, the library's product (with a norm kernel before it if ``scaled``, and the
-        activation kernel after it if ``kind`` is "gated") beats the few-row kernel that does it all; measured once."""
+        activation kernel after it if ``kind`` is "gated") beats the kernel of this repository that does it all;
+        ``kind`` "partial": the product in partial sums and the norm kernel that adds them up, against the library's
+        product and the plain norm kernel.  Measured once."""
         if not self.choose_by_measurement:
             return False
         rows, width = x.shape
-        key = (kind, rows, weight.shape[0], width, bool(scaled), bool(out_float32))
+        # Beyond the few-row kernels one measurement stands for eight neighbouring numbers of rows (portions of
+        # prompts come in every length, and each measurement takes a few milliseconds).
+        key = (kind, rows if rows <= 16 else -(-rows // 8) * 8, weight.shape[0], width, bool(scaled), bool(out_float32))
         known = self._library_faster.get(key)
         if known is not None:
             return known
@@ -174,7 +178,20 @@ class HipOps:
         normed = torch.empty_like(x) if scaled else None
         saved, self.choose_by_measurement = self.choose_by_measurement, False
         try:
-            if kind == "gated":
+            if kind == "partial":
+                stream = torch.zeros((rows, weight.shape[0]), device=x.device, dtype=x.dtype)
+                norm_weight = torch.ones(weight.shape[0], device=x.device, dtype=torch.float32)
+                normed = torch.empty_like(stream)
+
+                def few():
+                    sums = self.linear_partial_sums(x, weight, few_rows_too=True)
+                    if sums is not None:
+                        self.add_rmsnorm(stream, sums, norm_weight, 1e-6, normed)
+                    return sums
+
+                def library():
+                    self.add_rmsnorm(stream, torch.mm(x, weight.t()), norm_weight, 1e-6, normed)
+            elif kind == "gated":
                 hidden = torch.empty((rows, weight.shape[0] // 2), device=x.device, dtype=x.dtype)
 
                 def few():
@@ -193,7 +210,8 @@ class HipOps:
                         self.add_rmsnorm(stream, None, norm_weight, 1e-6, normed)
                     return torch.mm(x, weight.t(), out_dtype=torch.float32) if out_float32 else torch.mm(x, weight.t())
             if few() is None:
-                return False                              # no case for the few-row kernel: nothing to choose
+                self._library_faster[key] = False         # no case for this repository's kernel: nothing to choose
+                return False
             faster = self._second_is_faster(few, library)
         finally:
             self.choose_by_measurement = saved
@@ -293,6 +311,8 @@ class HipOps:
         if not ((0 if few_rows_too else self.skinny_rows) < rows <= self.SPLIT_ROWS) or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
                 or x.shape[1] != weight.shape[1] or not self.split_products:
             return None
+        if not few_rows_too and self.library_is_faster("partial", x, weight):
+            return None
         size = (rows, weight.shape[0], width)
         parts = self._split_parts.get(size)
         if parts is None:
@@ -366,7 +386,7 @@ class HipOps:
         fits = self._split_parts.get(size)
         if fits is None:
             fits = self._split_parts[size] = self._gemm.lsa_gemm_split_gated_fits(rows, inter, width)
-        if not fits:
+        if not fits or self.library_is_faster("gated", x, gate_up_weight):
             return None
         _check(x, "x", torch.bfloat16)
         _check(gate_up_weight, "gate_up_weight", torch.bfloat16)

@@ -551,15 +551,14 @@ def test_gated_product_with_activation_in_the_epilogue(ops, rows, inter, k):
 @pytest.mark.parametrize("inter, k", [(12288, 4096), (9000, 264), (10001, 72), (16384, 1000), (20000, 1000), (8192, 512), (1000, 1000)])
 def test_gated_product_beyond_few_rows(ops, rows, inter, k):
     """17 to 32 rows: the product that shares the activations through LDS, with the activation in its epilogue, where
-    the weight has rows enough for one workgroup to take the whole inner dimension, and not more than one round of
-    workgroups; elsewhere it is not offered."""
+    the weight has rows enough for one workgroup to take the whole inner dimension; elsewhere it is not offered."""
     print(f"gated product beyond few rows {rows} inter {inter} k {k}", flush=True)
     torch.manual_seed(rows + inter + k)
     x = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
     w = (torch.randn(2 * inter, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
     got = ops.linear_gated(x, w)
     offered = bool(ops._gemm.lsa_gemm_split_gated_fits(rows, inter, k))
-    assert offered == (rows <= 32 and 8192 < inter <= 16384)      # tiles of 64 pairs: more than half the compute units, not more than all
+    assert offered == (rows <= 32 and inter > 8192)               # tiles of 64 pairs: more than half as many as compute units
     assert (got is not None) == offered
     if got is not None:
         gate_up = x.double() @ w.double().t()
