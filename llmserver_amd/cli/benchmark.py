@@ -134,6 +134,9 @@ def main(argv=None) -> int:
                 body = prefix + body[args.shared_prefix_tokens:]
             prompts.append(body)
         rng.shuffle(prompts)
+        # A server captures its decode graphs (and measures its kernel choices) at start-up, before requests come
+        # (/root/reference/server.py:332): so does this workload, which stands for one.
+        engine.warmup_graphs(max_context=high + args.output_tokens)
         run_once(engine, build_prompts(vocab, 64, min(4, max_batch), "warm-mixed", args.seed), 4)
         for key in ("steps", "decode_steps", "prefill_steps", "tokens", "prefix_hit_tokens", "preemptions"):
             engine.step_profile[key] = 0

@@ -256,30 +256,38 @@ class Engine:
             self.preempt_request(victim)
 
     # -- one step ----------------------------------------------------------------------------
-    def warmup_graphs(self, batch_sizes=None) -> int:
+    def warmup_graphs(self, batch_sizes=None, max_context=None) -> int:
         """Capture the decode graphs of these numbers of rows (default: every size that decoding steps of up to
         ``max_batch_size`` rows are filled up to) before serving, so that the first steps of those sizes do not pay for
-        it; an idle engine only.  Returns how many graphs are held afterwards
-        (/root/reference/utils/engine.py:150-161).  The graphs serve contexts up to the first width of the block
-        table; longer ones are captured when they are reached."""
+        it, nor for the measurements by which kernels are chosen; an idle engine only.  Returns how many graphs are held
+        afterwards (/root/reference/utils/engine.py:150-161).  The graphs serve contexts up to the first width of the
+        block table, or, with ``max_context``, every width up to that context (the pool has to hold that many tokens
+        for every row meanwhile; sizes it cannot hold are left to be captured when they are met)."""
+        from .step import TABLE_WIDTH_STEP
         if not self.runner.use_graphs or self.active_requests:
             return 0
         most = self.scheduler.max_batch_size
         if batch_sizes is None:
             batch_sizes = sorted({min(most, padded_rows(rows)) for rows in range(1, most + 1)})
+        tokens_per_width = TABLE_WIDTH_STEP * self.block_size
+        contexts = [1] + [width * tokens_per_width + 1 for width in range(1, -(-(max_context or 1) // tokens_per_width))]
         try:
-            for rows in batch_sizes:
-                if not 0 < rows <= most or rows > self.kv_cache.available_pages()[0]:
-                    continue
-                names = [f"warmup-{i}" for i in range(rows)]
-                try:
-                    for name in names:
-                        self.kv_cache.open(name)
-                    self.runner.step([StepEntry(name, [0], [0]) for name in names])      # one token each: the captured kind of step
-                finally:
-                    for name in names:
-                        if name in self.kv_cache.requests:
-                            self.kv_cache.close(name)
+            for context in contexts:
+                pages_per_row = -(-context // self.block_size)
+                for rows in batch_sizes:
+                    if not 0 < rows <= most or rows * pages_per_row > min(self.kv_cache.available_pages()):
+                        continue
+                    names = [f"warmup-{i}" for i in range(rows)]
+                    try:
+                        for name in names:
+                            self.kv_cache.open(name)
+                            self.kv_cache.ensure(name, context)       # pages of zeros stand for a context of this length
+                            self.kv_cache.advance(name, context - 1)
+                        self.runner.step([StepEntry(name, [0], [0]) for name in names])  # one token each: the captured kind of step
+                    finally:
+                        for name in names:
+                            if name in self.kv_cache.requests:
+                                self.kv_cache.close(name)
         except Exception as error:               # as the reference: serving goes on, graphs are captured on first use
             import warnings
             warnings.warn(f"graph warm-up failed ({error!r}); graphs will be captured on first use")

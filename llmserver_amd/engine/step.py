@@ -26,7 +26,7 @@ from ..cache.manager import CacheManager
 from .batch import Staging, StepContext, StepEntry
 
 TABLE_WIDTH_STEP = 64      # captured steps serve block tables up to the next multiple of this many pages
-MAX_GRAPHS = 24
+MAX_GRAPHS = 96
 
 
 def padded_rows(rows: int) -> int:

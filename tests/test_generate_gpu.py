@@ -96,6 +96,14 @@ def test_graphs_captured_ahead_change_nothing():
     warmed.add_request(None, prompt_token_ids=[1, 2, 3])
     assert warmed.warmup_graphs() == 0                                   # not while requests are live
     warmed.kv_cache.check_invariants()
+    # longer contexts: a graph for every width of the block table up to the context, where the pool can hold the rows
+    roomy = Engine(model, None, max_new_tokens=10, max_batch_size=4, max_num_batched_tokens=64, kv_cache_num_blocks=200,
+                   kv_cache_block_size=page, ignore_eos=True)
+    assert roomy.warmup_graphs(batch_sizes=(1, 2, 4), max_context=64 * page + 70) == 5    # 1, 2, 4 rows; 1 and 2 rows behind 64 pages
+    assert sorted(key[:2] for key in roomy.runner._graphs) == [(1, 64), (1, 128), (2, 64), (2, 128), (4, 64)]
+    assert min(roomy.kv_cache.available_pages()) == 200 and not roomy.kv_cache.requests
+    assert roomy.generate(prompts) == plain_run
+    roomy.kv_cache.check_invariants()
 
 
 def test_temperature_sampling_is_seeded_per_request():
