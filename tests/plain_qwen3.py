@@ -53,9 +53,18 @@ def inverse_frequencies(head_dim, theta, dtype=torch.float64):
     return table.to(dtype)
 
 
-def rope_cos_sin(positions, head_dim, theta, dtype=torch.float64):
-    """angles = pos * inv_freq, duplicated over both halves  (/root/reference/utils/layers.py:160-164)."""
-    frequencies = positions.to(dtype).unsqueeze(-1) * inverse_frequencies(head_dim, theta, dtype)
+ANGLE_DTYPE = torch.float32     # precision of pos * inv_freq, as in the reference; tests of exact invariants set float64
+
+
+def rope_cos_sin(positions, head_dim, theta, dtype=torch.float64, angle_dtype=None):
+    """angles = pos * inv_freq, duplicated over both halves  (/root/reference/utils/layers.py:160-164).
+
+    The reference forms the product in float32 (line 160: ``pos_ids.to(torch.float32) * inv_freq``), and a
+    float32 angle of a few thousand radians is up to 2e-4 away from the exact product: that rounding is
+    part of the formula, so it is kept; cosine and sine of that angle are then taken in ``dtype``.
+    ``angle_dtype=torch.float64`` gives the exact product (for invariants that hold only without that rounding)."""
+    angle_dtype = angle_dtype or ANGLE_DTYPE
+    frequencies = (positions.to(angle_dtype).unsqueeze(-1) * inverse_frequencies(head_dim, theta, angle_dtype)).to(dtype)
     angles = torch.cat([frequencies, frequencies], dim=-1)
     return torch.cos(angles), torch.sin(angles)
 

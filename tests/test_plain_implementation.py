@@ -112,19 +112,25 @@ def test_rotation_sign_and_frequency_order():
 def test_rotated_scores_depend_on_distance_only():
     q, k = torch.randn(1, 1, 8, dtype=D64), torch.randn(1, 1, 8, dtype=D64)
     def score(pq, pk):
-        cq, sq = plain.rope_cos_sin(torch.tensor([pq]), 8, 100.0)
-        ck, sk = plain.rope_cos_sin(torch.tensor([pk]), 8, 100.0)
+        cq, sq = plain.rope_cos_sin(torch.tensor([pq]), 8, 100.0, angle_dtype=angle_dtype)
+        ck, sk = plain.rope_cos_sin(torch.tensor([pk]), 8, 100.0, angle_dtype=angle_dtype)
         return float((plain.apply_rope(q, cq, sq) * plain.apply_rope(k, ck, sk)).sum())
+    angle_dtype = D64                                 # exact angles: the invariance is exact
     assert abs(score(7, 3) - score(107, 103)) < 1e-9
     assert abs(score(7, 3) - score(7, 4)) > 1e-6
+    angle_dtype = torch.float32                       # the reference's float32 angles: exact up to their rounding
+    assert abs(score(7, 3) - score(107, 103)) < 1e-4
 
 
-def test_whole_model_is_invariant_to_a_shift_of_all_positions():
+def test_whole_model_is_invariant_to_a_shift_of_all_positions(monkeypatch):
     tensors = tiny_tensors(CONFIG)
     tokens = [3, 9, 1, 44, 17, 5, 5, 30]
+    with_float32_angles = plain.forward(CONFIG, tensors, tokens)
+    monkeypatch.setattr(plain, "ANGLE_DTYPE", D64)        # exact angles: the invariance is exact
     base = plain.forward(CONFIG, tensors, tokens)
     shifted = plain.forward(CONFIG, tensors, tokens, first_position=57)
     assert torch.allclose(base, shifted, atol=1e-9)
+    assert torch.allclose(base, with_float32_angles, atol=1e-5)   # the reference's float32 angles differ by their rounding only
 
 
 def test_swiglu_is_silu_gate_times_up():
