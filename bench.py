@@ -90,7 +90,9 @@ class DecodeBench:
     def step(self):
         entries = [self.StepEntry(rid, [token], [0]) for rid, token in zip(self.ids, self.last)]
         logits = self.runner.step(entries)
-        self.last = self.sampler.sample(logits, [0.0] * self.batch, [0.0] * self.batch)
+        sampled = self.sampler.launch(logits, [0.0] * self.batch, [0.0] * self.batch)
+        self.runner.prepare_ahead(self.ids)      # as the engine does: the next step's host work, while the GPU runs this one
+        self.last = sampled.tolist()
 
     def run(self, steps, warmup):
         torch = self.torch

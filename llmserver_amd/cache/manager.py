@@ -19,6 +19,7 @@ import hashlib
 import json
 from typing import Dict, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..parts.base import PagedKVSpec, StateSpec
@@ -67,6 +68,27 @@ class RequestCache:
         self.tables: List[List[int]] = [[] for _ in range(n_groups)]
         self.state_slot = -1
         self.num_computed = 0
+        self._arrays: List[Optional[np.ndarray]] = [None] * n_groups
+        self._synced = [0] * n_groups       # entries of each table that its array mirrors
+
+    def table_array(self, group: int) -> np.ndarray:
+        """The group's block table as an int32 array (a view that the next call may overwrite).  A table mostly
+        grows at its end, so only the new entries are converted; whoever changes entries in place or takes entries
+        away calls :meth:`table_changed`."""
+        table = self.tables[group]
+        n, array, synced = len(table), self._arrays[group], min(self._synced[group], len(table))
+        if array is None or array.shape[0] < n:
+            grown = np.empty(max(64, 2 * n), dtype=np.int32)
+            if synced:
+                grown[:synced] = array[:synced]
+            array = self._arrays[group] = grown
+        if synced < n:
+            array[synced:n] = table[synced:]
+        self._synced[group] = n
+        return array[:n]
+
+    def table_changed(self, group: int) -> None:
+        self._synced[group] = 0
 
 
 class CacheManager:
@@ -185,6 +207,7 @@ class CacheManager:
                 table = record.tables[group.index]
                 assert table[-1] == page
                 table.pop()
+                record.table_changed(group.index)
                 group.pool.release(page)
             raise
 
@@ -200,6 +223,7 @@ class CacheManager:
                 if table[block] >= 0:
                     group.pool.release(table[block])
                     table[block] = -1
+                    record.table_changed(group.index)
 
     def close(self, request_id) -> None:
         """The request ended (or is preempted): everything it holds is given back."""

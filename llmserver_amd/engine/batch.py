@@ -97,6 +97,18 @@ class StepContext:
 
     def upload(self):
         """Stage every host array of the step (the batch's and the mixers' plans) and copy once."""
+        self.stage()
+        self.staging.upload()
+
+    def set_token_ids(self, token_ids: np.ndarray) -> None:
+        """Replace the token ids of a step that is staged but not yet copied (see ``ModelRunner.prepare_ahead``)."""
+        if token_ids.shape != self.h_token_ids.shape:
+            raise ValueError(f"{token_ids.shape[0]} token ids for a step of {self.h_token_ids.shape[0]} tokens")
+        self.h_token_ids = np.ascontiguousarray(token_ids, dtype=np.int32)
+        self.staging.host_np[self._token_ids_at:self._token_ids_at + self.h_token_ids.size] = self.h_token_ids
+
+    def stage(self):
+        """Lay every host array of the step out in the staging buffer; nothing is copied yet."""
         plan_arrays = [(plan, name) for plan in self._plans.values() for name, value in plan.items()
                        if isinstance(value, np.ndarray)]
         arrays = [self.h_token_ids, self.h_positions, self.h_token_row, self.h_row_start, self.h_row_len, self.h_row_ctx,
@@ -107,6 +119,7 @@ class StepContext:
         self.staging.reset(needed, may_grow=self.static_max_keys is None)
         self.layout = tuple(a.shape for a in arrays) + tuple(plan[name].shape for plan, name in plan_arrays)
         stage = self.staging.stage
+        self._token_ids_at = self.staging.used
         self.token_ids, self.positions, self.token_row = stage(self.h_token_ids), stage(self.h_positions), stage(self.h_token_row)
         self.row_start, self.row_len, self.row_ctx = stage(self.h_row_start), stage(self.h_row_len), stage(self.h_row_ctx)
         self.logit_idx = stage(self.h_logit_idx)
@@ -114,7 +127,6 @@ class StepContext:
         self.state_slots = stage(self.h_state_slots) if self.h_state_slots is not None else None
         for plan, name in plan_arrays:
             plan[name] = stage(plan[name])
-        self.staging.upload()
 
     # -- used by the parts ---------------------------------------------------------------------
     def empty(self, shape, dtype=None):

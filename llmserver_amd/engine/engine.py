@@ -295,6 +295,22 @@ class Engine:
             return 0
         return self.runner.graph_count()
 
+    def prepare_next_step(self, sampled) -> bool:
+        """If the next step can only be a decoding step of known requests (nobody waits, nobody is still in its
+        prompt), let the runner lay it out before this step's tokens are back.  A request that stops at this step
+        for a reason the host cannot foresee (an end-of-sequence token, a cancellation) makes the next step another
+        one than the one prepared, which is then dropped."""
+        if self.scheduler.waiting:
+            return False
+        following = []
+        for request in self.scheduler.running:
+            if request.status == RequestStatus.DECODING:
+                if len(request.generated_token_ids) + 1 < request.max_new_tokens:
+                    following.append(request.request_id)
+            elif request.status == RequestStatus.PREFILL:
+                return False
+        return bool(following) and self.runner.prepare_ahead(following)
+
     def run_scheduled(self, out) -> None:
         """Turn the plan into one flat batch, run it, sample, and move every request on."""
         entries, sampled = [], []
@@ -314,7 +330,12 @@ class Engine:
         logits = self.runner.step(entries)
         temperatures = [r.sampling.temperature for r in sampled]
         uniforms = [request_uniform(r.sampling.seed, r.num_samples_drawn) if r.sampling.temperature > 0 else 0.0 for r in sampled]
-        token_ids = self.sampler.sample(logits, temperatures, uniforms)
+        if sampled:
+            pending = self.sampler.launch(logits, temperatures, uniforms)
+            self.prepare_next_step(sampled)           # the host's share of the next step, while the GPU works on this one
+            token_ids = pending.tolist()
+        else:
+            token_ids = []
         self.step_profile["tokens"] += sum(len(e.tokens) for e in entries)
         for request in out.decode_requests:
             request.complete_decode()

@@ -60,6 +60,8 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs and graph_safe)
         self._graphs: "OrderedDict[tuple, _CapturedStep]" = OrderedDict()
         self.graph_replays = 0
+        self._ahead = None          # (graph key, request ids, staged context) of a decoding step prepared ahead
+        self.steps_prepared_ahead = 0
 
     def build_context(self, entries: Sequence[StepEntry], staging: Optional[Staging] = None,
                       table_width: Optional[int] = None, filler_rows: int = 0) -> StepContext:
@@ -107,13 +109,12 @@ class ModelRunner:
             token_ids.append(0)
             positions.append(0)
         tables = []
+        records = [self.cache.record(rid) for rid in request_ids]
         for group in self.cache.groups:
-            width = max(1, max(len(self.cache.record(rid).tables[group.index]) for rid in request_ids))
-            if table_width is not None:
-                width = table_width
+            rows_pages = [record.table_array(group.index) for record in records]
+            width = table_width if table_width is not None else max(1, max(len(pages) for pages in rows_pages))
             table = np.full((len(entries) + filler_rows, width), -1, dtype=np.int32)
-            for row, rid in enumerate(request_ids):
-                pages = self.cache.record(rid).tables[group.index]
+            for row, pages in enumerate(rows_pages):
                 table[row, :len(pages)] = pages
             for filler in range(filler_rows):
                 table[len(entries) + filler, 0] = group.scratch_page(filler)
@@ -145,8 +146,66 @@ class ModelRunner:
             rows = wanted = padded_rows(rows)          # decoding: filled up to one of a few sizes
         return (rows, width, wanted)
 
+    def prepare_ahead(self, request_ids: Sequence[object]) -> bool:
+        """Do the host's share of the next step now, while the GPU still works on the last one.
+
+        The caller expects the next step to bring one token, as yet unknown, for each of ``request_ids`` in this order,
+        and to want its logits: a decoding step.  Pages are allocated, the batch and the mixers' plans are laid out in
+        the staging buffer of the captured step of that shape; :meth:`step` then only fills in the token ids, copies
+        and replays.  If the next step turns out to be another one, what was prepared is dropped (pages that were
+        allocated for a request stay in its table until they are needed or the request ends).  Returns whether a
+        step was prepared; shapes that have not been captured yet are not prepared."""
+        self._ahead = None
+        request_ids = list(request_ids)
+        if not self.use_graphs or not request_ids or len(set(request_ids)) != len(request_ids) \
+                or any(rid not in self.cache.requests for rid in request_ids):
+            return False
+        entries = [StepEntry(rid, (0,), (0,)) for rid in request_ids]
+        key = self._graph_key(entries)
+        captured = self._graphs.get(key) if key is not None else None
+        if captured is None:
+            return False
+        try:
+            ctx = self.build_context(entries, staging=captured.staging, table_width=key[1], filler_rows=key[0] - len(entries))
+        except BufferError:          # no page for one of them: the step itself will say so, or the caller makes room
+            return False
+        ctx.static_max_keys = key[1] * self.cache.page_size
+        self.model.prepare(ctx)
+        ctx.stage()
+        if ctx.layout != captured.layout:
+            return False
+        self._ahead = (key, request_ids, ctx)
+        return True
+
+    def _take_ahead(self, entries, key) -> Optional[StepContext]:
+        """The context prepared ahead if it is this step's: same shape, same requests in the same order at the same
+        places of their sequences, one token each with its logits wanted."""
+        ahead, self._ahead = self._ahead, None
+        if ahead is None or ahead[0] != key or len(ahead[1]) != len(entries):
+            return None
+        ctx = ahead[2]
+        for row, (entry, rid) in enumerate(zip(entries, ahead[1])):
+            if entry.request_id != rid or len(entry.tokens) != 1 or list(entry.want) != [0] \
+                    or self.cache.requests[rid].num_computed + 1 != int(ctx.h_row_ctx[row]):
+                return None
+        tokens = np.fromiter((entry.tokens[0] for entry in entries), dtype=np.int64, count=len(entries))
+        if int(tokens.min()) < 0 or int(tokens.max()) >= self.vocab:
+            return None              # the usual way names the token and the request
+        ids = ctx.h_token_ids.copy()
+        ids[:len(entries)] = tokens
+        ctx.set_token_ids(ids)
+        return ctx
+
     def _step_captured(self, entries, key) -> torch.Tensor:
         captured = self._graphs.get(key)
+        ctx = self._take_ahead(entries, key) if captured is not None else None
+        if ctx is not None:
+            self._graphs.move_to_end(key)
+            ctx.staging.upload()
+            captured.graph.replay()
+            self.graph_replays += 1
+            self.steps_prepared_ahead += 1
+            return captured.logits[:len(entries)]
         staging = captured.staging if captured is not None else Staging(self.device, capacity=4096)
         ctx = self.build_context(entries, staging=staging, table_width=key[1], filler_rows=key[0] - len(entries))
         wanted = sum(len(entry.want) for entry in entries)           # the fillers' logits come last and are dropped
@@ -187,6 +246,8 @@ class ModelRunner:
 
         The tensor a captured step returns is overwritten by the next step of the same shape."""
         key = self._graph_key(entries)
+        if key is None:
+            self._ahead = None
         if key is not None:
             logits = self._step_captured(entries, key)
             ctx_rows = [(entry.request_id, self.cache.record(entry.request_id).num_computed + 1) for entry in entries]

@@ -97,9 +97,36 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
     return most if estimate(most, 2.75, 1.40) < estimate(4, 2.0, 1.37) else 4
 
 
+def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int) -> AttentionPlan:
+    """The plan of a step in which every row brings one token and every tile gets ``splits`` key ranges: what the
+    loop of :func:`build_attention_plan` makes for it, row by row, computed for all rows at once (a decode step of
+    many rows is planned thousands of times a second)."""
+    n_rows = len(row_ctx)
+    rows = np.arange(n_rows, dtype=np.int64)
+    k_end = row_ctx
+    k_begin = np.zeros_like(k_end) if window is None else np.maximum(0, k_end - window)
+    zeros = np.zeros_like(rows)
+    if splits <= 1:
+        items = np.stack([rows, zeros, k_begin, k_end], axis=1).astype(np.int32)
+        return AttentionPlan(items, np.full(n_rows, -1, dtype=np.int32), np.zeros((0, 4), dtype=np.int32), 0)
+    start = (k_begin // KEY_ALIGN) * KEY_ALIGN
+    per = -(-(k_end - start) // splits)
+    per = -(-per // KEY_ALIGN) * KEY_ALIGN
+    piece = start[:, None] + np.arange(splits, dtype=np.int64)[None, :] * per[:, None]
+    lo = np.maximum(piece, k_begin[:, None])
+    hi = np.minimum(piece + per[:, None], k_end[:, None])
+    inside = lo < k_end[:, None]
+    first = np.where(inside, lo, k_end[:, None])
+    last = np.where(inside, np.maximum(lo, hi), k_end[:, None])
+    items = np.stack([np.repeat(rows, splits), np.zeros(n_rows * splits, dtype=np.int64), first.reshape(-1), last.reshape(-1)],
+                     axis=1).astype(np.int32)
+    merges = np.stack([rows, zeros, rows * splits, np.full(n_rows, splits, dtype=np.int64)], axis=1).astype(np.int32)
+    return AttentionPlan(items, np.arange(n_rows * splits, dtype=np.int32), merges, n_rows * splits)
+
+
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
-                         workgroup_tiles: int = 0) -> AttentionPlan:
+                         workgroup_tiles: int = 0, single_token_shortcut: bool = True) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
@@ -109,6 +136,8 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
+    if single_token_shortcut and fixed_splits is not None and len(row_len) and int(row_len.min()) == 1 == int(row_len.max()):
+        return _single_token_plan(row_ctx, window, int(fixed_splits))
     tiles_per_row = -(-row_len // tokens_per_tile)
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
     items, slots, merges, tiles = [], [], [], []

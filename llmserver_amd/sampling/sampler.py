@@ -25,13 +25,18 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
         """One token per row of ``logits [n, vocab]``; temperature 0 takes the first maximum."""
-        n = logits.shape[0]
-        if n == 0:
+        if logits.shape[0] == 0:
             return []
+        return self.launch(logits, temperatures, uniforms).tolist()
+
+    def launch(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> torch.Tensor:
+        """Start the sampling of one token per row and return the int32 device tensor they will be in: whoever reads
+        it (``tolist()``) waits for the step; until then the host is free for other work."""
+        n = logits.shape[0]
         host = np.empty((2, n), dtype=np.float32)
         host[0] = temperatures
         host[1] = uniforms
         both = torch.from_numpy(host).to(self.device, non_blocking=True)
         out = torch.empty(n, dtype=torch.int32, device=self.device)
         self.ops.sample(logits, both[0], both[1], out)
-        return out.tolist()
+        return out

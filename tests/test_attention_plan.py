@@ -91,6 +91,22 @@ def test_captured_steps_get_arrays_of_one_shape():
     assert fixed_split_count(64, group_size, n_kv, 4096) < fixed_split_count(1, group_size, n_kv, 4096)
 
 
+@pytest.mark.parametrize("seed", range(20))
+def test_plan_of_single_tokens_made_at_once_equals_the_plan_made_row_by_row(seed):
+    rng = random.Random(seed)
+    rows = rng.randint(1, 70)
+    contexts = [rng.choice((1, 2, 31, 32, 33, 64, 100, 1000, 4095, 4096, 4097, rng.randint(1, 9000))) for _ in range(rows)]
+    window = rng.choice((None, None, 1, 40, 700))
+    splits = rng.choice((1, 2, 3, 8, 16, 128))
+    group_size, n_kv = rng.choice((1, 4, 20)), rng.choice((1, 8))
+    fast = build_attention_plan([1] * rows, contexts, group_size, n_kv, window, fixed_splits=splits)
+    slow = build_attention_plan([1] * rows, contexts, group_size, n_kv, window, fixed_splits=splits, single_token_shortcut=False)
+    for name in ("items", "item_slot", "merges", "tiles"):
+        a, b = getattr(fast, name), getattr(slow, name)
+        assert a.dtype == b.dtype and a.shape == b.shape and (a == b).all(), name
+    assert fast.n_slots == slow.n_slots and fast.tiles_per_workgroup == slow.tiles_per_workgroup
+
+
 def test_four_or_eight_tiles_per_workgroup():
     """One short prompt is bounded by its longest workgroup and takes four tiles per workgroup; long rows and many rows
     keep every compute unit busy and take eight; a kernel that offers only four gets four."""

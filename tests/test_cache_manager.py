@@ -181,11 +181,16 @@ def test_random_orders_of_requests_lose_nothing(seed):
             m.advance(rid, grown)
             m.register_prefix(rid, prompts[rid], lengths[rid], grown)
             lengths[rid] = grown
+            if rng.random() < 0.5:       # the array a step copies into its block table mirrors the list, whatever changed it
+                for group in m.groups:
+                    assert m.record(rid).table_array(group.index).tolist() == m.record(rid).tables[group.index]
         elif live:
             rid = live.pop(rng.randrange(len(live)))
             m.close(rid)
         m.check_invariants()
     for rid in live:
+        for group in m.groups:
+            assert m.record(rid).table_array(group.index).tolist() == m.record(rid).tables[group.index]
         m.close(rid)
     m.check_invariants()
     for group in m.groups:

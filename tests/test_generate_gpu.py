@@ -93,6 +93,8 @@ def test_graphs_captured_ahead_change_nothing():
     replays = warmed.runner.graph_replays
     assert warmed.generate(prompts) == plain_run
     assert warmed.runner.graph_replays > replays and warmed.runner.graph_count() == 4     # no further capture was needed
+    assert warmed.runner.steps_prepared_ahead >= 6       # decoding steps were laid out while the step before them ran
+    assert min(warmed.kv_cache.available_pages()) == 40 and not warmed.kv_cache.requests
     warmed.add_request(None, prompt_token_ids=[1, 2, 3])
     assert warmed.warmup_graphs() == 0                                   # not while requests are live
     warmed.kv_cache.check_invariants()

@@ -49,3 +49,55 @@ def test_replayed_steps_equal_eager_steps(case, n_live, dtype):
     assert worst <= (1e-5 if dtype == "float32" else 2e-2), worst
     for runner in runners:
         runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_prepared_ahead_equal_steps_prepared_in_time(dtype):
+    """A decoding step whose host work was done before its tokens were known gives what the same step gives when
+    it is prepared the usual way; a step that turns out to be another one than the one prepared (other requests,
+    another order, a portion of a prompt between) drops what was prepared and is right all the same."""
+    from llmserver_amd.cache import CacheManager
+    from llmserver_amd.engine import ModelRunner, StepEntry, load_model
+    case = "B"
+    raw, _, page = CASES[case]
+    model = load_model(model_folder(case), "cuda", dtype)
+    runners = []
+    for _ in range(2):
+        cache = CacheManager(model.cache_specs(), page, 400, device="cuda", dtype=model.dtype)
+        runners.append(ModelRunner(model, cache, use_graphs=True))
+    ahead, plain = runners
+    lengths = [37, 5, 64, 1, 90, 16, 17]
+    prompts = {f"r{i}": random_tokens(raw["vocab_size"], n, 1 + i) for i, n in enumerate(lengths)}
+    feed = {rid: random_tokens(raw["vocab_size"], 60, 10 + i) for i, rid in enumerate(prompts)}
+    for runner in runners:
+        for rid, tokens in prompts.items():
+            runner.cache.open(rid)
+            runner.step([StepEntry(rid, tokens, [])])
+    worst, prepared = 0.0, 0
+    for turn in range(60):
+        live = list(prompts)
+        if turn % 10 == 4:
+            live = live[::2]                    # fewer requests than were prepared for
+        if turn % 10 == 7:
+            live = live[::-1]                   # the same requests in another order
+        entries = [StepEntry(rid, [feed[rid][turn]], [0]) for rid in live]
+        outs = [runner.step(entries).clone() for runner in runners]
+        torch.cuda.synchronize()
+        worst = max(worst, float((outs[0] - outs[1]).abs().max()))
+        if turn % 10 == 8:                      # a portion of another prompt between the preparation and the step
+            prepared += ahead.prepare_ahead(list(prompts))
+            for runner in runners:
+                runner.cache.open("tmp")
+                runner.step([StepEntry("tmp", random_tokens(raw["vocab_size"], 23, turn), [22])])
+                runner.cache.close("tmp")
+        prepared += ahead.prepare_ahead(list(prompts))
+    assert prepared >= 55                       # all but the first steps of a shape, which are captured the usual way
+    assert 35 <= ahead.steps_prepared_ahead < prepared and plain.steps_prepared_ahead == 0
+    assert worst <= (1e-5 if dtype == "float32" else 2e-2), worst
+    assert not ahead.prepare_ahead(["nobody"]) and not ahead.prepare_ahead([]) and not ahead.prepare_ahead(["r0", "r0"])
+    for runner in runners:
+        runner.cache.check_invariants()
+        for rid in prompts:
+            runner.cache.close(rid)
+        runner.cache.check_invariants()
+        assert all(group.pool.num_available == group.pool.num_pages for group in runner.cache.groups)
