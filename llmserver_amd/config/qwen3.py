@@ -3,7 +3,8 @@
 Keys and defaults follow what the reference reads (/root/reference/utils/architecture.py:72-107):
 ``head_dim`` defaults to ``hidden_size // num_attention_heads`` (line 88) and need not multiply
 back to the hidden size; ``rope_theta`` may sit at top level or inside ``rope_parameters`` /
-``rope_scaling`` and defaults to 10000.0 (lines 23-30); ``rms_norm_eps`` has no default (106).
+``rope_scaling`` and defaults to 10000.0 (lines 23-30); ``rms_norm_eps`` has no default (106);
+``num_key_value_heads``, when the file leaves it out, is the number of query heads (plain multi-head attention).
 The refusals are the reference's (72-86, /root/reference/utils/attention.py:186-187).
 """
 from __future__ import annotations
@@ -25,8 +26,8 @@ class Qwen3Config(ModelConfig):
     intermediate_size: int = field("intermediate_size", int)
     num_hidden_layers: int = field("num_hidden_layers", int)
     num_attention_heads: int = field("num_attention_heads", int)
-    num_key_value_heads: int = field("num_key_value_heads", int)
     rms_norm_eps: float = field("rms_norm_eps", float)
+    num_key_value_heads: int = field("num_key_value_heads", int, 0)
     head_dim: int = field("head_dim", int, 0)
     rope_theta: float = field("rope_theta", float, 0.0)
     attention_bias: bool = field("attention_bias", bool, False)
@@ -43,6 +44,8 @@ class Qwen3Config(ModelConfig):
             if self.num_attention_heads <= 0:
                 raise ConfigError("num_attention_heads must be positive")
             changes["head_dim"] = self.hidden_size // self.num_attention_heads
+        if self.num_key_value_heads == 0:            # absent: every query head has keys and values of its own
+            changes["num_key_value_heads"] = self.num_attention_heads
         if self.rope_theta == 0.0:
             parameters = raw.get("rope_scaling") or raw.get("rope_parameters") or {}
             changes["rope_theta"] = float(parameters.get("rope_theta", 10000.0))

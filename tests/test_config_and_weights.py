@@ -22,6 +22,13 @@ def test_config_reads_its_own_keys_and_defaults():
     assert c.head_dim == 64 // 4 and c.rope_theta == 10000.0            # reference defaults
     c = config_from_dict(dict(raw, rope_parameters={"rope_theta": 5e5}))
     assert c.rope_theta == 5e5
+    c = config_from_dict({k: v for k, v in raw.items() if k != "num_key_value_heads"})
+    assert c.num_key_value_heads == c.num_attention_heads == 4 and c.group_size == 1     # left out: multi-head attention
+    # keys a published config.json of the architecture carries beside the ones that are read change nothing
+    published = dict(TINY_A, architectures=["Qwen3ForCausalLM"], torch_dtype="bfloat16", sliding_window=None, use_sliding_window=False,
+                     max_window_layers=2, rope_scaling=None, attention_dropout=0.0, initializer_range=0.02, use_cache=True,
+                     transformers_version="4.51.0", layer_types=["full_attention", "full_attention"], rope_theta=10000)
+    assert config_from_dict(published) == a
     assert isinstance(a, Qwen3Config) and "qwen3" in registered_architectures()
 
 
