@@ -71,43 +71,46 @@ class ModelRunner:
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
-        token_ids: List[int] = []
-        positions: List[int] = []
-        token_row: List[int] = []
+        token_ids, positions, token_row = [], [], []         # one array per row
         row_start, row_len, row_ctx, logit_idx, request_ids = [], [], [], [], []
+        n_tokens = 0
         for row, entry in enumerate(entries):
             if entry.request_id in seen:
                 raise ValueError(f"request {entry.request_id!r} appears twice in one step")
             seen.add(entry.request_id)
-            tokens = list(entry.tokens)
-            if not tokens:
+            tokens = np.asarray(entry.tokens, dtype=np.int64).reshape(-1)
+            count = tokens.size
+            if not count:
                 raise ValueError(f"request {entry.request_id!r} brings no tokens")
-            for token in tokens:
-                if not 0 <= token < self.vocab:
-                    raise ValueError(f"token id {token} of request {entry.request_id!r} is outside the vocabulary of {self.vocab}")
+            if int(tokens.min()) < 0 or int(tokens.max()) >= self.vocab:
+                token = int(tokens[(tokens < 0) | (tokens >= self.vocab)][0])
+                raise ValueError(f"token id {token} of request {entry.request_id!r} is outside the vocabulary of {self.vocab}")
             record = self.cache.record(entry.request_id)
             start = record.num_computed
             for place in entry.want:
-                if not 0 <= place < len(tokens):
-                    raise ValueError(f"wanted place {place} is outside the {len(tokens)} tokens of request {entry.request_id!r}")
-                logit_idx.append(len(token_ids) + place)
-            row_start.append(len(token_ids))
-            row_len.append(len(tokens))
-            row_ctx.append(start + len(tokens))
+                if not 0 <= place < count:
+                    raise ValueError(f"wanted place {place} is outside the {count} tokens of request {entry.request_id!r}")
+                logit_idx.append(n_tokens + place)
+            row_start.append(n_tokens)
+            row_len.append(count)
+            row_ctx.append(start + count)
             request_ids.append(entry.request_id)
-            token_ids.extend(tokens)
-            positions.extend(range(start, start + len(tokens)))
-            token_row.extend([row] * len(tokens))
+            token_ids.append(tokens)
+            positions.append(np.arange(start, start + count, dtype=np.int64))
+            token_row.append(np.full(count, row, dtype=np.int64))
+            n_tokens += count
         for entry, ctx_len in zip(entries, row_ctx):
             self.cache.ensure(entry.request_id, ctx_len)
-        for filler in range(filler_rows):
-            logit_idx.append(len(token_ids))
-            row_start.append(len(token_ids))
-            row_len.append(1)
-            row_ctx.append(1)
-            token_row.append(len(entries) + filler)
-            token_ids.append(0)
-            positions.append(0)
+        if filler_rows:
+            fillers = np.arange(filler_rows, dtype=np.int64)
+            logit_idx.extend((n_tokens + fillers).tolist())
+            row_start.extend((n_tokens + fillers).tolist())
+            row_len.extend([1] * filler_rows)
+            row_ctx.extend([1] * filler_rows)
+            token_row.append(len(entries) + fillers)
+            token_ids.append(np.zeros(filler_rows, dtype=np.int64))
+            positions.append(np.zeros(filler_rows, dtype=np.int64))
+        token_ids, positions, token_row = np.concatenate(token_ids), np.concatenate(positions), np.concatenate(token_row)
         tables = []
         records = [self.cache.record(rid) for rid in request_ids]
         for group in self.cache.groups:
