@@ -72,6 +72,11 @@ constexpr int KEY_STEP = 16;
 constexpr int NS = D / 16;                   // 16-dim steps (four 16x16x4 MFMAs each)
 #endif
 
+// MODE is DecodeFusion::mode, known when the kernel is compiled: what a mode does not need is not in its code, and
+// no branch stands between the loads of the item's start (a load inside a branch makes every later wait a wait
+// for everything).
+// PLAIN: the step has both norm weights and a rotation (then nothing of the fused start depends on a flag).
+template <int MODE, bool PLAIN>
 __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
     const elem_t* keys, const elem_t* values,
@@ -82,163 +87,21 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     const int lane = threadIdx.x & 63;
     const int item_index = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (item_index >= n_items) return;
+    // The start of an item is a chain of loads, each of which needs the one before it (the item, its row, the row's
+    // queries and table entries, the first keys).  Every link costs a trip to memory, so everything that can be
+    // asked for is asked for as soon as its address is known, in the order in which it will be needed, and nothing
+    // is used before all of it is under way: three trips (item; row, table entries and norm weights; queries,
+    // rotation and first keys and values) instead of one per array.
     const Item item = items[item_index];
+    const int slot = item_slot[item_index];                    // needed at the very end only
     const int kv_head = blockIdx.y / g.gtiles, gtile = blockIdx.y % g.gtiles;
     const int col = lane & 15, quad = lane >> 4;
     const int row = item.row;
-    const int n = row_len[row], first_pos = row_ctx[row] - n, token0 = row_start[row] + item.q0;
-    // The pair this lane's column stands for.
-    const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
-    const bool pair_valid = pair_token < g.tokens_per_tile && item.q0 + pair_token < n && pair_head_in_group < g.group;
-    const int q_pos = pair_valid ? first_pos + item.q0 + pair_token : -1;
-    const int head = kv_head * g.group + pair_head_in_group;
     const int* row_table = table + (size_t)row * table_stride;
     const int ps = g.page_size;
     const size_t kv_head_keys = (size_t)kv_head * ps * D;      // offset of the head inside a key page
     const size_t kv_head_values = (size_t)kv_head * D * ps;
     const size_t page_elems = (size_t)g.n_kv * ps * D;
-
-    // Q^T operand, kept in registers for the whole item.
-#if LSA_BF16
-    bf16x8 qf[NS];
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        const int dim = 32 * s + 8 * quad;
-        bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (pair_valid && dim < D)
-            x = *reinterpret_cast<const bf16x8*>(q + (size_t)(token0 + pair_token) * q_token_stride + (size_t)head * D + dim);
-        qf[s] = x;
-    }
-    // A head in the operand layout (this lane: dims 32 s + 8 quad .. + 8 of every s), normalised over
-    // the head and rotated as the separate kernel does it; the four quads of a column share a head.
-    auto norm_rotate = [&](bf16x8 (&h)[NS], const float* weight, const float* cs) {
-        if (NS % 2) return;                               // head sizes in steps of 64 only (the host checks)
-        float x[NS][8];
-        float sq = 0.f;
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                x[s][e] = (float)h[s][e];
-                sq += x[s][e] * x[s][e];
-            }
-        if (weight) {
-            sq += __shfl_xor(sq, 16, 64);
-            sq += __shfl_xor(sq, 32, 64);
-            const float rstd = rsqrtf(sq / (float)D + fusion.eps);
-#pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                const f32x4 w0 = *reinterpret_cast<const f32x4*>(weight + 32 * s + 8 * quad);
-                const f32x4 w1 = *reinterpret_cast<const f32x4*>(weight + 32 * s + 8 * quad + 4);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) x[s][e] = x[s][e] * rstd * (e < 4 ? w0[e] : w1[e - 4]);
-            }
-        }
-        if (cs) {
-#pragma unroll
-            for (int s = 0; s < NS / 2; ++s) {
-                const float* c = cs + 32 * s + 8 * quad;
-                const f32x4 c0 = *reinterpret_cast<const f32x4*>(c), c1 = *reinterpret_cast<const f32x4*>(c + 4);
-                const f32x4 s0 = *reinterpret_cast<const f32x4*>(c + D / 2), s1 = *reinterpret_cast<const f32x4*>(c + D / 2 + 4);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float co = e < 4 ? c0[e] : c1[e - 4], si = e < 4 ? s0[e] : s1[e - 4];
-                    const float x1 = x[s][e], x2 = x[s + NS / 2][e];
-                    x[s][e] = x1 * co - x2 * si;
-                    x[s + NS / 2][e] = x2 * co + x1 * si;
-                }
-            }
-        }
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) h[s][e] = (bf16_t)x[s][e];
-    };
-    const float* token_cos_sin = fusion.cos_sin ? fusion.cos_sin + (size_t)token0 * D : nullptr;
-    if (fusion.mode & 1) {
-        norm_rotate(qf, fusion.q_weight, token_cos_sin);
-        if (!pair_valid) {
-#pragma unroll
-            for (int s = 0; s < NS; ++s) qf[s] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-        }
-    }
-#else
-    f32x4 qf[NS];
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        f32x4 x = {0.f, 0.f, 0.f, 0.f};
-        if (pair_valid)
-            x = *reinterpret_cast<const f32x4*>(q + (size_t)(token0 + pair_token) * q_token_stride + (size_t)head * D + 16 * s + 4 * quad);
-        qf[s] = x;
-    }
-#endif
-
-    f32x4 acc[ND];
-#pragma unroll
-    for (int c = 0; c < ND; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float run_max = NEG_INF, run_sum = 0.f;    // run_sum: this lane's share (its keys) of the pair's sum
-
-    int item_k_end = item.k_end;
-#if LSA_BF16
-    if ((fusion.mode & 2) && item.k_begin < item.k_end && item.k_end == row_ctx[row]) {
-        // This item ends at the row's new token.  Its key and value come from the projection, not from the
-        // pages: the online softmax starts from this one key (maximum = its score, sum = 1, output = its
-        // value) and the walk over the pages stops before it.  Column 0 puts both into the cache.
-        const int new_pos = item.k_end - 1;
-        const elem_t* token_qkv = q + (size_t)token0 * q_token_stride;
-        bf16x8 kh[NS];
-#pragma unroll
-        for (int s = 0; s < NS; ++s) kh[s] = *reinterpret_cast<const bf16x8*>(token_qkv + (size_t)(g.n_q + kv_head) * D + 32 * s + 8 * quad);
-        norm_rotate(kh, fusion.k_weight, token_cos_sin);
-        float dot = 0.f;
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) dot += (float)kh[s][e] * (float)qf[s][e];
-        dot += __shfl_xor(dot, 16, 64);
-        dot += __shfl_xor(dot, 32, 64);
-        const elem_t* vh = token_qkv + (size_t)(g.n_q + g.n_kv + kv_head) * D + 4 * quad;
-        bf16x4 vnew[ND];
-#pragma unroll
-        for (int c = 0; c < ND; ++c) vnew[c] = *reinterpret_cast<const bf16x4*>(vh + 16 * c);
-        if (pair_valid) {
-            run_max = dot * g.scale;
-            run_sum = quad == 0 ? 1.f : 0.f;
-#pragma unroll
-            for (int c = 0; c < ND; ++c)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[c][r] = (float)vnew[c][r];
-        }
-        if (col == 0) {
-            const int block = (int)__umulhi((unsigned)new_pos, g.page_magic);
-            const int slot = new_pos - block * ps;
-            const size_t page = (size_t)row_table[block] * page_elems;
-            elem_t* kp = const_cast<elem_t*>(keys) + page + kv_head_keys + (size_t)slot * D + 8 * quad;
-#pragma unroll
-            for (int s = 0; s < NS; ++s) *reinterpret_cast<bf16x8*>(kp + 32 * s) = kh[s];
-            elem_t* vp = const_cast<elem_t*>(values) + page + kv_head_values + (size_t)(4 * quad) * ps + slot;
-#pragma unroll
-            for (int c = 0; c < ND; ++c)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) vp[(size_t)(16 * c + r) * ps] = vnew[c][r];
-        }
-        item_k_end = new_pos;
-    }
-#endif
-    const int k_begin = item.k_begin, k_end = item_k_end;
-
-    // One step of KEY_STEP keys: the K rows and V^T pieces this lane feeds to the MFMAs.  Steps are
-    // loaded one ahead of the step being computed, so the loads of the next step are in flight
-    // while the softmax and the products of this one run.
-    struct Step {
-#if LSA_BF16
-        bf16x8 k[2][NS];
-        bf16x4 v[ND][2];
-#else
-        f32x4 k[NS];
-        f32x4 v[ND];
-#endif
-    };
 
     // Page ids come from the block table 64 logical blocks at a time: lane l of `pages_cur` holds
     // the page of block 64 * chunk + l, and a lane fetches the entry it needs with a shuffle.  The
@@ -254,8 +117,104 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
             pages_next = table_chunk(c + 1);
         }
     };
+    const int kt_first = (item.k_begin / KEY_STEP) * KEY_STEP;
+    chunk = (int)__umulhi((unsigned)kt_first, g.page_magic) >> 6;      // the table entries of the first keys need the item only
+    pages_cur = table_chunk(chunk);
+    pages_next = table_chunk(chunk + 1);
+#if LSA_BF16
+    // Norm weights and rotation of a head in the operand layout (this lane: dims 32 s + 8 quad .. + 8 of every s).
+    constexpr bool FUSABLE = NS % 2 == 0;                      // head sizes in steps of 64 only (the host checks)
+    constexpr int NR = NS / 2 > 0 ? NS / 2 : 1;
+    struct HeadWeights { f32x4 w[NS][2]; };
+    struct Rotation { f32x4 c[NR][2], s[NR][2]; };
+    auto load_weights = [&](HeadWeights& hw, const float* weight) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            hw.w[s][0] = *reinterpret_cast<const f32x4*>(weight + 32 * s + 8 * quad);
+            hw.w[s][1] = *reinterpret_cast<const f32x4*>(weight + 32 * s + 8 * quad + 4);
+        }
+    };
+    constexpr bool FUSED_Q = FUSABLE && (MODE & 1), NEW_TOKEN = FUSABLE && (MODE & 2);
+    // Where a step has no norm weights or no rotation, the loads read the start of the projection instead (any
+    // readable 4 D bytes will do: a row of it has at least 6 D) and what they bring is not used.
+    const float* readable = reinterpret_cast<const float*>(q);
+    const bool normed = PLAIN || fusion.q_weight != nullptr, rotated = PLAIN || fusion.cos_sin != nullptr;
+    HeadWeights q_weights;
+    if constexpr (FUSED_Q) load_weights(q_weights, normed ? fusion.q_weight : readable);
+#else
+    constexpr bool NEW_TOKEN = false;
+#endif
+    const int n = row_len[row], ctx = row_ctx[row], first_pos = ctx - n, token0 = row_start[row] + item.q0;
+    __builtin_amdgcn_sched_barrier(0);          // all of the above is asked for before any of it is waited for
+    // The pair this lane's column stands for.
+    const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
+    const bool pair_valid = pair_token < g.tokens_per_tile && item.q0 + pair_token < n && pair_head_in_group < g.group;
+    const int q_pos = pair_valid ? first_pos + item.q0 + pair_token : -1;
+    const int head = kv_head * g.group + pair_head_in_group;
+    // Decode steps: the item that ends at the row's new token takes that token's key and value from the projection,
+    // and walks the pages up to the key before it.
+    const bool takes_new_token = NEW_TOKEN && item.k_begin < item.k_end && item.k_end == ctx;
+    const int k_begin = item.k_begin, k_end = takes_new_token ? item.k_end - 1 : item.k_end;
+    // Q^T operand, kept in registers for the whole item.  Lanes without a pair read the first pair's (their
+    // operand is zeroed below): no branch stands between the loads.
+    const elem_t* q_lane = q + (size_t)(token0 + (pair_valid ? pair_token : 0)) * q_token_stride
+                             + (size_t)(pair_valid ? head : kv_head * g.group) * D;
+#if LSA_BF16
+    bf16x8 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int dim = 32 * s + 8 * quad;
+        if (32 * s + 32 <= D) {
+            qf[s] = *reinterpret_cast<const bf16x8*>(q_lane + dim);
+        } else {                                               // head size not a multiple of 32: the last step is half empty
+            bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (dim < D) x = *reinterpret_cast<const bf16x8*>(q_lane + dim);
+            qf[s] = x;
+        }
+    }
+    const float* token_cos_sin = rotated ? fusion.cos_sin + (size_t)token0 * D : readable;
+    Rotation rotation;
+    if constexpr (FUSED_Q || NEW_TOKEN) {
+#pragma unroll
+        for (int s = 0; s < NS / 2; ++s) {
+            const float* c = token_cos_sin + 32 * s + 8 * quad;
+            rotation.c[s][0] = *reinterpret_cast<const f32x4*>(c);
+            rotation.c[s][1] = *reinterpret_cast<const f32x4*>(c + 4);
+            rotation.s[s][0] = *reinterpret_cast<const f32x4*>(c + D / 2);
+            rotation.s[s][1] = *reinterpret_cast<const f32x4*>(c + D / 2 + 4);
+        }
+    }
+    const elem_t* token_qkv = q + (size_t)token0 * q_token_stride;
+    bf16x8 kh[NS];
+    bf16x4 vnew[ND];
+    if constexpr (NEW_TOKEN) {                  // every item asks for them (they are there for every row): no branch
+#pragma unroll
+        for (int s = 0; s < NS; ++s) kh[s] = *reinterpret_cast<const bf16x8*>(token_qkv + (size_t)(g.n_q + kv_head) * D + 32 * s + 8 * quad);
+        const elem_t* vh = token_qkv + (size_t)(g.n_q + g.n_kv + kv_head) * D + 4 * quad;
+#pragma unroll
+        for (int c = 0; c < ND; ++c) vnew[c] = *reinterpret_cast<const bf16x4*>(vh + 16 * c);
+    }
+#else
+    f32x4 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) qf[s] = *reinterpret_cast<const f32x4*>(q_lane + 16 * s + 4 * quad);
+#endif
+
+    // One step of KEY_STEP keys: the K rows and V^T pieces this lane feeds to the MFMAs.  Steps are
+    // loaded one ahead of the step being computed, so the loads of the next step are in flight
+    // while the softmax and the products of this one run.
+    struct Step {
+#if LSA_BF16
+        bf16x8 k[2][NS];
+        bf16x4 v[ND][2];
+#else
+        f32x4 k[NS];
+        f32x4 v[ND];
+#endif
+    };
+
     // Element offset of key `key` inside the pool: page * page_elems (+ what the caller adds).
-    auto locate = [&](int key, int& slot) {
+    auto locate_key = [&](int key, int& slot) {
         const int block = (int)__umulhi((unsigned)key, g.page_magic);
         slot = key - block * ps;
         return (size_t)__shfl(pages_cur, block - 64 * chunk, 64) * page_elems;
@@ -267,6 +226,13 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     auto load_step = [&](Step& f, int kt) {
         enter_chunk(kt);
         const int lo = max(k_begin, kt), hi = min(k_end, kt + KEY_STEP) - 1;      // valid keys of this step
+        // An item without keys (the first step is asked for before anybody looks) reads the start of the pool.
+        const bool none = hi < lo;
+        auto locate = [&](int key, int& slot) {
+            const size_t page = locate_key(key, slot);
+            if (none) slot = 0;
+            return none ? (size_t)0 : page;
+        };
 #if LSA_BF16
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
@@ -308,6 +274,106 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
         for (int c = 0; c < ND; ++c) f.v[c] = *reinterpret_cast<const f32x4*>(vp + (size_t)(16 * c) * ps);
 #endif
     };
+
+    // The first step's keys and values: under way while the queries are prepared.
+    Step a, b;
+    load_step(a, kt_first);                     // also for an item without keys: see load_step
+    __builtin_amdgcn_sched_barrier(0);          // and so are the queries, the rotation, the new key and value and the first keys
+
+#if LSA_BF16
+    // A head in the operand layout, normalised over the head and rotated as the separate kernel does it; the four
+    // quads of a column share a head.
+    auto norm_rotate = [&](bf16x8 (&h)[NS], bool normed, const HeadWeights& hw, bool rotated) {
+        float x[NS][8];
+        float sq = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[s][e] = (float)h[s][e];
+                sq += x[s][e] * x[s][e];
+            }
+        if (normed) {
+            sq += __shfl_xor(sq, 16, 64);
+            sq += __shfl_xor(sq, 32, 64);
+            const float rstd = rsqrtf(sq / (float)D + fusion.eps);
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[s][e] = x[s][e] * rstd * (e < 4 ? hw.w[s][0][e] : hw.w[s][1][e - 4]);
+        }
+        if (rotated) {
+#pragma unroll
+            for (int s = 0; s < NS / 2; ++s)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float co = e < 4 ? rotation.c[s][0][e] : rotation.c[s][1][e - 4];
+                    const float si = e < 4 ? rotation.s[s][0][e] : rotation.s[s][1][e - 4];
+                    const float x1 = x[s][e], x2 = x[s + NS / 2][e];
+                    x[s][e] = x1 * co - x2 * si;
+                    x[s + NS / 2][e] = x2 * co + x1 * si;
+                }
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[s][e] = (bf16_t)x[s][e];
+    };
+    if constexpr (FUSED_Q) norm_rotate(qf, normed, q_weights, rotated);
+    HeadWeights k_weights;
+    if constexpr (NEW_TOKEN) load_weights(k_weights, normed ? fusion.k_weight : readable);
+#endif
+    if (!pair_valid) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#if LSA_BF16
+            qf[s] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+#else
+            qf[s] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#endif
+    }
+
+    f32x4 acc[ND];
+#pragma unroll
+    for (int c = 0; c < ND; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float run_max = NEG_INF, run_sum = 0.f;    // run_sum: this lane's share (its keys) of the pair's sum
+
+#if LSA_BF16
+    if constexpr (NEW_TOKEN) if (takes_new_token) {
+        // The online softmax starts from the new token's key (maximum = its score, sum = 1, output = its value);
+        // column 0 puts key and value into the cache.
+        const int new_pos = item.k_end - 1;
+        norm_rotate(kh, normed, k_weights, rotated);
+        float dot = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dot += (float)kh[s][e] * (float)qf[s][e];
+        dot += __shfl_xor(dot, 16, 64);
+        dot += __shfl_xor(dot, 32, 64);
+        if (pair_valid) {
+            run_max = dot * g.scale;
+            run_sum = quad == 0 ? 1.f : 0.f;
+#pragma unroll
+            for (int c = 0; c < ND; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[c][r] = (float)vnew[c][r];
+        }
+        if (col == 0) {
+            const int block = (int)__umulhi((unsigned)new_pos, g.page_magic);
+            const int new_slot = new_pos - block * ps;
+            const size_t page = (size_t)row_table[block] * page_elems;
+            elem_t* kp = const_cast<elem_t*>(keys) + page + kv_head_keys + (size_t)new_slot * D + 8 * quad;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) *reinterpret_cast<bf16x8*>(kp + 32 * s) = kh[s];
+            elem_t* vp = const_cast<elem_t*>(values) + page + kv_head_values + (size_t)(4 * quad) * ps + new_slot;
+#pragma unroll
+            for (int c = 0; c < ND; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vp[(size_t)(16 * c + r) * ps] = vnew[c][r];
+        }
+    }
+#endif
 
     auto compute_step = [&](Step& f, int kt) {
         const bool edge = kt < k_begin || kt + KEY_STEP > k_end;
@@ -410,10 +476,8 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     };
 
     if (k_begin < k_end) {
-        Step a, b;
         int kt = (k_begin / KEY_STEP) * KEY_STEP;
         int steps = (k_end - kt + KEY_STEP - 1) / KEY_STEP;
-        load_step(a, kt);
         // Steady state without a branch between the loads of one step and the products of the
         // step before it, so that the wait for operands leaves the newer loads in flight.
         while (steps >= 3) {
@@ -436,7 +500,6 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     run_sum += __shfl_xor(run_sum, 16, 64);
     run_sum += __shfl_xor(run_sum, 32, 64);
     if (!pair_valid) return;
-    const int slot = item_slot[item_index];
     if (slot < 0) {
         const float inv = run_sum > 0.f ? 1.f / run_sum : 0.f;
         elem_t* o = out + ((size_t)(token0 + pair_token) * g.n_q + head) * D + 4 * quad;
@@ -932,9 +995,19 @@ LSA_EXPORT int lsa_paged_attention(
     }
     if (n_items <= 0) return 0;
     dim3 grid((n_items + 3) / 4, n_kv * gtiles);
-    paged_attention_kernel<<<grid, 256, 0, stream>>>(
-        (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
-        row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g, fusion);
+#define LSA_LAUNCH_ITEMS(MODE, PLAIN) paged_attention_kernel<MODE, PLAIN><<<grid, 256, 0, stream>>>( \
+        (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride, \
+        row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g, fusion)
+#if LSA_BF16
+    const bool plain = q_weight != nullptr && cos_sin != nullptr;
+    if (decode_fusion == 3 && plain) LSA_LAUNCH_ITEMS(3, true);
+    else if (decode_fusion == 3) LSA_LAUNCH_ITEMS(3, false);
+    else if (decode_fusion == 1 && plain) LSA_LAUNCH_ITEMS(1, true);
+    else if (decode_fusion == 1) LSA_LAUNCH_ITEMS(1, false);
+    else
+#endif
+    LSA_LAUNCH_ITEMS(0, false);
+#undef LSA_LAUNCH_ITEMS
     int err = (int)hipGetLastError();
     if (err || n_merges <= 0) return err;
     dim3 mgrid(n_merges, n_kv * gtiles, 16);
