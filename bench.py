@@ -87,21 +87,26 @@ class DecodeBench:
         self.last = torch.randint(0, vocab, (batch,), generator=generator).tolist()
         torch.cuda.synchronize()
 
-    def step(self):
+    def step(self, more_follow=True):
         entries = [self.StepEntry(rid, [token], [0]) for rid, token in zip(self.ids, self.last)]
         logits = self.runner.step(entries)
         sampled = self.sampler.launch(logits, [0.0] * self.batch, [0.0] * self.batch)
-        self.runner.prepare_ahead(self.ids)      # as the engine does: the next step's host work, while the GPU runs this one
+        # As the engine does while it knows that all requests go on: the next step is laid out on the host while the
+        # GPU runs this one, and started with the sampled tokens still on the device.
+        if more_follow and self.runner.prepare_ahead(self.ids):
+            self.runner.launch_ahead(sampled.device)
         self.last = sampled.tolist()
 
     def run(self, steps, warmup):
+        """Seconds for exactly ``steps`` decode steps: the last warm-up step starts nothing that the timed steps would
+        find done, and the last timed step starts nothing that would run beyond them."""
         torch = self.torch
-        for _ in range(warmup):
-            self.step()
+        for index in range(warmup):
+            self.step(more_follow=index + 1 < warmup)
         torch.cuda.synchronize()
         start = time.perf_counter()
-        for _ in range(steps):
-            self.step()
+        for index in range(steps):
+            self.step(more_follow=index + 1 < steps)
         torch.cuda.synchronize()
         return time.perf_counter() - start
 

@@ -45,7 +45,7 @@ class Engine:
     def __init__(self, model, tokenizer=None, max_new_tokens=128, max_batch_size=8, max_num_batched_tokens=2048,
                  max_completed_requests=1000, completed_request_ttl_seconds=3600, prefill_chunk_size=None,
                  kv_cache_num_blocks=500, kv_cache_block_size=500, stream_text=True, ignore_eos=False,
-                 temperature=0.0, seed=0, enable_prefix_caching=True, ops=None):
+                 temperature=0.0, seed=0, enable_prefix_caching=True, ops=None, launch_ahead=True):
         if max_new_tokens <= 0:
             raise ValueError(f"max_new_tokens is <= 0: {max_new_tokens}")
         if max_num_batched_tokens <= 0:
@@ -62,6 +62,7 @@ class Engine:
         self.stream_text = stream_text
         self.ignore_eos = ignore_eos
         self.temperature, self.seed = float(temperature), int(seed)
+        self.launch_ahead = bool(launch_ahead)      # decoding steps may start before the host has seen the tokens they bring
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_completed_requests = max_completed_requests
         self.completed_request_ttl = timedelta(seconds=completed_request_ttl_seconds)
@@ -295,11 +296,13 @@ class Engine:
             return 0
         return self.runner.graph_count()
 
-    def prepare_next_step(self, sampled) -> bool:
+    def prepare_next_step(self, sampled, pending=None) -> bool:
         """If the next step can only be a decoding step of known requests (nobody waits, nobody is still in its
-        prompt), let the runner lay it out before this step's tokens are back.  A request that stops at this step
-        for a reason the host cannot foresee (an end-of-sequence token, a cancellation) makes the next step another
-        one than the one prepared, which is then dropped."""
+        prompt), let the runner lay it out before this step's tokens are back; and if it brings exactly the requests
+        that were sampled just now, in their order, start it at once with the tokens ``pending`` that are still on the
+        device, so that the GPU does not wait for the host between the steps.  A request that stops at this step for
+        a reason the host cannot foresee (an end-of-sequence token, a cancellation) makes the next step another one
+        than the one prepared or started, which is then dropped and run again without that request."""
         if self.scheduler.waiting:
             return False
         following = []
@@ -309,7 +312,11 @@ class Engine:
                     following.append(request.request_id)
             elif request.status == RequestStatus.PREFILL:
                 return False
-        return bool(following) and self.runner.prepare_ahead(following)
+        if not following or not self.runner.prepare_ahead(following):
+            return False
+        if self.launch_ahead and pending is not None and following == [request.request_id for request in sampled]:
+            self.runner.launch_ahead(pending.device)
+        return True
 
     def run_scheduled(self, out) -> None:
         """Turn the plan into one flat batch, run it, sample, and move every request on."""
@@ -332,7 +339,7 @@ class Engine:
         uniforms = [request_uniform(r.sampling.seed, r.num_samples_drawn) if r.sampling.temperature > 0 else 0.0 for r in sampled]
         if sampled:
             pending = self.sampler.launch(logits, temperatures, uniforms)
-            self.prepare_next_step(sampled)           # the host's share of the next step, while the GPU works on this one
+            self.prepare_next_step(sampled, pending)  # the host's share of the next step, while the GPU works on this one
             token_ids = pending.tolist()
         else:
             token_ids = []

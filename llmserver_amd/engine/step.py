@@ -61,7 +61,9 @@ class ModelRunner:
         self._graphs: "OrderedDict[tuple, _CapturedStep]" = OrderedDict()
         self.graph_replays = 0
         self._ahead = None          # (graph key, request ids, staged context) of a decoding step prepared ahead
+        self._launched = None       # (request ids, their contexts after it, logits) of a step started ahead of its tokens
         self.steps_prepared_ahead = 0
+        self.steps_launched_ahead = 0
 
     def build_context(self, entries: Sequence[StepEntry], staging: Optional[Staging] = None,
                       table_width: Optional[int] = None, filler_rows: int = 0) -> StepContext:
@@ -149,6 +151,7 @@ class ModelRunner:
             rows = wanted = padded_rows(rows)          # decoding: filled up to one of a few sizes
         return (rows, width, wanted)
 
+    @torch.inference_mode()
     def prepare_ahead(self, request_ids: Sequence[object]) -> bool:
         """Do the host's share of the next step now, while the GPU still works on the last one.
 
@@ -179,6 +182,43 @@ class ModelRunner:
             return False
         self._ahead = (key, request_ids, ctx)
         return True
+
+    @torch.inference_mode()
+    def launch_ahead(self, device_tokens: torch.Tensor) -> bool:
+        """Start the step that :meth:`prepare_ahead` laid out, with token ids that are still on the device: row ``i``
+        gets ``device_tokens[i]`` (int32, one per request of the prepared step; the sampler's output for the step
+        before).  The host has not seen the tokens yet, so the GPU goes from one step to the next without waiting
+        for it.  The next :meth:`step` must bring these requests, in this order, with one token each and its logits
+        wanted: it then takes the result.  Any other step drops it: what it wrote into the pages lies at places that
+        are written again, with the same values, by the step that takes their tokens, or that nobody reads."""
+        ahead, self._ahead = self._ahead, None
+        if ahead is None or self._launched is not None:
+            return False
+        key, request_ids, ctx = ahead
+        captured = self._graphs.get(key)
+        if captured is None or device_tokens.dtype != torch.int32 or tuple(device_tokens.shape) != (len(request_ids),) \
+                or device_tokens.device != ctx.token_ids.device:
+            return False
+        self._graphs.move_to_end(key)
+        ctx.staging.upload()
+        ctx.token_ids[:len(request_ids)].copy_(device_tokens)       # on the device, in stream order behind the upload
+        captured.graph.replay()
+        self.graph_replays += 1
+        self.steps_launched_ahead += 1
+        self._launched = (request_ids, [int(c) for c in ctx.h_row_ctx[:len(request_ids)]], captured.logits[:len(request_ids)])
+        return True
+
+    def _take_launched(self, entries) -> Optional[torch.Tensor]:
+        """The logits of the step started ahead if ``entries`` are that step; it is dropped otherwise."""
+        launched, self._launched = self._launched, None
+        if launched is None or len(launched[0]) != len(entries):
+            return None
+        for entry, rid, ctx_len in zip(entries, launched[0], launched[1]):
+            record = self.cache.requests.get(rid)
+            if entry.request_id != rid or len(entry.tokens) != 1 or list(entry.want) != [0] or record is None \
+                    or record.num_computed + 1 != ctx_len:
+                return None
+        return launched[2]
 
     def _take_ahead(self, entries, key) -> Optional[StepContext]:
         """The context prepared ahead if it is this step's: same shape, same requests in the same order at the same
@@ -248,13 +288,14 @@ class ModelRunner:
         """Run one step; returns float32 logits ``[wanted, vocab]`` in the order of the entries and their ``want``.
 
         The tensor a captured step returns is overwritten by the next step of the same shape."""
-        key = self._graph_key(entries)
-        if key is None:
-            self._ahead = None
-        if key is not None:
-            logits = self._step_captured(entries, key)
+        logits = self._take_launched(entries) if self._launched is not None else None
+        key = self._graph_key(entries) if logits is None else None
+        if logits is not None or key is not None:
+            if logits is None:
+                logits = self._step_captured(entries, key)
             ctx_rows = [(entry.request_id, self.cache.record(entry.request_id).num_computed + 1) for entry in entries]
         else:
+            self._ahead = None
             ctx = self.build_context(entries)
             self.model.prepare(ctx)
             ctx.upload()

@@ -19,9 +19,31 @@ def request_uniform(seed: int, draw: int) -> float:
     return random.Random(f"{seed}:{draw}").random()
 
 
+class PendingTokens:
+    """Sampled tokens on their way to the host: ``device`` is the int32 tensor the kernels write, and a copy into
+    pinned host memory follows them in the stream.  :meth:`tolist` waits for that copy only, so work that is put
+    into the stream afterwards (the next step, started ahead) does not hold the tokens back."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor):
+        self.device = device
+        self._host = host[:device.shape[0]]
+        self._host.copy_(device, non_blocking=True)
+        self._copied = None
+        if device.is_cuda:
+            self._copied = torch.cuda.Event()
+            self._copied.record()
+
+    def tolist(self) -> List[int]:
+        if self._copied is not None:
+            self._copied.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
     def __init__(self, ops, device):
         self.ops, self.device = ops, torch.device(device)
+        self._host_buffers = []          # pinned buffers the sampled tokens are copied into, used in turn
+        self._turn = 0
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
         """One token per row of ``logits [n, vocab]``; temperature 0 takes the first maximum."""
@@ -29,9 +51,18 @@ class Sampler:
             return []
         return self.launch(logits, temperatures, uniforms).tolist()
 
-    def launch(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> torch.Tensor:
-        """Start the sampling of one token per row and return the int32 device tensor they will be in: whoever reads
-        it (``tolist()``) waits for the step; until then the host is free for other work."""
+    def _host_buffer(self, n: int) -> torch.Tensor:
+        pinned = self.device.type == "cuda"
+        if len(self._host_buffers) < 4:
+            self._host_buffers.append(torch.empty(max(n, 256), dtype=torch.int32, pin_memory=pinned))
+        self._turn = (self._turn + 1) % len(self._host_buffers)
+        if self._host_buffers[self._turn].shape[0] < n:
+            self._host_buffers[self._turn] = torch.empty(2 * n, dtype=torch.int32, pin_memory=pinned)
+        return self._host_buffers[self._turn]
+
+    def launch(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> PendingTokens:
+        """Start the sampling of one token per row, and the copy of the tokens to the host behind it; whoever reads
+        them (``tolist()``) waits for that copy; until then the host is free for other work."""
         n = logits.shape[0]
         host = np.empty((2, n), dtype=np.float32)
         host[0] = temperatures
@@ -39,4 +70,4 @@ class Sampler:
         both = torch.from_numpy(host).to(self.device, non_blocking=True)
         out = torch.empty(n, dtype=torch.int32, device=self.device)
         self.ops.sample(logits, both[0], both[1], out)
-        return out
+        return PendingTokens(out, self._host_buffer(n))

@@ -93,7 +93,8 @@ def test_graphs_captured_ahead_change_nothing():
     replays = warmed.runner.graph_replays
     assert warmed.generate(prompts) == plain_run
     assert warmed.runner.graph_replays > replays and warmed.runner.graph_count() == 4     # no further capture was needed
-    assert warmed.runner.steps_prepared_ahead >= 6       # decoding steps were laid out while the step before them ran
+    # decoding steps were laid out, most of them also started, while the step before them ran
+    assert warmed.runner.steps_prepared_ahead + warmed.runner.steps_launched_ahead >= 6 and warmed.runner.steps_launched_ahead >= 3
     assert min(warmed.kv_cache.available_pages()) == 40 and not warmed.kv_cache.requests
     warmed.add_request(None, prompt_token_ids=[1, 2, 3])
     assert warmed.warmup_graphs() == 0                                   # not while requests are live
@@ -146,3 +147,40 @@ def test_engine_refuses_to_run_without_its_kernels(monkeypatch):
     monkeypatch.setattr(torch.cuda, "is_available", lambda: False)
     with pytest.raises(KernelLibraryMissing):
         ops.HipOps()
+
+
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_steps_started_ahead_give_the_same_tokens_also_when_requests_stop_unforeseen(temperature):
+    """Decoding steps are started before the host has seen the tokens they bring; an end-of-sequence token makes the
+    step that was started another one than the step that follows.  Same tokens, same reasons to stop and every page
+    back, with and without starting ahead (bfloat16, requests of different lengths, stops by token and by length)."""
+    from llmserver_amd import Engine, load_model
+    print(f"steps started ahead, temperature {temperature}", flush=True)
+    case = "A"
+    raw, _, page = CASES[case]
+    prompts = [random_tokens(raw["vocab_size"], n, 500 + i) for i, n in enumerate((5, 17, 33, 9, 2, 21))]
+    limits = [40, 12, 40, 25, 40, 7]
+    model = load_model(model_folder(case), "cuda", "bfloat16")
+    def make(launch_ahead):
+        return Engine(model, None, max_new_tokens=40, max_batch_size=6, max_num_batched_tokens=128, kv_cache_num_blocks=60,
+                      kv_cache_block_size=page, ignore_eos=False, temperature=temperature, seed=3, launch_ahead=launch_ahead)
+    free_run = make(False)
+    free = [free_run.add_request(None, prompt_token_ids=prompt, max_new_tokens=limit) for prompt, limit in zip(prompts, limits)]
+    while free_run.step():
+        pass
+    # tokens that some requests produce in the middle of their run end those requests (and whoever else produces them)
+    stops = {free[0].generated_token_ids[6], free[2].generated_token_ids[10], free[4].generated_token_ids[3]}
+    outcomes = []
+    for launch_ahead in (False, True):
+        engine = make(launch_ahead)
+        engine.eos_token_ids = set(stops)
+        requests = [engine.add_request(None, prompt_token_ids=prompt, max_new_tokens=limit) for prompt, limit in zip(prompts, limits)]
+        while engine.step():
+            pass
+        outcomes.append([(list(r.generated_token_ids), r.finish_reason) for r in requests])
+        assert min(engine.kv_cache.available_pages()) == 60 and not engine.kv_cache.requests
+        engine.kv_cache.check_invariants()
+        assert (engine.runner.steps_launched_ahead > 0) == launch_ahead
+    assert outcomes[0] == outcomes[1]
+    reasons = {reason.value for _, reason in outcomes[1]}
+    assert len(reasons) == 2, reasons                                        # some stopped by a token, some by their length

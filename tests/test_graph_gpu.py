@@ -101,3 +101,55 @@ def test_steps_prepared_ahead_equal_steps_prepared_in_time(dtype):
             runner.cache.close(rid)
         runner.cache.check_invariants()
         assert all(group.pool.num_available == group.pool.num_pages for group in runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_started_ahead_of_their_tokens_equal_steps_started_in_time(dtype):
+    """Greedy decoding in which every step is started with the tokens of the step before still on the device, against
+    the same decoding step by step; now and then the step that follows is another one than the one started (a request
+    leaves, a portion of another prompt comes between), which must drop it and change nothing."""
+    from llmserver_amd.cache import CacheManager
+    from llmserver_amd.engine import ModelRunner, StepEntry, load_model
+    case = "B"
+    raw, _, page = CASES[case]
+    model = load_model(model_folder(case), "cuda", dtype)
+    runners = []
+    for _ in range(2):
+        cache = CacheManager(model.cache_specs(), page, 400, device="cuda", dtype=model.dtype)
+        runners.append(ModelRunner(model, cache, use_graphs=True))
+    ahead, plain = runners
+    lengths = [37, 5, 64, 1, 90, 16]
+    prompts = {f"r{i}": random_tokens(raw["vocab_size"], n, 1 + i) for i, n in enumerate(lengths)}
+    last = {}
+    for runner in runners:
+        for rid, tokens in prompts.items():
+            runner.cache.open(rid)
+            logits = runner.step([StepEntry(rid, tokens, [len(tokens) - 1])])
+            last[rid] = int(logits[0].argmax())
+    live = list(prompts)
+    worst = 0.0
+    for turn in range(50):
+        if turn == 20:
+            live = live[:-1]                    # a request leaves after a step was started with it
+        entries = [StepEntry(rid, [last[rid]], [0]) for rid in live]
+        got, want = ahead.step(entries), plain.step(entries)
+        worst = max(worst, float((got - want).abs().max()))
+        sampled = want.argmax(dim=-1).to(torch.int32)       # both runners go on with the same tokens
+        if turn % 10 == 6:                      # a portion of another prompt between the start and the step
+            assert ahead.prepare_ahead(live) and ahead.launch_ahead(sampled)
+            for runner in runners:
+                runner.cache.open("tmp")
+                runner.step([StepEntry("tmp", random_tokens(raw["vocab_size"], 23, turn), [22])])
+                runner.cache.close("tmp")
+        elif turn >= 2:
+            assert ahead.prepare_ahead(live) and ahead.launch_ahead(sampled)
+            assert not ahead.launch_ahead(sampled)          # nothing is prepared any more
+        for rid, token in zip(live, sampled.tolist()):
+            last[rid] = token
+    assert ahead.steps_launched_ahead >= 45 and plain.steps_launched_ahead == 0
+    assert worst <= (1e-5 if dtype == "float32" else 2e-2), worst
+    for runner in runners:
+        runner.cache.check_invariants()
+        for rid in prompts:
+            runner.cache.close(rid)
+        assert all(group.pool.num_available == group.pool.num_pages for group in runner.cache.groups)
