@@ -297,21 +297,25 @@ class Engine:
         return self.runner.graph_count()
 
     def prepare_next_step(self, sampled, pending=None) -> bool:
-        """If the next step can only be a decoding step of known requests (nobody waits, nobody is still in its
+        """If the next step can only be a decoding step of known requests (nobody can join, nobody is still in its
         prompt), let the runner lay it out before this step's tokens are back; and if it brings exactly the requests
         that were sampled just now, in their order, start it at once with the tokens ``pending`` that are still on the
         device, so that the GPU does not wait for the host between the steps.  A request that stops at this step for
         a reason the host cannot foresee (an end-of-sequence token, a cancellation) makes the next step another one
         than the one prepared or started, which is then dropped and run again without that request."""
-        if self.scheduler.waiting:
-            return False
-        following = []
+        following, someone_leaves = [], False
         for request in self.scheduler.running:
             if request.status == RequestStatus.DECODING:
                 if len(request.generated_token_ids) + 1 < request.max_new_tokens:
                     following.append(request.request_id)
+                else:
+                    someone_leaves = True
             elif request.status == RequestStatus.PREFILL:
                 return False
+        # Requests that wait can only join when a place is free: with every place taken and nobody about to leave,
+        # the next step is a decoding step of the same requests all the same.
+        if self.scheduler.waiting and (someone_leaves or len(self.scheduler.running) < self.scheduler.max_batch_size):
+            return False
         if not following or not self.runner.prepare_ahead(following):
             return False
         if self.launch_ahead and pending is not None and following == [request.request_id for request in sampled]:

@@ -149,20 +149,22 @@ def test_engine_refuses_to_run_without_its_kernels(monkeypatch):
         ops.HipOps()
 
 
+@pytest.mark.parametrize("places", [6, 3])
 @pytest.mark.parametrize("temperature", [0.0, 0.8])
-def test_steps_started_ahead_give_the_same_tokens_also_when_requests_stop_unforeseen(temperature):
+def test_steps_started_ahead_give_the_same_tokens_also_when_requests_stop_unforeseen(temperature, places):
     """Decoding steps are started before the host has seen the tokens they bring; an end-of-sequence token makes the
     step that was started another one than the step that follows.  Same tokens, same reasons to stop and every page
     back, with and without starting ahead (bfloat16, requests of different lengths, stops by token and by length)."""
     from llmserver_amd import Engine, load_model
-    print(f"steps started ahead, temperature {temperature}", flush=True)
+    print(f"steps started ahead, temperature {temperature}, {places} places", flush=True)
     case = "A"
     raw, _, page = CASES[case]
     prompts = [random_tokens(raw["vocab_size"], n, 500 + i) for i, n in enumerate((5, 17, 33, 9, 2, 21))]
     limits = [40, 12, 40, 25, 40, 7]
     model = load_model(model_folder(case), "cuda", "bfloat16")
     def make(launch_ahead):
-        return Engine(model, None, max_new_tokens=40, max_batch_size=6, max_num_batched_tokens=128, kv_cache_num_blocks=60,
+        # with three places for six requests some wait while the others decode: steps are started ahead all the same
+        return Engine(model, None, max_new_tokens=40, max_batch_size=places, max_num_batched_tokens=128, kv_cache_num_blocks=60,
                       kv_cache_block_size=page, ignore_eos=False, temperature=temperature, seed=3, launch_ahead=launch_ahead)
     free_run = make(False)
     free = [free_run.add_request(None, prompt_token_ids=prompt, max_new_tokens=limit) for prompt, limit in zip(prompts, limits)]
