@@ -82,11 +82,12 @@ def test_random_configuration_matches_the_plain_implementation(seed, tmp_path):
                 errors.append(float(np.abs(results[(rid, position)] - want).max()) / max(1.0, float(np.abs(want).max())))
         errors = np.asarray(errors)
         assert np.isfinite(errors).all()
+        print(f"  {dtype}: median {np.median(errors):.2e} worst {errors.max():.2e}", flush=True)
         if dtype == "float32":
-            assert errors.max() <= 1e-4, f"{dtype}: {errors.max()} at {int(errors.argmax())}"
+            assert errors.max() <= 1e-5, f"{dtype}: {errors.max()} at {int(errors.argmax())}"
         else:
             # Rounding to 8 bits at a few places per layer: a smooth spread whose median is near one per cent of the
             # largest logit and whose tail stays within a few times that; a fault of the cache or a kernel is not smooth.
-            assert np.median(errors) <= 0.02 and errors.max() <= 0.05, f"{dtype}: median {np.median(errors)} worst {errors.max()}"
+            assert np.median(errors) <= 0.012 and errors.max() <= 0.03, f"{dtype}: median {np.median(errors)} worst {errors.max()}"
         del runner
         torch.cuda.empty_cache()
