@@ -42,8 +42,9 @@ class PendingTokens:
 class Sampler:
     def __init__(self, ops, device):
         self.ops, self.device = ops, torch.device(device)
-        self._host_buffers = []          # pinned buffers the sampled tokens are copied into, used in turn
+        self._host_buffers = []          # pinned buffers (sampled tokens on their way back, temperatures on their way there), used in turn
         self._turn = 0
+        self._greedy = {}                # rows -> zeros on the device for steps without a temperature
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
         """One token per row of ``logits [n, vocab]``; temperature 0 takes the first maximum."""
@@ -53,7 +54,7 @@ class Sampler:
 
     def _host_buffer(self, n: int) -> torch.Tensor:
         pinned = self.device.type == "cuda"
-        if len(self._host_buffers) < 4:
+        if len(self._host_buffers) < 8:
             self._host_buffers.append(torch.empty(max(n, 256), dtype=torch.int32, pin_memory=pinned))
         self._turn = (self._turn + 1) % len(self._host_buffers)
         if self._host_buffers[self._turn].shape[0] < n:
@@ -64,10 +65,17 @@ class Sampler:
         """Start the sampling of one token per row, and the copy of the tokens to the host behind it; whoever reads
         them (``tolist()``) waits for that copy; until then the host is free for other work."""
         n = logits.shape[0]
-        host = np.empty((2, n), dtype=np.float32)
-        host[0] = temperatures
-        host[1] = uniforms
-        both = torch.from_numpy(host).to(self.device, non_blocking=True)
+        if not any(temperatures):
+            both = self._greedy.get(n)               # greedy rows read neither their temperature's inverse nor a number
+            if both is None:
+                both = self._greedy[n] = torch.zeros((2, n), dtype=torch.float32, device=self.device)
+        else:
+            # Through pinned memory: a copy from pageable memory would make the host wait for everything the stream
+            # still has to do, the running step included.
+            staged = self._host_buffer(2 * n).view(torch.float32)[:2 * n].view(2, n)
+            staged[0] = torch.as_tensor(temperatures, dtype=torch.float32)
+            staged[1] = torch.as_tensor(uniforms, dtype=torch.float32)
+            both = staged.to(self.device, non_blocking=True)
         out = torch.empty(n, dtype=torch.int32, device=self.device)
         self.ops.sample(logits, both[0], both[1], out)
         return PendingTokens(out, self._host_buffer(n))
