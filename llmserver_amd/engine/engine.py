@@ -127,12 +127,28 @@ class Engine:
         self.scheduler.waiting.append(request)
         return request
 
-    def _open_cache(self, request: Request) -> None:
+    def _open_cache(self, request: Request, share: bool = True) -> None:
         """Give the request its block tables and state slot and attach cached prefix pages
         (/root/reference/utils/engine.py:197-208)."""
         record = self.kv_cache.open(request.request_id)
         request.block_table = record.tables[0] if record.tables else []
-        self._share_prefix(request)
+        if share:
+            self._share_prefix(request)
+
+    def release_waiting_prefixes(self) -> int:
+        """Take back the cached prefix pages that waiting requests hold (they have computed nothing themselves).  A
+        page that a waiting request holds cannot be evicted, and enough of them leave the running requests without
+        room to grow; given back, the pages stay cached for as long as nobody needs the room, and a request looks
+        its prefix up again when it is up for admission.  Returns the number of pages let go."""
+        let_go = 0
+        for request in self.scheduler.waiting:
+            if request.block_table and self.kv_cache.has(request.request_id):
+                let_go += len(request.block_table)
+                self.step_profile["prefix_hit_tokens"] -= request.num_computed_tokens
+                self.kv_cache.close(request.request_id)
+                request.num_computed_tokens = 0
+                self._open_cache(request, share=False)
+        return let_go
 
     def _share_prefix(self, request: Request) -> None:
         """Attach cached pages of the prompt's prefix.  Done when the request arrives, as in the
@@ -233,11 +249,16 @@ class Engine:
         return min(self.kv_cache.available_pages()) if self.kv_cache.groups else 1 << 30
 
     def schedule_step(self):
+        share = True
         while True:
-            for request in self.scheduler.waiting:      # a preempted request gets a fresh table (and any cached prefix) back
+            # A preempted request gets a fresh table back; the requests that a free place may admit now also look
+            # their prefix up (again): what arrived together with them may have computed it meanwhile.
+            places = self.scheduler.max_batch_size - len(self.scheduler.running)
+            for index, request in enumerate(self.scheduler.waiting):
+                admissible = share and index < places
                 if not self.kv_cache.has(request.request_id):
-                    self._open_cache(request)
-                elif request.num_computed_tokens < len(request.prefix_digests or ()) * self.block_size:
+                    self._open_cache(request, share=admissible)
+                elif admissible and request.num_computed_tokens < len(request.prefix_digests or ()) * self.block_size:
                     self._share_prefix(request)
             available = self.available_blocks()
             out = self.scheduler.plan(available, self.block_size)
@@ -248,6 +269,9 @@ class Engine:
             if needed <= available:
                 self.scheduler.commit(out)
                 return out
+            if share and self.release_waiting_prefixes():
+                share = False             # pages that waiting requests held come first; then running requests are preempted
+                continue
             if len(self.scheduler.running) == 1:
                 raise CacheExhaustedError(f"Required blocks {needed} in KV cache exceeds currently free blocks")
             candidates = [r for r in reversed(self.scheduler.running) if r.block_table]

@@ -334,3 +334,48 @@ def test_requests_that_arrive_together_share_what_the_first_of_them_computed():
     assert second.block_table[:2] == first.block_table[:2]
     assert engine.step_profile["prefix_hit_tokens"] == 8
     engine.kv_cache.check_invariants()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_so_few_pages_that_requests_take_turns_still_ends(seed):
+    """Eight requests, three places, a pool that holds one or two of them: requests are preempted over and over.
+    Waiting requests must not keep the cached pages of their prefixes from the running ones (held pages cannot be
+    evicted), and two requests that do not fit together must not throw each other out for ever: a preempted request
+    comes back when all it has to compute again fits at once.  Everybody finishes with all tokens, in few steps."""
+    import random
+    rng = random.Random(seed)
+    pages = rng.choice((9, 10, 12, 14))
+    engine, script = scripted_engine([], max_new_tokens=8, max_batch_size=3, max_num_batched_tokens=8, kv_cache_num_blocks=pages,
+                                     kv_cache_block_size=2)
+    requests = [engine.add_request(None, [rng.randrange(5, 60) for _ in range(rng.randint(3, 9))]) for _ in range(8)]
+    steps = 0
+    while engine.step():
+        steps += 1
+        engine.kv_cache.check_invariants()
+        assert steps < 200, "requests take turns without getting anywhere"
+    assert all(r.status == RequestStatus.FINISHED and len(r.generated_token_ids) == 8 for r in requests)
+    assert engine.step_profile["preemptions"] > 0
+    assert min(engine.kv_cache.available_pages()) == pages and not engine.kv_cache.requests
+
+
+def test_waiting_requests_give_their_cached_prefix_back_when_pages_run_short():
+    """One place, five pages.  A finished request leaves two cached pages; a waiting request with the same prefix
+    holds them (so they cannot be evicted) while the running request grows to need all five pages: the waiting one
+    gives them back instead of the engine giving up, and computes its prompt itself when its turn comes."""
+    engine, script = scripted_engine([], max_new_tokens=6, max_batch_size=1, max_num_batched_tokens=8, kv_cache_num_blocks=5,
+                                     kv_cache_block_size=2)
+    first = engine.add_request(None, [7, 8, 9, 10, 11], max_new_tokens=1)
+    assert not engine.step() and first.status == RequestStatus.FINISHED      # its two complete pages stay cached
+    assert engine.kv_cache.groups[0].pool.num_idle == 2
+    running = engine.add_request(None, [20, 21, 22, 23, 24])
+    waiting = engine.add_request(None, [7, 8, 9, 10, 12])
+    assert len(waiting.block_table) == 2 and waiting.num_computed_tokens == 4 and engine.step_profile["prefix_hit_tokens"] == 4
+    while running.status != RequestStatus.FINISHED:        # ten tokens in the cache: five pages, two are the waiting request's
+        assert engine.step()
+        engine.kv_cache.check_invariants()
+    assert running.generated_token_ids == [0] * 6 and engine.step_profile["preemptions"] == 0
+    assert waiting.block_table == [] or waiting.status != RequestStatus.WAITING
+    while engine.step():
+        pass
+    assert waiting.status == RequestStatus.FINISHED and len(waiting.generated_token_ids) == 6
+    assert min(engine.kv_cache.available_pages()) == 5 and not engine.kv_cache.requests
