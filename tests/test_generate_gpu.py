@@ -186,3 +186,48 @@ def test_steps_started_ahead_give_the_same_tokens_also_when_requests_stop_unfore
     assert outcomes[0] == outcomes[1]
     reasons = {reason.value for _, reason in outcomes[1]}
     assert len(reasons) == 2, reasons                                        # some stopped by a token, some by their length
+
+
+@pytest.mark.parametrize("case, seed", [("A", 0), ("B", 1), ("C", 2), ("B", 4)])
+def test_requests_arriving_over_time_with_shared_prefixes_and_few_pages(case, seed):
+    """Fourteen requests, half of them behind a common prefix, arrive while others run; places, token budget and
+    pages are few (requests wait, prompts are cut, pages of finished requests are cached and used again, requests
+    are preempted); steps are started ahead or not.  Greedy float32 tokens of every request against the plain
+    implementation."""
+    import random
+    from llmserver_amd import Engine, load_model
+    print(f"arrivals over time {case} {seed}", flush=True)
+    raw, _, page = CASES[case]
+    config, tensors = plain_model(case)
+    model = load_model(model_folder(case), "cuda", "float32")
+    rng = random.Random(seed)
+    prefix = random_tokens(raw["vocab_size"], rng.choice((2 * page, 3 * page + 1, 5 * page)), 900 + seed)
+    prompts, limits = [], []
+    for i in range(14):
+        body = random_tokens(raw["vocab_size"], rng.randint(1, 60), 1000 + 50 * seed + i)
+        prompts.append(prefix + body if rng.random() < 0.5 else body)
+        limits.append(rng.randint(1, 20))
+    expected = [plain.greedy_generate(config, tensors, p, n) for p, n in zip(prompts, limits)]
+    longest = max(len(p) + n for p, n in zip(prompts, limits))
+    preemptions = hits = 0
+    for launch_ahead in (True, False):
+        for pages in (400, -(-longest // page) + rng.choice((1, 3, 8))):
+            engine = Engine(model, None, max_new_tokens=20, max_batch_size=rng.choice((2, 4, 6)), max_num_batched_tokens=rng.choice((16, 32, 128)),
+                            kv_cache_num_blocks=pages, kv_cache_block_size=page, ignore_eos=True, launch_ahead=launch_ahead)
+            order, requests, steps = list(range(len(prompts))), {}, 0
+            while order or engine.scheduler.waiting or engine.scheduler.running:
+                for _ in range(rng.choice((0, 1, 1, 3))):
+                    if order:
+                        i = order.pop(0)
+                        requests[i] = engine.add_request(None, prompt_token_ids=prompts[i], max_new_tokens=limits[i])
+                if engine.scheduler.waiting or engine.scheduler.running:
+                    engine.step()
+                    steps += 1
+                assert steps < 2000
+            engine.kv_cache.check_invariants()
+            assert min(engine.kv_cache.available_pages()) == pages and not engine.kv_cache.requests
+            for i in range(len(prompts)):
+                assert list(requests[i].generated_token_ids) == expected[i], (launch_ahead, pages, i)
+            preemptions += engine.step_profile["preemptions"]
+            hits += engine.step_profile["prefix_hit_tokens"]
+    assert hits > 0
