@@ -102,3 +102,55 @@ def test_long_decoding_and_first_tokens(dtype, tmp_path):
             np.testing.assert_allclose(got, expected[position], err_msg=f"position {position}", **TOLERANCE["float32"])
         else:
             assert float(np.abs(got - expected[position]).max()) <= bf16_atol(expected[position]), position
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_unusual_steps(dtype, tmp_path):
+    """Wanted places out of order and twice; a step with nothing in it; a first token alone; five live requests; a
+    request left out of steps; a name ended and used again for other tokens; an end of somebody unknown; a step
+    that wants nothing (no file)."""
+    import plain_qwen3 as plain
+    from helpers import plain_model
+    case = "B"
+    vocab = CASES[case][0]["vocab_size"]
+    config, tensors = plain_model(case)
+    t = {k: random_tokens(vocab, n, 70 + i) for i, (k, n) in enumerate({"a": 64, "b": 1, "c": 30, "d": 64, "e": 17, "f": 5}.items())}
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": t["a"][:10], "want": [9, 0, 9, 3]}, {"id": "b", "tokens": t["b"], "want": [0]}], "end": ["b", "nobody"]},
+        {"step": 1, "entries": [], "end": []},
+        {"step": 2, "entries": [{"id": "c", "tokens": t["c"][:1], "want": [0]}], "end": []},
+        {"step": 3, "entries": [{"id": "a", "tokens": t["a"][10:12], "want": []}, {"id": "c", "tokens": t["c"][1:2], "want": []}], "end": []},
+        {"step": 4, "entries": [{"id": "c", "tokens": t["c"][2:3], "want": [0]}, {"id": "d", "tokens": t["d"][:1], "want": []},
+                                {"id": "e", "tokens": t["e"][:1], "want": [0]}, {"id": "f", "tokens": t["f"][:1], "want": [0]},
+                                {"id": "a", "tokens": t["a"][12:13], "want": [0]}], "end": ["f"]},
+        {"step": 5, "entries": [{"id": "b", "tokens": t["c"][:7], "want": [6]}], "end": []},
+        {"step": 6, "entries": [{"id": "a", "tokens": t["a"][13:64], "want": [50]}, {"id": "d", "tokens": t["d"][1:64], "want": [62, 0]}],
+         "end": ["a", "d", "e", "b", "c"]},
+        {"step": 7, "entries": [{"id": "a", "tokens": t["d"][:64], "want": [63]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    command = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_folder(case), "--dtype", dtype,
+               "--out", str(out), "--max-tokens", str(5 * 64), "--page-size", "8"]
+    done = subprocess.run(command, input=traces.to_lines(steps), capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    assert done.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+    assert sorted(os.listdir(out)) == ["0.f32", "2.f32", "4.f32", "5.f32", "6.f32", "7.f32"]       # steps 1 and 3 want nothing
+    fed, place = {}, {}
+    for step in steps:
+        wanted = sum(len(e["want"]) for e in step["entries"])
+        rows = np.fromfile(out / f"{step['step']}.f32", dtype="<f4").reshape(wanted, vocab) if wanted else None
+        row = 0
+        for entry in step["entries"]:
+            start = place.get(entry["id"], 0)
+            fed.setdefault(entry["id"], []).extend(entry["tokens"])
+            for want in entry["want"]:
+                expected = plain.forward(config, tensors, fed[entry["id"]]).numpy()[start + want]
+                if dtype == "float32":
+                    np.testing.assert_allclose(rows[row], expected, err_msg=f"step {step['step']} {entry['id']} place {want}", **TOLERANCE["float32"])
+                else:
+                    assert float(np.abs(rows[row] - expected).max()) <= bf16_atol(expected), (step["step"], entry["id"], want)
+                row += 1
+            place[entry["id"]] = start + len(entry["tokens"])
+        for name in step["end"]:
+            place.pop(name, None)
+            fed.pop(name, None)
