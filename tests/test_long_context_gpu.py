@@ -41,7 +41,6 @@ def sharp_model(tmp_path_factory):
     with torch.no_grad():
         expected = {"main": plain.forward(config, tensors, main).numpy()}
         expected.update({rid: plain.forward(config, tensors, tokens).numpy() for rid, tokens in others.items()})
-    # the oracle's own softmax is as sharp as intended: the largest probability of a late query is far above 1 / context
     return folder, main, others, expected
 
 
