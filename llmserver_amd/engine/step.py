@@ -12,6 +12,11 @@ everything that changes from the staged arrays, whose addresses and shapes stay 
 steps are filled up with rows of nobody's to one of a few sizes, so that few graphs serve every batch.  The
 reference replays its decode pass from a CUDA graph in the same way
 (/root/reference/utils/cuda_graph.py:51-99).
+
+Such a step can be laid out on the host while the GPU still runs the step before it (``prepare_ahead``: everything but
+the token ids is known then), and started before the host has seen those tokens (``launch_ahead``: the ids are copied
+on the device from the sampler's output); ``step`` then finds its work done, or drops it if the step that comes is
+another one.
 """
 from __future__ import annotations
 
