@@ -76,7 +76,10 @@ constexpr int NS = D / 16;                   // 16-dim steps (four 16x16x4 MFMAs
 // no branch stands between the loads of the item's start (a load inside a branch makes every later wait a wait
 // for everything).
 // PLAIN: the step has both norm weights and a rotation (then nothing of the fused start depends on a flag).
-template <int MODE, bool PLAIN>
+// WG_MERGE: the four items of a workgroup are the four key ranges of one tile (the plan says so), and the workgroup
+// merges them itself through LDS and writes the output: no partial results in memory, no merge launch.  For steps
+// whose contexts are short, where that launch costs as much as the attention.
+template <int MODE, bool PLAIN, bool WG_MERGE>
 __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
     const elem_t* keys, const elem_t* values,
@@ -86,14 +89,15 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     float* __restrict__ part_acc, float* __restrict__ part_ml, Geometry g, DecodeFusion fusion) {
     const int lane = threadIdx.x & 63;
     const int item_index = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item_index >= n_items) return;
+    if (!WG_MERGE && item_index >= n_items) return;      // with WG_MERGE every wavefront has to reach the barrier at the end
     // The start of an item is a chain of loads, each of which needs the one before it (the item, its row, the row's
     // queries and table entries, the first keys).  Every link costs a trip to memory, so everything that can be
     // asked for is asked for as soon as its address is known, in the order in which it will be needed, and nothing
     // is used before all of it is under way: three trips (item; row, table entries and norm weights; queries,
     // rotation and first keys and values) instead of one per array.
-    const Item item = items[item_index];
-    const int slot = item_slot[item_index];                    // needed at the very end only
+    Item item = items[min(item_index, n_items - 1)];
+    if (WG_MERGE && item_index >= n_items) item.k_begin = item.k_end;      // (the launcher refuses such a launch) no keys, no weight
+    const int slot = item_slot[min(item_index, n_items - 1)];  // needed at the very end only
     const int kv_head = blockIdx.y / g.gtiles, gtile = blockIdx.y % g.gtiles;
     const int col = lane & 15, quad = lane >> 4;
     const int row = item.row;
@@ -499,6 +503,50 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
 
     run_sum += __shfl_xor(run_sum, 16, 64);
     run_sum += __shfl_xor(run_sum, 32, 64);
+    if constexpr (WG_MERGE) {
+        // Every wavefront of the workgroup gets here (the launch has no workgroup with fewer than four items, and
+        // nothing above returns): wavefronts 1 to 3 leave their sums in LDS, wavefront 0 adds them up by log-sum-exp.
+        __shared__ f32x4 others_acc[3][ND][64];
+        __shared__ float ranges_max[4][16], ranges_sum[4][16];
+        const int wave = threadIdx.x >> 6;
+        if (quad == 0) {
+            ranges_max[wave][col] = run_max;
+            ranges_sum[wave][col] = run_sum;
+        }
+        if (wave > 0) {
+#pragma unroll
+            for (int c = 0; c < ND; ++c) others_acc[wave - 1][c][lane] = acc[c];
+        }
+        __syncthreads();
+        if (wave > 0 || !pair_valid) return;
+        float top = NEG_INF;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) top = fmaxf(top, ranges_max[w][col]);
+        float weight[4], total = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float m = ranges_max[w][col];
+            weight[w] = m == NEG_INF ? 0.f : expf(m - top);
+            total += weight[w] * ranges_sum[w][col];
+        }
+        const float inv = total > 0.f ? 1.f / total : 0.f;
+        elem_t* o = out + ((size_t)(token0 + pair_token) * g.n_q + head) * D + 4 * quad;
+#pragma unroll
+        for (int c = 0; c < ND; ++c) {
+            f32x4 sum = acc[c] * weight[0];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) sum += others_acc[w - 1][c][lane] * weight[w];
+#if LSA_BF16
+            bf16x4 r4;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) r4[r] = (bf16_t)(sum[r] * inv);
+            *reinterpret_cast<bf16x4*>(o + 16 * c) = r4;
+#else
+            *reinterpret_cast<f32x4*>(o + 16 * c) = sum * inv;
+#endif
+        }
+        return;
+    }
     if (!pair_valid) return;
     if (slot < 0) {
         const float inv = run_sum > 0.f ? 1.f / run_sum : 0.f;
@@ -964,7 +1012,7 @@ LSA_EXPORT int lsa_paged_attention(
     const void* merges, int n_merges, int n_slots, float* part_acc, float* part_ml, const void* tiles, int n_tiles, float scale,
     int window, int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
     int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, int tiles_per_workgroup,
-    hipStream_t stream) {
+    int merge_in_workgroup, hipStream_t stream) {
     if (n_items <= 0 && n_tiles <= 0) return 0;
     // decode_fusion (see DecodeFusion::mode): the caller promises that every row of the step brings one token.
     DecodeFusion fusion = {q_weight, k_weight, cos_sin, norm_eps, decode_fusion};
@@ -994,19 +1042,31 @@ LSA_EXPORT int lsa_paged_attention(
 #endif
     }
     if (n_items <= 0) return 0;
+    // merge_in_workgroup: items 4 i .. 4 i + 3 are the four key ranges of one tile (some may be empty), no item has a
+    // slot, nothing is left to merge.
+    if (merge_in_workgroup && (n_items % 4 != 0 || n_merges != 0)) return -1;
     dim3 grid((n_items + 3) / 4, n_kv * gtiles);
-#define LSA_LAUNCH_ITEMS(MODE, PLAIN) paged_attention_kernel<MODE, PLAIN><<<grid, 256, 0, stream>>>( \
+#define LSA_LAUNCH_ITEMS(MODE, PLAIN) LSA_LAUNCH_ITEMS_MERGE(MODE, PLAIN, false)
+#define LSA_LAUNCH_ITEMS_MERGE(MODE, PLAIN, WG_MERGE) paged_attention_kernel<MODE, PLAIN, WG_MERGE><<<grid, 256, 0, stream>>>( \
         (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride, \
         row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g, fusion)
 #if LSA_BF16
     const bool plain = q_weight != nullptr && cos_sin != nullptr;
-    if (decode_fusion == 3 && plain) LSA_LAUNCH_ITEMS(3, true);
+    if (merge_in_workgroup && decode_fusion && !plain) return -1;      // the caller asks lsa_attention_merges_in_workgroup first
+    if (merge_in_workgroup && decode_fusion == 3) LSA_LAUNCH_ITEMS_MERGE(3, true, true);
+    else if (merge_in_workgroup && decode_fusion == 1) LSA_LAUNCH_ITEMS_MERGE(1, true, true);
+    else if (merge_in_workgroup) LSA_LAUNCH_ITEMS_MERGE(0, false, true);
+    else if (decode_fusion == 3 && plain) LSA_LAUNCH_ITEMS(3, true);
     else if (decode_fusion == 3) LSA_LAUNCH_ITEMS(3, false);
     else if (decode_fusion == 1 && plain) LSA_LAUNCH_ITEMS(1, true);
     else if (decode_fusion == 1) LSA_LAUNCH_ITEMS(1, false);
     else
+#else
+    if (merge_in_workgroup) LSA_LAUNCH_ITEMS_MERGE(0, false, true);
+    else
 #endif
     LSA_LAUNCH_ITEMS(0, false);
+#undef LSA_LAUNCH_ITEMS_MERGE
 #undef LSA_LAUNCH_ITEMS
     int err = (int)hipGetLastError();
     if (err || n_merges <= 0) return err;

@@ -288,14 +288,15 @@ class Engine:
         afterwards (/root/reference/utils/engine.py:150-161).  The graphs serve contexts up to the first width of the
         block table, or, with ``max_context``, every width up to that context (the pool has to hold that many tokens
         for every row meanwhile; sizes it cannot hold are left to be captured when they are met)."""
-        from .step import TABLE_WIDTH_STEP
+        from .step import SHORT_CONTEXT, TABLE_WIDTH_STEP
         if not self.runner.use_graphs or self.active_requests:
             return 0
         most = self.scheduler.max_batch_size
         if batch_sizes is None:
             batch_sizes = sorted({min(most, padded_rows(rows)) for rows in range(1, most + 1)})
         tokens_per_width = TABLE_WIDTH_STEP * self.block_size
-        contexts = [1] + [width * tokens_per_width + 1 for width in range(1, -(-(max_context or 1) // tokens_per_width))]
+        # one token (the shape of short contexts), the first context that is not short, then every width of the table
+        contexts = [1, SHORT_CONTEXT + 1] + [width * tokens_per_width + 1 for width in range(1, -(-(max_context or 1) // tokens_per_width))]
         try:
             for context in contexts:
                 pages_per_row = -(-context // self.block_size)

@@ -31,6 +31,8 @@ from ..cache.manager import CacheManager
 from .batch import Staging, StepContext, StepEntry
 
 TABLE_WIDTH_STEP = 64      # captured steps serve block tables up to the next multiple of this many pages
+SHORT_CONTEXT = 512        # captured steps whose contexts all stay within this are a shape of their own (``ctx.short_contexts``):
+                           # mixers may then do with less machinery (attention merges its key ranges inside its workgroups)
 MAX_GRAPHS = 96
 
 
@@ -144,17 +146,18 @@ class ModelRunner:
     def _graph_key(self, entries: Sequence[StepEntry]):
         if not self.use_graphs or any(len(entry.tokens) != 1 for entry in entries):
             return None
-        blocks = 1
+        longest = 1
         for entry in entries:
             record = self.cache.requests.get(entry.request_id)
             if record is None:
                 return None
-            blocks = max(blocks, -(-(record.num_computed + 1) // self.cache.page_size))
+            longest = max(longest, record.num_computed + 1)
+        blocks = -(-longest // self.cache.page_size)
         width = -(-blocks // TABLE_WIDTH_STEP) * TABLE_WIDTH_STEP
         rows, wanted = len(entries), sum(len(entry.want) for entry in entries)
         if all(len(entry.want) == 1 for entry in entries):
             rows = wanted = padded_rows(rows)          # decoding: filled up to one of a few sizes
-        return (rows, width, wanted)
+        return (rows, width, wanted, longest <= SHORT_CONTEXT)
 
     @torch.inference_mode()
     def prepare_ahead(self, request_ids: Sequence[object]) -> bool:
@@ -181,6 +184,7 @@ class ModelRunner:
         except BufferError:          # no page for one of them: the step itself will say so, or the caller makes room
             return False
         ctx.static_max_keys = key[1] * self.cache.page_size
+        ctx.short_contexts = key[3]
         self.model.prepare(ctx)
         ctx.stage()
         if ctx.layout != captured.layout:
@@ -258,6 +262,7 @@ class ModelRunner:
         ctx = self.build_context(entries, staging=staging, table_width=key[1], filler_rows=key[0] - len(entries))
         wanted = sum(len(entry.want) for entry in entries)           # the fillers' logits come last and are dropped
         ctx.static_max_keys = key[1] * self.cache.page_size
+        ctx.short_contexts = key[3]
         self.model.prepare(ctx)
         if captured is None:
             ctx.static_max_keys = None           # the first upload may size the staging buffer

@@ -547,6 +547,11 @@ class HipOps:
             if cos_sin is not None:
                 _check(cos_sin, "cos_sin", torch.float32, (n, head_dim))
             fusion_mode = 3 if write_cache else 1
+        merge_in_workgroup = int(bool(plan.get("merge_in_workgroup", 0)))
+        if merge_in_workgroup and (n_items % 4 or n_merges or n_slots or n_tiles or n != rows
+                                   or (decode_fusion is not None and (q_weight is None or cos_sin is None))):
+            raise ValueError("merging in the workgroup takes steps of one token per row whose plan gives every tile four key ranges "
+                             "and no slots, and, with decode fusion, both norm weights and a rotation")
         lib = self._attention_library(qkv.dtype, head_dim)
         if plan.get("most_splits", 0) > lib.lsa_attention_most_splits():
             raise ValueError(f"the plan splits a tile's keys into {plan['most_splits']} ranges, the merge kernel takes {lib.lsa_attention_most_splits()}")
@@ -555,7 +560,7 @@ class HipOps:
             _ptr(row_len), _ptr(row_ctx), _ptr(plan["items"]), _ptr(plan["item_slot"]), n_items, _ptr(plan["merges"]),
             n_merges, n_slots, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), n_tiles, float(scale), int(window) if window else 0,
             page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, fusion_mode, _ptr(q_weight), _ptr(k_weight), float(norm_eps),
-            _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), _stream()), "paged_attention")
+            _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), merge_in_workgroup, _stream()), "paged_attention")
 
     def sample(self, logits, temperature, uniform, out):
         n, vocab = logits.shape

@@ -56,6 +56,7 @@ class AttentionPlan:
         self.items, self.item_slot, self.merges, self.n_slots = items, item_slot, merges, n_slots
         self.tiles = tiles if tiles is not None else np.zeros((0, 4), dtype=np.int32)
         self.tiles_per_workgroup = tiles_per_workgroup
+        self.merge_in_workgroup = False      # items 4 i .. 4 i + 3 are one tile's key ranges, merged by their workgroup
 
 
 def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: int, target_waves: int = TARGET_WAVES) -> int:
@@ -97,7 +98,11 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
     return most if estimate(most, 2.75, 1.40) < estimate(4, 2.0, 1.37) else 4
 
 
-def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int) -> AttentionPlan:
+WORKGROUP_RANGES = 4    # key ranges of a tile that one workgroup (four wavefronts) walks and merges itself
+SHORT_CONTEXT = 512     # up to this context a step of single tokens is merged in its workgroups (measured against the merge launch)
+
+
+def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, merge_in_workgroup: bool = False) -> AttentionPlan:
     """The plan of a step in which every row brings one token and every tile gets ``splits`` key ranges: what the
     loop of :func:`build_attention_plan` makes for it, row by row, computed for all rows at once (a decode step of
     many rows is planned thousands of times a second)."""
@@ -106,11 +111,13 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int) 
     k_end = row_ctx
     k_begin = np.zeros_like(k_end) if window is None else np.maximum(0, k_end - window)
     zeros = np.zeros_like(rows)
-    if splits <= 1:
+    if splits <= 1 and not merge_in_workgroup:
         items = np.stack([rows, zeros, k_begin, k_end], axis=1).astype(np.int32)
         return AttentionPlan(items, np.full(n_rows, -1, dtype=np.int32), np.zeros((0, 4), dtype=np.int32), 0)
+    if merge_in_workgroup:          # four items a tile; with fewer ranges wanted, the last ones come out empty
+        ranges, splits = max(1, min(splits, WORKGROUP_RANGES)), WORKGROUP_RANGES
     start = (k_begin // KEY_ALIGN) * KEY_ALIGN
-    per = -(-(k_end - start) // splits)
+    per = -(-(k_end - start) // (ranges if merge_in_workgroup else splits))
     per = -(-per // KEY_ALIGN) * KEY_ALIGN
     piece = start[:, None] + np.arange(splits, dtype=np.int64)[None, :] * per[:, None]
     lo = np.maximum(piece, k_begin[:, None])
@@ -120,13 +127,17 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int) 
     last = np.where(inside, np.maximum(lo, hi), k_end[:, None])
     items = np.stack([np.repeat(rows, splits), np.zeros(n_rows * splits, dtype=np.int64), first.reshape(-1), last.reshape(-1)],
                      axis=1).astype(np.int32)
+    if merge_in_workgroup:          # the four items of a tile are one workgroup's: no slots, nothing left to merge
+        plan = AttentionPlan(items, np.full(n_rows * splits, -1, dtype=np.int32), np.zeros((0, 4), dtype=np.int32), 0)
+        plan.merge_in_workgroup = True
+        return plan
     merges = np.stack([rows, zeros, rows * splits, np.full(n_rows, splits, dtype=np.int64)], axis=1).astype(np.int32)
     return AttentionPlan(items, np.arange(n_rows * splits, dtype=np.int32), merges, n_rows * splits)
 
 
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
-                         workgroup_tiles: int = 0, single_token_shortcut: bool = True) -> AttentionPlan:
+                         workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: bool = False) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
@@ -136,8 +147,11 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
-    if single_token_shortcut and fixed_splits is not None and len(row_len) and int(row_len.min()) == 1 == int(row_len.max()):
-        return _single_token_plan(row_ctx, window, int(fixed_splits))
+    if merge_in_workgroup and not (len(row_len) and int(row_len.min()) == 1 == int(row_len.max())):
+        raise ValueError("key ranges are merged in the workgroup only in steps of one token per row")
+    if (merge_in_workgroup or (single_token_shortcut and fixed_splits is not None)) and len(row_len) \
+            and int(row_len.min()) == 1 == int(row_len.max()):
+        return _single_token_plan(row_ctx, window, int(fixed_splits or WORKGROUP_RANGES), merge_in_workgroup)
     tiles_per_row = -(-row_len // tokens_per_tile)
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
     items, slots, merges, tiles = [], [], [], []
@@ -244,15 +258,23 @@ class GQAttention(Mixer):
         fixed = None
         if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
             fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys)
+        # Short contexts (the step says so, and keeps saying so for as long as its shape is replayed): four key ranges
+        # a tile, which the workgroup that walks them merges itself.
+        # So does a step with so many rows that a tile gets four ranges anyway: the merge launch is all that differs.
+        # (With two or three ranges a tile, half of a workgroup's wavefronts would idle through the others' walk:
+        # measured at 64 rows behind 4,096 tokens, a tenth slower than with the merge launch.)
+        in_workgroup = ctx.n_tokens == ctx.n_rows and (bool(getattr(ctx, "short_contexts", False)) or fixed == WORKGROUP_RANGES)
+        if in_workgroup and getattr(ctx, "short_contexts", False):
+            fixed = WORKGROUP_RANGES
         import torch
         per_workgroup = getattr(ctx.ops, "attention_workgroup_tiles", None)
         per_workgroup = per_workgroup(ctx.dtype, self.head_dim) if per_workgroup is not None else 0
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
-                                    fixed_splits=fixed, workgroup_tiles=per_workgroup)
+                                    fixed_splits=fixed, workgroup_tiles=per_workgroup, merge_in_workgroup=in_workgroup)
         ctx.set_plan(key, {
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
             "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),
-            "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup,
+            "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup, "merge_in_workgroup": int(plan.merge_in_workgroup),
             "most_splits": int(plan.merges[:, 3].max()) if len(plan.merges) else 0,
         })
 
@@ -264,7 +286,10 @@ class GQAttention(Mixer):
         # A step of single tokens: the attention kernel does the norm, the rotation and the cache write itself.
         fits = getattr(ctx.ops, "decode_fusion_fits", None)
         fusion = None
-        if fits is not None and ctx.n_tokens == ctx.n_rows and fits(qkv.dtype, self.head_dim):
+        # (the kernel that merges a tile's key ranges in its workgroup fuses only the whole of norm and rotation)
+        whole = self.q_norm_weight is not None and cos_sin is not None
+        if fits is not None and ctx.n_tokens == ctx.n_rows and fits(qkv.dtype, self.head_dim) \
+                and (whole or not ctx.get_plan(self.plan_key()).get("merge_in_workgroup")):
             fusion = (self.q_norm_weight, self.k_norm_weight, eps, cos_sin, cache.writable)
         else:
             ctx.ops.qk_norm_rope_kv_write(

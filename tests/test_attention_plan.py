@@ -107,6 +107,28 @@ def test_plan_of_single_tokens_made_at_once_equals_the_plan_made_row_by_row(seed
     assert fast.n_slots == slow.n_slots and fast.tiles_per_workgroup == slow.tiles_per_workgroup
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_plan_whose_key_ranges_are_merged_in_the_workgroup(seed):
+    """Four items a row, in the row's order, without slots or merges; the ranges follow one another from the first key
+    the token may see to itself, at multiples of KEY_ALIGN; empty ranges lie at the end."""
+    rng = random.Random(seed)
+    rows = rng.randint(1, 70)
+    contexts = [rng.choice((1, 2, 31, 32, 33, 64, 100, 300, 511, 512, 513, 1024, rng.randint(1, 2000))) for _ in range(rows)]
+    window = rng.choice((None, None, 1, 40, 700))
+    plan = build_attention_plan([1] * rows, contexts, rng.choice((1, 4, 20)), rng.choice((1, 8)), window, fixed_splits=rng.choice((None, 1, 16)),
+                                merge_in_workgroup=True)
+    assert plan.merge_in_workgroup and plan.items.shape == (4 * rows, 4) and plan.n_slots == 0 and plan.merges.shape == (0, 4)
+    assert (plan.item_slot == -1).all() and plan.tiles.shape == (0, 4)
+    for row, context in enumerate(contexts):
+        ranges = plan.items[4 * row:4 * row + 4].tolist()
+        assert all(r == row and q0 == 0 for r, q0, _, _ in ranges)
+        first = 0 if window is None else max(0, context - window)
+        filled = [(b, e) for _, _, b, e in ranges if b < e]
+        assert filled and filled[0][0] == first and filled[-1][1] == context
+        assert all(a[1] == b[0] and b[0] % KEY_ALIGN == 0 for a, b in zip(filled, filled[1:]))
+        assert [(b, e) for _, _, b, e in ranges][len(filled):] == [(context, context)] * (4 - len(filled))
+
+
 def test_four_or_eight_tiles_per_workgroup():
     """One short prompt is bounded by its longest workgroup and takes four tiles per workgroup; long rows and many rows
     keep every compute unit busy and take eight; a kernel that offers only four gets four."""

@@ -88,11 +88,11 @@ def test_graphs_captured_ahead_change_nothing():
                       kv_cache_block_size=page, ignore_eos=True)
     plain_run = engine().generate(prompts)
     warmed = engine()
-    assert warmed.warmup_graphs() == 4                                   # 1, 2, 3 and 4 rows
+    assert warmed.warmup_graphs() == 5                                   # 1, 2, 3 and 4 rows of short contexts; 1 row beyond them
     assert min(warmed.kv_cache.available_pages()) == 40 and not warmed.kv_cache.requests
     replays = warmed.runner.graph_replays
     assert warmed.generate(prompts) == plain_run
-    assert warmed.runner.graph_replays > replays and warmed.runner.graph_count() == 4     # no further capture was needed
+    assert warmed.runner.graph_replays > replays and warmed.runner.graph_count() == 5     # no further capture was needed
     # decoding steps were laid out, most of them also started, while the step before them ran
     assert warmed.runner.steps_prepared_ahead + warmed.runner.steps_launched_ahead >= 6 and warmed.runner.steps_launched_ahead >= 3
     assert min(warmed.kv_cache.available_pages()) == 40 and not warmed.kv_cache.requests
@@ -102,8 +102,10 @@ def test_graphs_captured_ahead_change_nothing():
     # longer contexts: a graph for every width of the block table up to the context, where the pool can hold the rows
     roomy = Engine(model, None, max_new_tokens=10, max_batch_size=4, max_num_batched_tokens=64, kv_cache_num_blocks=200,
                    kv_cache_block_size=page, ignore_eos=True)
-    assert roomy.warmup_graphs(batch_sizes=(1, 2, 4), max_context=64 * page + 70) == 5    # 1, 2, 4 rows; 1 and 2 rows behind 64 pages
-    assert sorted(key[:2] for key in roomy.runner._graphs) == [(1, 64), (1, 128), (2, 64), (2, 128), (4, 64)]
+    # 1, 2, 4 rows of short contexts, the same beyond them, 1 and 2 rows behind 64 pages
+    assert roomy.warmup_graphs(batch_sizes=(1, 2, 4), max_context=64 * page + 70) == 8
+    assert sorted((key[0], key[1], key[3]) for key in roomy.runner._graphs) == [
+        (1, 64, False), (1, 64, True), (1, 128, False), (2, 64, False), (2, 64, True), (2, 128, False), (4, 64, False), (4, 64, True)]
     assert min(roomy.kv_cache.available_pages()) == 200 and not roomy.kv_cache.requests
     assert roomy.generate(prompts) == plain_run
     roomy.kv_cache.check_invariants()

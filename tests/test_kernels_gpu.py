@@ -137,7 +137,8 @@ def test_qk_norm_rope_kv_write(ops, dtype, n_q, n_kv, d, page):
             assert not got_k.any() and not got_v.any()
 
 
-def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, needle=True, seed=0, target_waves=None, workgroup_tiles=None):
+def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, needle=True, seed=0, target_waves=None, workgroup_tiles=None,
+                   merge_in_workgroup=False):
     """Random q/k/v through both implementations.  Pages are handed out in scrambled order from a
     pool that first held other data (as if used before).  With ``needle``, one far key per request
     is made to dominate its first query's softmax."""
@@ -179,13 +180,15 @@ def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, need
         assert workgroup_tiles <= most
         attention_module._workgroup_tiles_that_pay = lambda *args, **kwargs: workgroup_tiles
     try:
-        plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, workgroup_tiles=most,
+        plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, workgroup_tiles=0 if merge_in_workgroup else most,
+                                    merge_in_workgroup=merge_in_workgroup,
                                     **({} if target_waves is None else {"target_waves": target_waves}))
     finally:
         attention_module._workgroup_tiles_that_pay = chooser
     staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
               "merges": torch.from_numpy(plan.merges).to(DEV), "tiles": torch.from_numpy(plan.tiles).to(DEV), "n_tiles": len(plan.tiles),
-              "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup}
+              "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup,
+              "merge_in_workgroup": int(plan.merge_in_workgroup)}
     t = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
     got = torch.zeros(tokens, n_q * d, device=DEV, dtype=dtype)
     ref = torch.zeros_like(got)
@@ -209,6 +212,23 @@ def test_attention_mixed_batch(ops, dtype, n_q, n_kv, d, page):
     ctxs = [1, 33, 300, 17, 140, 65, 1025]
     plan, _ = attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, seed=n_q * d)
     assert plan.n_slots > 0                                     # long contexts of single tokens were split
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (6, 2, 48, 12), (32, 8, 128, 16), (5, 1, 80, 8), (20, 1, 64, 16), (2, 1, 256, 64)])
+@pytest.mark.parametrize("window", [None, 40])
+def test_attention_key_ranges_merged_in_the_workgroup(ops, dtype, n_q, n_kv, d, page, window):
+    """Steps of single tokens whose tiles get four key ranges each, walked by the four wavefronts of one workgroup and
+    merged there (no partial results, no merge launch): contexts of one token (three ranges empty), at the edges of
+    pages and key steps, with a far key that decides the first query; queries and keys prepared by the separate kernel."""
+    print(f"attention merged in the workgroup {dtype} {n_q}/{n_kv} d{d} page{page} window {window}", flush=True)
+    ctxs = [1, 2, 3, 4, 5, 31, 32, 33, 63, 64, 65, 127, 128, 129, 300, 511, 512, 1025]
+    plan, ref = attention_case(ops, dtype, n_q, n_kv, d, page, [1] * len(ctxs), ctxs, window=window, seed=n_q * d + 1, merge_in_workgroup=True)
+    assert plan.merge_in_workgroup and len(plan.items) == 4 * len(ctxs) and plan.n_slots == 0 and len(plan.merges) == 0
+    if window is None:
+        assert float(ref[-1, :d].float().mean()) > 5.0           # the far key won the last row's first head
+    with pytest.raises(ValueError):                              # a row of two tokens
+        build_attention_plan([1, 2], [5, 9], n_q // n_kv, n_kv, window, merge_in_workgroup=True)
 
 
 @pytest.mark.parametrize("n_q, n_kv, d, page", [(32, 8, 128, 16), (4, 2, 64, 8), (20, 1, 64, 16), (6, 3, 192, 12), (2, 1, 256, 64)])
@@ -250,13 +270,16 @@ def test_attention_decode_fusion(ops, n_q, n_kv, d, page, window):
     inv_freq = (1.0 / (1e6 ** (torch.arange(0, d, 2).float() / d))).to(DEV)
     cos_sin = ops.rotary_table(positions, inv_freq)
     scale = d ** -0.5
-    for fixed in (None, 8):
-        plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, fixed_splits=fixed)
+    for fixed in (None, 8, "in the workgroup"):
+        in_workgroup = fixed == "in the workgroup"                           # four key ranges a tile, merged by the workgroup that walks them
+        plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, fixed_splits=8 if in_workgroup else fixed,
+                                    merge_in_workgroup=in_workgroup)
         staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
                   "merges": torch.from_numpy(plan.merges).to(DEV), "n_items": len(plan.items), "n_merges": len(plan.merges),
-                  "n_slots": plan.n_slots}
-        assert plan.n_slots > 0 or window is not None                       # long contexts are split, unless a window keeps them short
-        for norm, rope in ((True, True), (False, True), (True, False)):
+                  "n_slots": plan.n_slots, "merge_in_workgroup": int(plan.merge_in_workgroup)}
+        assert plan.n_slots > 0 or window is not None or in_workgroup        # long contexts are split, unless a window keeps them short
+        assert not in_workgroup or (len(plan.items) == 4 * rows and plan.n_slots == 0 and not len(plan.merges))
+        for norm, rope in ((True, True),) if in_workgroup else ((True, True), (False, True), (True, False)):
             w_q, w_k, cs = (qw if norm else None), (kw if norm else None), (cos_sin if rope else None)
             # the separate kernels, and the plain twin of both
             sep_qkv, sep_k, sep_v = qkv.clone(), keys0.clone(), values0.clone()
