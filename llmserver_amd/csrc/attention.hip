@@ -76,10 +76,11 @@ constexpr int NS = D / 16;                   // 16-dim steps (four 16x16x4 MFMAs
 // no branch stands between the loads of the item's start (a load inside a branch makes every later wait a wait
 // for everything).
 // PLAIN: the step has both norm weights and a rotation (then nothing of the fused start depends on a flag).
-// WG_MERGE: the four items of a workgroup are the four key ranges of one tile (the plan says so), and the workgroup
-// merges them itself through LDS and writes the output: no partial results in memory, no merge launch.  For steps
-// whose contexts are short, where that launch costs as much as the attention.
-template <int MODE, bool PLAIN, bool WG_MERGE>
+// WG_RANGES (0, 2 or 4): the four items of a workgroup are the four key ranges of one tile, or the two ranges of each
+// of two tiles (the plan says so), and the workgroup merges them itself through LDS and writes the output: no partial
+// results in memory, no merge launch.  For steps whose contexts are short, where that launch costs as much as the
+// attention, and for steps of many rows, whose tiles get no more ranges than that anyway.
+template <int MODE, bool PLAIN, int WG_RANGES>
 __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
     const elem_t* keys, const elem_t* values,
@@ -89,6 +90,7 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     float* __restrict__ part_acc, float* __restrict__ part_ml, Geometry g, DecodeFusion fusion) {
     const int lane = threadIdx.x & 63;
     const int item_index = blockIdx.x * 4 + (threadIdx.x >> 6);
+    constexpr bool WG_MERGE = WG_RANGES > 0;
     if (!WG_MERGE && item_index >= n_items) return;      // with WG_MERGE every wavefront has to reach the barrier at the end
     // The start of an item is a chain of loads, each of which needs the one before it (the item, its row, the row's
     // queries and table entries, the first keys).  Every link costs a trip to memory, so everything that can be
@@ -505,29 +507,31 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     run_sum += __shfl_xor(run_sum, 32, 64);
     if constexpr (WG_MERGE) {
         // Every wavefront of the workgroup gets here (the launch has no workgroup with fewer than four items, and
-        // nothing above returns): wavefronts 1 to 3 leave their sums in LDS, wavefront 0 adds them up by log-sum-exp.
-        __shared__ f32x4 others_acc[3][ND][64];
+        // nothing above returns).  The wavefronts of a tile are neighbours: all but the first leave their sums in LDS,
+        // the first adds them up by log-sum-exp.
+        constexpr int R = WG_RANGES > 0 ? WG_RANGES : 1, TILES = 4 / R;
+        __shared__ f32x4 others_acc[4 - TILES][ND][64];
         __shared__ float ranges_max[4][16], ranges_sum[4][16];
-        const int wave = threadIdx.x >> 6;
+        const int wave = threadIdx.x >> 6, first_wave = wave / R * R, member = wave - first_wave;
         if (quad == 0) {
             ranges_max[wave][col] = run_max;
             ranges_sum[wave][col] = run_sum;
         }
-        if (wave > 0) {
+        if (member > 0) {
 #pragma unroll
-            for (int c = 0; c < ND; ++c) others_acc[wave - 1][c][lane] = acc[c];
+            for (int c = 0; c < ND; ++c) others_acc[first_wave / R * (R - 1) + member - 1][c][lane] = acc[c];
         }
         __syncthreads();
-        if (wave > 0 || !pair_valid) return;
+        if (member > 0 || !pair_valid) return;
         float top = NEG_INF;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) top = fmaxf(top, ranges_max[w][col]);
-        float weight[4], total = 0.f;
+        for (int w = 0; w < R; ++w) top = fmaxf(top, ranges_max[first_wave + w][col]);
+        float weight[R], total = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float m = ranges_max[w][col];
+        for (int w = 0; w < R; ++w) {
+            const float m = ranges_max[first_wave + w][col];
             weight[w] = m == NEG_INF ? 0.f : expf(m - top);
-            total += weight[w] * ranges_sum[w][col];
+            total += weight[w] * ranges_sum[first_wave + w][col];
         }
         const float inv = total > 0.f ? 1.f / total : 0.f;
         elem_t* o = out + ((size_t)(token0 + pair_token) * g.n_q + head) * D + 4 * quad;
@@ -535,7 +539,7 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
         for (int c = 0; c < ND; ++c) {
             f32x4 sum = acc[c] * weight[0];
 #pragma unroll
-            for (int w = 1; w < 4; ++w) sum += others_acc[w - 1][c][lane] * weight[w];
+            for (int w = 1; w < R; ++w) sum += others_acc[first_wave / R * (R - 1) + w - 1][c][lane] * weight[w];
 #if LSA_BF16
             bf16x4 r4;
 #pragma unroll
@@ -1042,27 +1046,31 @@ LSA_EXPORT int lsa_paged_attention(
 #endif
     }
     if (n_items <= 0) return 0;
-    // merge_in_workgroup: items 4 i .. 4 i + 3 are the four key ranges of one tile (some may be empty), no item has a
-    // slot, nothing is left to merge.
-    if (merge_in_workgroup && (n_items % 4 != 0 || n_merges != 0)) return -1;
+    // merge_in_workgroup (0, 2 or 4 ranges a tile): items 4 i .. 4 i + 3 are the four key ranges of one tile, or the two
+    // ranges of each of two tiles (some may be empty), no item has a slot, nothing is left to merge.
+    if (merge_in_workgroup && ((merge_in_workgroup != 2 && merge_in_workgroup != 4) || n_items % 4 != 0 || n_merges != 0)) return -1;
     dim3 grid((n_items + 3) / 4, n_kv * gtiles);
-#define LSA_LAUNCH_ITEMS(MODE, PLAIN) LSA_LAUNCH_ITEMS_MERGE(MODE, PLAIN, false)
-#define LSA_LAUNCH_ITEMS_MERGE(MODE, PLAIN, WG_MERGE) paged_attention_kernel<MODE, PLAIN, WG_MERGE><<<grid, 256, 0, stream>>>( \
+#define LSA_LAUNCH_ITEMS(MODE, PLAIN) LSA_LAUNCH_ITEMS_MERGE(MODE, PLAIN, 0)
+#define LSA_LAUNCH_ITEMS_MERGE(MODE, PLAIN, RANGES) paged_attention_kernel<MODE, PLAIN, RANGES><<<grid, 256, 0, stream>>>( \
         (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride, \
         row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g, fusion)
 #if LSA_BF16
     const bool plain = q_weight != nullptr && cos_sin != nullptr;
     if (merge_in_workgroup && decode_fusion && !plain) return -1;      // the caller asks lsa_attention_merges_in_workgroup first
-    if (merge_in_workgroup && decode_fusion == 3) LSA_LAUNCH_ITEMS_MERGE(3, true, true);
-    else if (merge_in_workgroup && decode_fusion == 1) LSA_LAUNCH_ITEMS_MERGE(1, true, true);
-    else if (merge_in_workgroup) LSA_LAUNCH_ITEMS_MERGE(0, false, true);
+    if (merge_in_workgroup == 4 && decode_fusion == 3) LSA_LAUNCH_ITEMS_MERGE(3, true, 4);
+    else if (merge_in_workgroup == 4 && decode_fusion == 1) LSA_LAUNCH_ITEMS_MERGE(1, true, 4);
+    else if (merge_in_workgroup == 4) LSA_LAUNCH_ITEMS_MERGE(0, false, 4);
+    else if (merge_in_workgroup == 2 && decode_fusion == 3) LSA_LAUNCH_ITEMS_MERGE(3, true, 2);
+    else if (merge_in_workgroup == 2 && decode_fusion == 1) LSA_LAUNCH_ITEMS_MERGE(1, true, 2);
+    else if (merge_in_workgroup == 2) LSA_LAUNCH_ITEMS_MERGE(0, false, 2);
     else if (decode_fusion == 3 && plain) LSA_LAUNCH_ITEMS(3, true);
     else if (decode_fusion == 3) LSA_LAUNCH_ITEMS(3, false);
     else if (decode_fusion == 1 && plain) LSA_LAUNCH_ITEMS(1, true);
     else if (decode_fusion == 1) LSA_LAUNCH_ITEMS(1, false);
     else
 #else
-    if (merge_in_workgroup) LSA_LAUNCH_ITEMS_MERGE(0, false, true);
+    if (merge_in_workgroup == 4) LSA_LAUNCH_ITEMS_MERGE(0, false, 4);
+    else if (merge_in_workgroup == 2) LSA_LAUNCH_ITEMS_MERGE(0, false, 2);
     else
 #endif
     LSA_LAUNCH_ITEMS(0, false);

@@ -547,11 +547,11 @@ class HipOps:
             if cos_sin is not None:
                 _check(cos_sin, "cos_sin", torch.float32, (n, head_dim))
             fusion_mode = 3 if write_cache else 1
-        merge_in_workgroup = int(bool(plan.get("merge_in_workgroup", 0)))
+        merge_in_workgroup = int(plan.get("merge_in_workgroup", 0))
         if merge_in_workgroup and (n_items % 4 or n_merges or n_slots or n_tiles or n != rows
                                    or (decode_fusion is not None and (q_weight is None or cos_sin is None))):
             raise ValueError("merging in the workgroup takes steps of one token per row whose plan gives every tile four key ranges "
-                             "and no slots, and, with decode fusion, both norm weights and a rotation")
+                             "(or two, with tiles in pairs) and no slots, and, with decode fusion, both norm weights and a rotation")
         lib = self._attention_library(qkv.dtype, head_dim)
         if plan.get("most_splits", 0) > lib.lsa_attention_most_splits():
             raise ValueError(f"the plan splits a tile's keys into {plan['most_splits']} ranges, the merge kernel takes {lib.lsa_attention_most_splits()}")

@@ -56,7 +56,8 @@ class AttentionPlan:
         self.items, self.item_slot, self.merges, self.n_slots = items, item_slot, merges, n_slots
         self.tiles = tiles if tiles is not None else np.zeros((0, 4), dtype=np.int32)
         self.tiles_per_workgroup = tiles_per_workgroup
-        self.merge_in_workgroup = False      # items 4 i .. 4 i + 3 are one tile's key ranges, merged by their workgroup
+        self.merge_in_workgroup = 0          # 4: items 4 i .. 4 i + 3 are one tile's key ranges, merged by their workgroup;
+                                             # 2: they are the two ranges of each of two tiles
 
 
 def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: int, target_waves: int = TARGET_WAVES) -> int:
@@ -102,7 +103,7 @@ WORKGROUP_RANGES = 4    # key ranges of a tile that one workgroup (four wavefron
 SHORT_CONTEXT = 512     # up to this context a step of single tokens is merged in its workgroups (measured against the merge launch)
 
 
-def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, merge_in_workgroup: bool = False) -> AttentionPlan:
+def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, merge_in_workgroup: int = 0) -> AttentionPlan:
     """The plan of a step in which every row brings one token and every tile gets ``splits`` key ranges: what the
     loop of :func:`build_attention_plan` makes for it, row by row, computed for all rows at once (a decode step of
     many rows is planned thousands of times a second)."""
@@ -114,8 +115,8 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, 
     if splits <= 1 and not merge_in_workgroup:
         items = np.stack([rows, zeros, k_begin, k_end], axis=1).astype(np.int32)
         return AttentionPlan(items, np.full(n_rows, -1, dtype=np.int32), np.zeros((0, 4), dtype=np.int32), 0)
-    if merge_in_workgroup:          # four items a tile; with fewer ranges wanted, the last ones come out empty
-        ranges, splits = max(1, min(splits, WORKGROUP_RANGES)), WORKGROUP_RANGES
+    if merge_in_workgroup:          # four (or two) items a tile; with fewer ranges wanted, the last ones come out empty
+        ranges, splits = max(1, min(splits, merge_in_workgroup)), merge_in_workgroup
     start = (k_begin // KEY_ALIGN) * KEY_ALIGN
     per = -(-(k_end - start) // (ranges if merge_in_workgroup else splits))
     per = -(-per // KEY_ALIGN) * KEY_ALIGN
@@ -129,7 +130,7 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, 
                      axis=1).astype(np.int32)
     if merge_in_workgroup:          # the four items of a tile are one workgroup's: no slots, nothing left to merge
         plan = AttentionPlan(items, np.full(n_rows * splits, -1, dtype=np.int32), np.zeros((0, 4), dtype=np.int32), 0)
-        plan.merge_in_workgroup = True
+        plan.merge_in_workgroup = merge_in_workgroup
         return plan
     merges = np.stack([rows, zeros, rows * splits, np.full(n_rows, splits, dtype=np.int64)], axis=1).astype(np.int32)
     return AttentionPlan(items, np.arange(n_rows * splits, dtype=np.int32), merges, n_rows * splits)
@@ -137,7 +138,7 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, 
 
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
-                         workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: bool = False) -> AttentionPlan:
+                         workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: int = 0) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
@@ -147,11 +148,14 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
+    merge_in_workgroup = WORKGROUP_RANGES if merge_in_workgroup is True else int(merge_in_workgroup)
     if merge_in_workgroup and not (len(row_len) and int(row_len.min()) == 1 == int(row_len.max())):
         raise ValueError("key ranges are merged in the workgroup only in steps of one token per row")
+    if merge_in_workgroup not in (0, 2, WORKGROUP_RANGES) or (merge_in_workgroup == 2 and len(row_len) % 2):
+        raise ValueError("a workgroup merges four key ranges of one tile, or two ranges of each of two tiles (an even number of rows)")
     if (merge_in_workgroup or (single_token_shortcut and fixed_splits is not None)) and len(row_len) \
             and int(row_len.min()) == 1 == int(row_len.max()):
-        return _single_token_plan(row_ctx, window, int(fixed_splits or WORKGROUP_RANGES), merge_in_workgroup)
+        return _single_token_plan(row_ctx, window, int(fixed_splits or merge_in_workgroup or 1), merge_in_workgroup)
     tiles_per_row = -(-row_len // tokens_per_tile)
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
     items, slots, merges, tiles = [], [], [], []
@@ -263,9 +267,13 @@ class GQAttention(Mixer):
         # So does a step with so many rows that a tile gets four ranges anyway: the merge launch is all that differs.
         # (With two or three ranges a tile, half of a workgroup's wavefronts would idle through the others' walk:
         # measured at 64 rows behind 4,096 tokens, a tenth slower than with the merge launch.)
-        in_workgroup = ctx.n_tokens == ctx.n_rows and (bool(getattr(ctx, "short_contexts", False)) or fixed == WORKGROUP_RANGES)
-        if in_workgroup and getattr(ctx, "short_contexts", False):
-            fixed = WORKGROUP_RANGES
+        # Two ranges a tile: two tiles to a workgroup, if the rows come in pairs.
+        in_workgroup = 0
+        if ctx.n_tokens == ctx.n_rows:
+            if getattr(ctx, "short_contexts", False):
+                in_workgroup = fixed = WORKGROUP_RANGES
+            elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
+                in_workgroup = fixed
         import torch
         per_workgroup = getattr(ctx.ops, "attention_workgroup_tiles", None)
         per_workgroup = per_workgroup(ctx.dtype, self.head_dim) if per_workgroup is not None else 0

@@ -115,18 +115,23 @@ def test_plan_whose_key_ranges_are_merged_in_the_workgroup(seed):
     rows = rng.randint(1, 70)
     contexts = [rng.choice((1, 2, 31, 32, 33, 64, 100, 300, 511, 512, 513, 1024, rng.randint(1, 2000))) for _ in range(rows)]
     window = rng.choice((None, None, 1, 40, 700))
+    per_tile = rng.choice((4, 4, 2))               # two ranges a tile: two tiles to a workgroup, rows in pairs
+    if per_tile == 2 and rows % 2:
+        with pytest.raises(ValueError):
+            build_attention_plan([1] * rows, contexts, 4, 8, window, merge_in_workgroup=2)
+        rows, contexts = rows + 1, contexts + [77]
     plan = build_attention_plan([1] * rows, contexts, rng.choice((1, 4, 20)), rng.choice((1, 8)), window, fixed_splits=rng.choice((None, 1, 16)),
-                                merge_in_workgroup=True)
-    assert plan.merge_in_workgroup and plan.items.shape == (4 * rows, 4) and plan.n_slots == 0 and plan.merges.shape == (0, 4)
-    assert (plan.item_slot == -1).all() and plan.tiles.shape == (0, 4)
+                                merge_in_workgroup=per_tile)
+    assert plan.merge_in_workgroup == per_tile and plan.items.shape == (per_tile * rows, 4) and plan.n_slots == 0 and plan.merges.shape == (0, 4)
+    assert (plan.item_slot == -1).all() and plan.tiles.shape == (0, 4) and len(plan.items) % 4 == 0
     for row, context in enumerate(contexts):
-        ranges = plan.items[4 * row:4 * row + 4].tolist()
+        ranges = plan.items[per_tile * row:per_tile * row + per_tile].tolist()
         assert all(r == row and q0 == 0 for r, q0, _, _ in ranges)
         first = 0 if window is None else max(0, context - window)
         filled = [(b, e) for _, _, b, e in ranges if b < e]
         assert filled and filled[0][0] == first and filled[-1][1] == context
         assert all(a[1] == b[0] and b[0] % KEY_ALIGN == 0 for a, b in zip(filled, filled[1:]))
-        assert [(b, e) for _, _, b, e in ranges][len(filled):] == [(context, context)] * (4 - len(filled))
+        assert [(b, e) for _, _, b, e in ranges][len(filled):] == [(context, context)] * (per_tile - len(filled))
 
 
 def test_four_or_eight_tiles_per_workgroup():

@@ -217,18 +217,19 @@ def test_attention_mixed_batch(ops, dtype, n_q, n_kv, d, page):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (6, 2, 48, 12), (32, 8, 128, 16), (5, 1, 80, 8), (20, 1, 64, 16), (2, 1, 256, 64)])
 @pytest.mark.parametrize("window", [None, 40])
-def test_attention_key_ranges_merged_in_the_workgroup(ops, dtype, n_q, n_kv, d, page, window):
+@pytest.mark.parametrize("per_tile", [4, 2])
+def test_attention_key_ranges_merged_in_the_workgroup(ops, dtype, n_q, n_kv, d, page, window, per_tile):
     """Steps of single tokens whose tiles get four key ranges each, walked by the four wavefronts of one workgroup and
     merged there (no partial results, no merge launch): contexts of one token (three ranges empty), at the edges of
     pages and key steps, with a far key that decides the first query; queries and keys prepared by the separate kernel."""
-    print(f"attention merged in the workgroup {dtype} {n_q}/{n_kv} d{d} page{page} window {window}", flush=True)
+    print(f"attention merged in the workgroup {dtype} {n_q}/{n_kv} d{d} page{page} window {window}, {per_tile} ranges a tile", flush=True)
     ctxs = [1, 2, 3, 4, 5, 31, 32, 33, 63, 64, 65, 127, 128, 129, 300, 511, 512, 1025]
-    plan, ref = attention_case(ops, dtype, n_q, n_kv, d, page, [1] * len(ctxs), ctxs, window=window, seed=n_q * d + 1, merge_in_workgroup=True)
-    assert plan.merge_in_workgroup and len(plan.items) == 4 * len(ctxs) and plan.n_slots == 0 and len(plan.merges) == 0
+    plan, ref = attention_case(ops, dtype, n_q, n_kv, d, page, [1] * len(ctxs), ctxs, window=window, seed=n_q * d + 1, merge_in_workgroup=per_tile)
+    assert plan.merge_in_workgroup == per_tile and len(plan.items) == per_tile * len(ctxs) and plan.n_slots == 0 and len(plan.merges) == 0
     if window is None:
         assert float(ref[-1, :d].float().mean()) > 5.0           # the far key won the last row's first head
     with pytest.raises(ValueError):                              # a row of two tokens
-        build_attention_plan([1, 2], [5, 9], n_q // n_kv, n_kv, window, merge_in_workgroup=True)
+        build_attention_plan([1, 2], [5, 9], n_q // n_kv, n_kv, window, merge_in_workgroup=per_tile)
 
 
 @pytest.mark.parametrize("n_q, n_kv, d, page", [(32, 8, 128, 16), (4, 2, 64, 8), (20, 1, 64, 16), (6, 3, 192, 12), (2, 1, 256, 64)])
@@ -273,7 +274,7 @@ def test_attention_decode_fusion(ops, n_q, n_kv, d, page, window):
     for fixed in (None, 8, "in the workgroup"):
         in_workgroup = fixed == "in the workgroup"                           # four key ranges a tile, merged by the workgroup that walks them
         plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, fixed_splits=8 if in_workgroup else fixed,
-                                    merge_in_workgroup=in_workgroup)
+                                    merge_in_workgroup=4 if in_workgroup else 0)
         staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
                   "merges": torch.from_numpy(plan.merges).to(DEV), "n_items": len(plan.items), "n_merges": len(plan.merges),
                   "n_slots": plan.n_slots, "merge_in_workgroup": int(plan.merge_in_workgroup)}
