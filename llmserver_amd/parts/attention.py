@@ -100,7 +100,6 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
 
 
 WORKGROUP_RANGES = 4    # key ranges of a tile that one workgroup (four wavefronts) walks and merges itself
-SHORT_CONTEXT = 512     # up to this context a step of single tokens is merged in its workgroups (measured against the merge launch)
 
 
 def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, merge_in_workgroup: int = 0) -> AttentionPlan:
@@ -262,19 +261,17 @@ class GQAttention(Mixer):
         fixed = None
         if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
             fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys)
-        # Short contexts (the step says so, and keeps saying so for as long as its shape is replayed): four key ranges
-        # a tile, which the workgroup that walks them merges itself.
-        # So does a step with so many rows that a tile gets four ranges anyway: the merge launch is all that differs.
-        # (With two or three ranges a tile, half of a workgroup's wavefronts would idle through the others' walk:
-        # measured at 64 rows behind 4,096 tokens, a tenth slower than with the merge launch.)
-        # Two ranges a tile: two tiles to a workgroup, if the rows come in pairs.
+        # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:
+        #  * short contexts (the step says so, and keeps saying so for as long as its shape is replayed): four ranges a tile;
+        #  * so many rows that a tile gets four ranges anyway;
+        #  * two ranges a tile: two tiles to a workgroup, if the rows come in pairs.  (Two or three ranges in a workgroup
+        #    of one tile leave wavefronts idle through the others' walk: a tenth slower at 64 rows behind 4,096 tokens.)
         in_workgroup = 0
         if ctx.n_tokens == ctx.n_rows:
             if getattr(ctx, "short_contexts", False):
                 in_workgroup = fixed = WORKGROUP_RANGES
             elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
                 in_workgroup = fixed
-        import torch
         per_workgroup = getattr(ctx.ops, "attention_workgroup_tiles", None)
         per_workgroup = per_workgroup(ctx.dtype, self.head_dim) if per_workgroup is not None else 0
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
