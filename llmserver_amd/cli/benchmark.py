@@ -4,6 +4,11 @@ meanings follow it where it has them.
 
     python benchmark.py --model DIR --prompt-tokens 128,1024 --batch-sizes 1,8,32 --output-tokens 128
     python benchmark.py --random-config qwen3-8b --prompt-tokens 2048 --batch-sizes 1,8,64 --output-tokens 2048
+    python benchmark.py --model DIR --prompt-token-ids 151644,872,198 --max-new-tokens 32 --repeats 3
+
+With ``--prompt`` (text, if the model folder has a ``tokenizer.json``) or ``--prompt-token-ids`` it benchmarks one prompt
+in the manner of the reference's ``benchmark.py`` (/root/reference/benchmark.py:68-88, 339-341): model load, time to
+the first token, generation and decode throughput, medians over ``--repeats``.
 
 For each (prompt length, batch size):
   * ttft_s  = time to generate 1 token for the whole batch (prefill latency)
@@ -64,10 +69,72 @@ def run_once(engine, prompts, new_tokens):
     return time.perf_counter() - start, [list(r.generated_token_ids) for r in requests]
 
 
+def one_prompt(args, model, load_seconds) -> int:
+    """One prompt, ``--repeats`` fresh requests: the reference's single-prompt statistics
+    (/root/reference/benchmark.py:68-88)."""
+    import os
+
+    import torch
+
+    from ..engine import Engine
+    tokenizer = None
+    if args.prompt is not None:
+        path = os.path.join(args.model or "", "tokenizer.json")
+        if not args.model or not os.path.isfile(path):
+            print("--prompt needs a model folder with a tokenizer.json; pass --prompt-token-ids instead", file=sys.stderr)
+            return 2
+        from tokenizers import Tokenizer
+        tokenizer = Tokenizer.from_file(path)
+        prompt_ids = tokenizer.encode(args.prompt).ids
+    else:
+        prompt_ids = parse_ints(args.prompt_token_ids)
+    if not prompt_ids or args.max_new_tokens <= 0:
+        print("the prompt must hold at least one token and --max-new-tokens must be positive", file=sys.stderr)
+        return 2
+    blocks = math.ceil((len(prompt_ids) + args.max_new_tokens) / args.block_size) + 8
+    engine = Engine(model, None, max_new_tokens=args.max_new_tokens, max_batch_size=1,
+                    max_num_batched_tokens=max(args.max_num_batched_tokens, 1), prefill_chunk_size=args.prefill_chunk_size,
+                    kv_cache_num_blocks=blocks, kv_cache_block_size=args.block_size, stream_text=False, max_completed_requests=0,
+                    ignore_eos=False, temperature=args.temperature, seed=args.seed, enable_prefix_caching=False)
+    run_once(engine, [prompt_ids], min(args.max_new_tokens, 4))               # graphs and kernel choices, before the clock
+    results = []
+    for _ in range(args.repeats):
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        request = engine.add_request(None, prompt_token_ids=prompt_ids, max_new_tokens=args.max_new_tokens)
+        first = None
+        while engine.step():
+            if first is None and request.generated_token_ids:
+                first = time.perf_counter() - start
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - start
+        results.append((list(request.generated_token_ids), seconds, first if first is not None else seconds))
+    tokens, seconds, first = results[-1]
+    print(f"\nPrompt: {args.prompt if args.prompt is not None else prompt_ids}")
+    print(f"Response: {tokenizer.decode(tokens) if tokenizer is not None else tokens}")
+    print(f"\nDevice: {torch.cuda.get_device_name(0)} | Model: {model.name}")
+    print(f"Prompt tokens: {len(prompt_ids)} | Generated tokens: {len(tokens)}")
+    print(f"Model load: {load_seconds:.2f} s | Generation: {seconds:.3f} s")
+    print(f"Time to first token: {first:.4f} s")
+    print(f"Generation throughput: {len(tokens) / seconds:.2f} tokens/s")
+    if len(tokens) > 1:
+        print(f"Decode throughput: {(len(tokens) - 1) / (seconds - first):.2f} tokens/s")
+    if len(results) > 1:
+        print(f"median over {len(results)} runs: Generation: {statistics.median(r[1] for r in results):.3f} s | "
+              f"Time to first token: {statistics.median(r[2] for r in results):.4f} s")
+        speeds = [(len(r[0]) - 1) / (r[1] - r[2]) for r in results if len(r[0]) > 1]
+        if speeds:
+            print(f"median decode throughput: {statistics.median(speeds):.2f} tokens/s")
+    return 0
+
+
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     parser.add_argument("--model", default=None, help="model folder (config.json + safetensors)")
     parser.add_argument("--random-config", default=None, choices=sorted(RANDOM_CONFIGS), help="seeded random weights of a named size instead of --model")
+    parser.add_argument("--prompt", default=None, help="one prompt as text (needs tokenizer.json in the model folder)")
+    parser.add_argument("--prompt-token-ids", default=None, help="one prompt as comma-separated token ids")
+    parser.add_argument("--max-new-tokens", type=int, default=32, help="tokens to generate for --prompt / --prompt-token-ids")
     parser.add_argument("--prompt-tokens", default="128,1024")
     parser.add_argument("--batch-sizes", default="1,8,32")
     parser.add_argument("--output-tokens", type=int, default=128)
@@ -109,6 +176,8 @@ def main(argv=None) -> int:
     torch.cuda.synchronize()
     print(f"loaded {model.name} in {time.perf_counter() - started:.1f} s", flush=True)
     vocab = model.config.vocab_size
+    if args.prompt is not None or args.prompt_token_ids is not None:
+        return one_prompt(args, model, time.perf_counter() - started)
     prompt_lengths, batches = parse_ints(args.prompt_tokens), parse_ints(args.batch_sizes)
     if args.mixed_requests:
         low, high = parse_ints(args.mixed_prompt_range)
