@@ -71,6 +71,7 @@ def write_random_model(config: ModelConfig, folder: str, init: RandomInit = Rand
         values = random_tensor(name, spec, init)
         tensors[name] = values if spec.role == INT_TABLE else values.to(dtype)
     save_file(tensors, os.path.join(folder, "model.safetensors"))
+    os.chmod(os.path.join(folder, "model.safetensors"), 0o644)       # readable by whoever runs the model, as config.json is
     with open(os.path.join(folder, "config.json"), "w") as handle:
         json.dump(config.to_dict(), handle, indent=1)
     return folder

@@ -148,3 +148,27 @@ def test_missing_folder_parts_are_named(tmp_path):
         json.dump(TINY_A, handle)
     with pytest.raises(FileNotFoundError, match="model.safetensors"):
         load_model(str(tmp_path), "cpu", torch.float32)
+
+
+def test_random_model_command_writes_a_folder_that_loads_and_repeats(tmp_path):
+    """bin/random_model: a named size, then the config.json it wrote: the same seed gives the same tensors."""
+    import subprocess
+    import sys
+    from safetensors import safe_open
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    command = [sys.executable, os.path.join(root, "bin", "random_model")]
+    first, second = str(tmp_path / "first"), str(tmp_path / "second")
+    done = subprocess.run(command + ["--random-config", "tiny-b", "--out", first, "--seed", "3", "--norm-noise", "0.1"], capture_output=True, text=True)
+    assert done.returncode == 0 and "model.safetensors" in done.stdout, done.stderr
+    done = subprocess.run(command + ["--config", os.path.join(first, "config.json"), "--out", second, "--seed", "3", "--norm-noise", "0.1",
+                                     "--dtype", "float32"], capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
+    model = load_model(first, "cpu", torch.float32)
+    assert model.config.num_hidden_layers == 3 and model.config.attention_bias
+    with safe_open(os.path.join(first, "model.safetensors"), "pt") as a, safe_open(os.path.join(second, "model.safetensors"), "pt") as b:
+        assert sorted(a.keys()) == sorted(b.keys())
+        for name in a.keys():
+            assert a.get_tensor(name).dtype == torch.bfloat16 and b.get_tensor(name).dtype == torch.float32
+            assert torch.equal(a.get_tensor(name), b.get_tensor(name).to(torch.bfloat16)), name
+    assert os.stat(os.path.join(first, "model.safetensors")).st_mode & 0o044 == 0o044
+    assert subprocess.run(command + ["--out", first], capture_output=True).returncode == 2          # neither a config nor a named size
