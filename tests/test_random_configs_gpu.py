@@ -55,14 +55,34 @@ def random_trace(rng, vocab):
     return steps, requests
 
 
+ODD_WIDTHS = {"odd": dict(hidden_size=33, intermediate_size=25, vocab_size=101, head_dim=16, attention_bias=False),
+              "few": dict(hidden_size=7, intermediate_size=5, vocab_size=3, head_dim=32, attention_bias=True),
+              "one": dict(hidden_size=1, intermediate_size=1, vocab_size=2, head_dim=48, attention_bias=False),
+              "wide": dict(hidden_size=129, intermediate_size=1027, vocab_size=7, head_dim=16, attention_bias=True)}
+
+
+@pytest.mark.parametrize("name", sorted(ODD_WIDTHS))
+def test_widths_that_no_vector_load_divides(name, tmp_path):
+    """Widths, intermediate sizes and vocabularies that are odd or smaller than one vector load: rows then start at
+    addresses that no wide load may assume, and the last partial vector must neither be dropped nor read past."""
+    sizes = ODD_WIDTHS[name]
+    raw = dict(model_type="qwen3", num_hidden_layers=2, num_attention_heads=3, num_key_value_heads=1, rope_theta=1e4,
+               rms_norm_eps=1e-6, tie_word_embeddings=sizes["attention_bias"], **sizes)
+    check_configuration(raw, 16, random.Random(len(name)), 7, tmp_path)
+
+
 @pytest.mark.parametrize("seed", SEEDS)
 def test_random_configuration_matches_the_plain_implementation(seed, tmp_path):
-    from llmserver_amd.engine.replay import make_runner, replay
-
     rng = random.Random(seed)
     raw = random_config(rng)
     page_size = rng.choice((16, 16, 16, 4, 8, 32, 64))
-    print(f"random configuration {seed}: page {page_size} {raw}", flush=True)
+    check_configuration(raw, page_size, rng, seed, tmp_path)
+
+
+def check_configuration(raw, page_size, rng, seed, tmp_path):
+    from llmserver_amd.engine.replay import make_runner, replay
+
+    print(f"configuration {seed}: page {page_size} {raw}", flush=True)
     folder = str(tmp_path / "model")
     write_random_model(config_from_dict(dict(raw)), folder, RandomInit(seed=seed, std=rng.choice((0.02, 0.05)), norm_noise=0.1))
     steps, requests = random_trace(rng, raw["vocab_size"])
