@@ -43,6 +43,8 @@ struct Fusion {
     bf16_t* resid_out;                   // [M, N]
     bf16_t* weighted_out;                // [M, N]
     float* square_sums_out;              // [M, P], P as lsa_gemm_skinny_parts tells
+    // Bias (null: none), added to the float32 sum before its one rounding; plain results only.
+    const float* bias;                   // [N]
 };
 
 // The partial sums of wavefront `wave`'s row are loaded behind the last operands of the product
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
             if (j == 0 && m < M) fusion.square_sums_out[(size_t)m * gridDim.x + blockIdx.x] = sq;
             continue;
         }
-        if (m < M && j < R && n < N) y[(size_t)m * N + n] = (OutT)total;
+        if (m < M && j < R && n < N) y[(size_t)m * N + n] = (OutT)(fusion.bias ? total + fusion.bias[n] : total);
     }
 }
 
@@ -333,7 +335,7 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_wide_kernel(const
         if (!tile && j == 0 && m < M) fusion.square_sums_out[(size_t)m * gridDim.x + blockIdx.x] = sq + second_tile_sums[m];
         return;
     }
-    if (m < M && own && n < N) y[(size_t)m * N + n] = (OutT)total;
+    if (m < M && own && n < N) y[(size_t)m * N + n] = (OutT)(fusion.bias ? total + fusion.bias[n] : total);
 }
 
 // The chunk size in 4..8 that wastes the fewest loads past the end of a wavefront's share of K.
@@ -613,13 +615,14 @@ static bool fusion_fits(int M, const float* square_sums, int n_parts, const void
 
 // out_float32: 0 writes bfloat16, 1 writes float32.  rows: rows of W per workgroup, 1 to 32 (more than 16
 // only for M <= 16), or 0 to let the size decide.  square_sums [M, n_parts] (or null) asks for the row scale
-// rsqrt(sum / K + eps), M <= 16.  Refuses (returns -1) what it cannot take.
+// rsqrt(sum / K + eps), M <= 16.  bias [N] (or null) is added to the sums before they are rounded.  Refuses
+// (returns -1) what it cannot take.
 LSA_EXPORT int lsa_gemm_skinny(int out_float32, const void* x, const void* w, void* y, int M, int N, int K, int rows,
-                               const float* square_sums, int n_parts, float eps, hipStream_t stream) {
+                               const float* square_sums, int n_parts, float eps, const float* bias, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K % 8 != 0 || K < 8 || rows < 0 || rows > 32 || (rows > 16 && M > 16)) return -1;
     if (!fusion_fits(M, square_sums, n_parts, nullptr)) return -1;
-    const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr};
+    const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr, bias};
     rows = choose_rows(M, N, false, rows);
     return out_float32 ? launch<float, false>((const bf16_t*)x, (const bf16_t*)w, (float*)y, M, N, K, rows, fusion, stream)
                        : launch<bf16_t, false>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, rows, fusion, stream);
@@ -646,7 +649,7 @@ LSA_EXPORT int lsa_gemm_skinny_stream(const void* x, const void* w, int M, int N
         return -1;
     if (!fusion_fits(M, square_sums, n_parts, resid)) return -1;
     const Fusion fusion = {square_sums, n_parts, eps, (const bf16_t*)resid, norm_weight, (bf16_t*)resid_out, (bf16_t*)weighted_out,
-                           square_sums_out};
+                           square_sums_out, nullptr};
     return launch<bf16_t, false>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)nullptr, M, N, K, choose_rows(M, N, false, rows), fusion, stream);
 }
 
@@ -658,7 +661,7 @@ LSA_EXPORT int lsa_gemm_skinny_gated(const void* x, const void* gate_up, void* h
     if (M <= 0 || I <= 0) return 0;
     if (M > 16 || K % 8 != 0 || K < 8 || I % 8 != 0 || rows < -1 || rows > 16) return -1;
     if (!fusion_fits(M, square_sums, n_parts, nullptr)) return -1;
-    const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr};
+    const Fusion fusion = {square_sums, n_parts, eps, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     return launch<bf16_t, true>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)hidden, M, 2 * I, K, choose_rows(M, 2 * I, true, rows),
                                 fusion, stream);
 }

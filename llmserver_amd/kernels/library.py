@@ -25,7 +25,7 @@ _SIGNATURES = {
     "lsa_attention_most_splits": [],
     "lsa_attention_head_dim": [],
     "lsa_attention_is_bf16": [],
-    "lsa_gemm_skinny": [c_int, _P, _P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P],
+    "lsa_gemm_skinny": [c_int, _P, _P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P, _P],
     "lsa_gemm_skinny_parts": [c_int, c_int, c_int],
     "lsa_gemm_skinny_stream": [_P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P, _P, _P, _P, _P, _P],
     "lsa_gemm_skinny_gated": [_P, _P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P],

@@ -269,24 +269,40 @@ class HipOps:
         """Whether the few-row products take ``x`` with this ``row_scale`` (then they do not return None for it)."""
         return x.shape[1] == weight.shape[1] and self._few_rows(x, weight) and self._row_scale_fits(row_scale, x.shape[0])
 
-    def linear(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0):
+    fuses_bias = True       # linear() and linear_few_rows() take the bias themselves
+
+    def linear(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0, bias=None, bias_rounded=None):
         """``x [T, in] @ weight[out, in]^T``; float32 result if asked (the output head).  ``rows_per_workgroup``
-        fixes the few-row kernel's share of the weight per workgroup (1 to 32; 0 lets the size decide)."""
+        fixes the few-row kernel's share of the weight per workgroup (1 to 32; 0 lets the size decide).
+
+        ``bias [out]`` (float32) is added to the product.  In bfloat16 the sum is rounded once, as a library's
+        product with a bias rounds it: by the few-row kernel, or by the library if ``bias_rounded`` gives the same
+        numbers in ``x``'s type; a bias that has no such form is added to the rounded product."""
         if x.shape[1] != weight.shape[1]:
             raise ValueError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
+        if bias is not None:
+            _check(bias, "bias", torch.float32, (weight.shape[0],))
         if self._few_rows(x, weight) and (rows_per_workgroup or not self.library_is_faster("plain", x, weight, False, out_float32)):
             # Few rows: the product is a stream over the weights; the hand-written kernel reads them once at HBM rate.
-            return self.linear_few_rows(x, weight, out=out, out_float32=out_float32, rows_per_workgroup=rows_per_workgroup)
+            return self.linear_few_rows(x, weight, out=out, out_float32=out_float32, rows_per_workgroup=rows_per_workgroup, bias=bias)
         if out_float32 and x.dtype != torch.float32:
-            return torch.mm(x, weight.t(), out_dtype=torch.float32)
-        return torch.mm(x, weight.t(), out=out) if out is not None else torch.mm(x, weight.t())
+            y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+        elif bias is not None and bias_rounded is not None and bias_rounded.dtype == x.dtype and x.dtype != torch.float32:
+            _check(bias_rounded, "bias_rounded", x.dtype, (weight.shape[0],))
+            return torch.addmm(bias_rounded, x, weight.t(), out=out) if out is not None else torch.addmm(bias_rounded, x, weight.t())
+        else:
+            y = torch.mm(x, weight.t(), out=out) if out is not None else torch.mm(x, weight.t())
+        if bias is not None:
+            self.add_bias_(y, bias)
+        return y
 
-    def linear_few_rows(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0, row_scale=None):
+    def linear_few_rows(self, x, weight, out=None, out_float32=False, rows_per_workgroup=0, row_scale=None, bias=None):
         """The weight-streaming product, or None if this is no case for it.
 
         ``row_scale = (square_sums [T, P], eps)``: ``x`` is a residual stream already multiplied by a norm's
         weights, ``square_sums`` are partial sums of the stream's squares, and the result rows are divided by the
-        stream's root mean square, so that the result is the product of the normalised stream (up to 16 rows)."""
+        stream's root mean square, so that the result is the product of the normalised stream (up to 16 rows).
+        ``bias [out]`` (float32) is added before the result is rounded."""
         rows, width = x.shape
         if x.shape[1] != weight.shape[1] or not self._few_rows(x, weight) or not self._row_scale_fits(row_scale, rows) \
                 or (rows_per_workgroup > 16 and rows > 16):
@@ -297,8 +313,11 @@ class HipOps:
             out = torch.empty((rows, weight.shape[0]), device=x.device, dtype=torch.float32 if out_float32 else torch.bfloat16)
         _check(out, "out", None, (rows, weight.shape[0]))
         sums, parts, eps = self._row_scale_args(row_scale, rows)
+        if bias is not None:
+            _check(bias, "bias", torch.float32, (weight.shape[0],))
         _launched(self._gemm.lsa_gemm_skinny(1 if out_float32 else 0, _ptr(x), _ptr(weight), _ptr(out), rows, weight.shape[0], width,
-                                             int(rows_per_workgroup), sums, parts, eps, _stream()), "gemm_skinny")
+                                             int(rows_per_workgroup), sums, parts, eps, _ptr(bias) if bias is not None else None,
+                                             _stream()), "gemm_skinny")
         return out
 
     SPLIT_ROWS = 128        # most rows the product that leaves partial sums takes (it starts above the few-row kernels')

@@ -34,6 +34,7 @@ class Linear(Part):
         self._b: Dict[str, torch.Tensor] = {}
         self.weight = None   # [out, in] compute dtype
         self.bias = None     # [out] float32
+        self.bias_rounded = None   # the bias in the weight's type, if that type holds it exactly (a library's product takes it so)
 
     def param_specs(self):
         specs = {}
@@ -58,6 +59,9 @@ class Linear(Part):
         if self.has_bias and self.bias is None:
             bs = [self._b[p] for p in self.pieces]
             self.bias = bs[0] if len(bs) == 1 else torch.cat(bs, dim=0)
+        if self.bias is not None and self.weight.dtype != torch.float32:
+            rounded = self.bias.to(self.weight.dtype)
+            self.bias_rounded = rounded if torch.equal(rounded.to(self.bias.dtype), self.bias) else None
         self._w.clear()
         self._b.clear()
 
@@ -93,6 +97,11 @@ class Linear(Part):
             if sums is not None:
                 stream = sink.stream()
                 return StreamUpdate(sink.norm, stream, normed=sink.norm.add_norm(stream, sums, ctx))
+        if self.bias is not None and getattr(ops, "fuses_bias", False):
+            # The bias joins the product's float32 sums, which are then rounded once.
+            if row_scale is not None:
+                return ops.linear_few_rows(x, self.weight, out=out, out_float32=self.out_float32, row_scale=row_scale, bias=self.bias)
+            return ops.linear(x, self.weight, out=out, out_float32=self.out_float32, bias=self.bias, bias_rounded=self.bias_rounded)
         if row_scale is not None:
             y = ops.linear_few_rows(x, self.weight, out=out, out_float32=self.out_float32, row_scale=row_scale)
         else:

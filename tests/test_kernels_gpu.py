@@ -432,9 +432,34 @@ def test_skinny_gemm(ops, rows, n, k):
     finally:
         ops.skinny_rows = saved
     with pytest.raises(RuntimeError):
-        ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, 0, None, 0, 0.0, None)
+        ops._gemm_refusal_check = ops._gemm.lsa_gemm_skinny(0, x.data_ptr(), w.data_ptr(), got16.data_ptr(), 65, n, k, 0, None, 0, 0.0, None, None)
         if ops._gemm_refusal_check != 0:
             raise RuntimeError("refused")
+
+
+@pytest.mark.parametrize("rows", [1, 7, 16, 17, 33, 64, 65, 300])
+@pytest.mark.parametrize("n, k", [(48, 72), (301, 520), (1030, 264), (96, 33), (6144, 4096)])
+def test_product_with_bias_is_rounded_once(ops, rows, n, k):
+    """``x w^T + b`` in bfloat16: the bias joins the float32 sums and the result is rounded once, so it lies within
+    half a bfloat16 step of the exact value (a product that is rounded before the bias is added misses by up to a
+    whole step, and by more where the bias cancels the product).  Through the few-row kernels and the library."""
+    print(f"product with bias rows {rows} n {n} k {k}", flush=True)
+    torch.manual_seed(rows + n + k)
+    x = torch.randn(rows, k, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(n, k, device=DEV) / k ** 0.5).to(torch.bfloat16)
+    bias = torch.randn(n, device=DEV).to(torch.bfloat16).float()
+    exact = x.double() @ w.double().t() + bias.double()
+    got = ops.linear(x, w, bias=bias, bias_rounded=bias.to(torch.bfloat16))
+    assert got.dtype == torch.bfloat16 and got.shape == (rows, n)
+    half_step = exact.abs() * 2.0 ** -8
+    float32_sums = 1e-6 * (x.double().abs() @ w.double().abs().t() + bias.double().abs())
+    assert bool(((got.double() - exact).abs() <= half_step + float32_sums).all())
+    # a bias that bfloat16 does not hold is added to the rounded product (and so is every bias in float32)
+    odd_bias = bias + 2.0 ** -12
+    got = ops.linear(x, w, bias=odd_bias, bias_rounded=None)
+    torch.testing.assert_close(got.float(), (exact + 2.0 ** -12).float(), atol=3e-2, rtol=2e-2)
+    got = ops.linear(x.float(), w.float(), bias=odd_bias)
+    torch.testing.assert_close(got, (exact + 2.0 ** -12).float(), atol=2e-4, rtol=1e-4)
 
 
 @pytest.mark.parametrize("rows", [9, 16, 17, 32, 33, 48, 49, 64, 65, 96, 97, 128])
