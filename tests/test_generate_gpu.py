@@ -24,6 +24,21 @@ def test_greedy_generation_matches_the_plain_implementation(case):
     assert agree >= 20, (got_bf16, expected)             # bfloat16 may leave the greedy path where two logits nearly tie
 
 
+@pytest.mark.parametrize("case", ["A", "B"])
+def test_engine_with_its_default_pages_of_500_tokens(case):
+    """The engine's own defaults (500 pages of 500 tokens, as the reference's engine has them): prompts that end
+    inside the first page and one that crosses into a second, decoded past the page's edge."""
+    from llmserver_amd import Engine, load_model
+    print(f"engine with default pages, case {case}", flush=True)
+    config, tensors = plain_model(case)
+    prompts = [random_tokens(config["vocab_size"], n, 70 + i) for i, n in enumerate((3, 40, 493, 620))]
+    expected = [plain.greedy_generate(config, tensors, prompt, 12) for prompt in prompts]
+    engine = Engine(load_model(model_folder(case), "cuda", "float32"), None, max_new_tokens=12, max_batch_size=4, ignore_eos=True)
+    assert engine.block_size == 500
+    assert engine.generate(prompts) == expected
+    engine.kv_cache.check_invariants()
+
+
 @pytest.mark.parametrize("case", ["A", "B", "C"])
 @pytest.mark.parametrize("rows", [5, 12, 16, 24])
 def test_wide_decode_steps_match_the_plain_implementation(case, rows):
