@@ -7,7 +7,9 @@
 // head.  The wavefront walks the keys in steps, keeps a running maximum and sum per pair (online
 // softmax, 32-bit) and accumulates the output in MFMA registers.  If the item covers every key
 // its pairs can see, it writes the output; otherwise it writes its maximum, sum and unnormalised
-// output to a partial slot and `merge` combines the slots by log-sum-exp.
+// output to a partial slot and `merge` combines the slots by log-sum-exp; where a plan gives every
+// tile four (or two) key ranges, the wavefronts of a workgroup are those ranges and combine them
+// through LDS themselves, without slots and without the second launch.
 //
 // MFMA use (64-lane wavefront, lane = 16 * quad + col):
 //   scores:  S^T[key][pair] = K[key][:] . Q[pair][:]      A = K rows (lane: key col, 8 or 4 dims of quad)
