@@ -140,6 +140,8 @@ def main(argv=None) -> int:
     parser.add_argument("--output-tokens", type=int, default=128)
     parser.add_argument("--repeats", type=int, default=3)
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
+    parser.add_argument("--custom-dtype", default=None, choices=("source", "fp32", "fp16"),
+                        help="the reference's name of --dtype (/root/reference/benchmark.py:344): source = bfloat16 as stored, fp32 = float32; fp16 is not built")
     parser.add_argument("--device", default="cuda")
     parser.add_argument("--block-size", type=int, default=16)
     parser.add_argument("--max-num-batched-tokens", type=int, default=16384)
@@ -157,6 +159,10 @@ def main(argv=None) -> int:
     args = parser.parse_args(argv)
     if (args.model is None) == (args.random_config is None):
         parser.error("pass exactly one of --model and --random-config")
+    if args.custom_dtype == "fp16":
+        parser.error("--custom-dtype fp16: this engine computes in bfloat16 (source) or float32 (fp32) only")
+    if args.custom_dtype is not None:
+        args.dtype = {"source": "bfloat16", "fp32": "float32"}[args.custom_dtype]
 
     import torch
 

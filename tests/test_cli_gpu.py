@@ -28,7 +28,7 @@ def test_matrix_one_prompt_and_mixed_workload(tmp_path, capsys):
     assert results[0]["tokens"][0] == plain.greedy_generate(config, tensors, prompt, 6)
     capsys.readouterr()
     prompt = random_tokens(raw["vocab_size"], 7, 3)
-    assert benchmark.main(["--model", folder, "--dtype", "float32", "--prompt-token-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5",
+    assert benchmark.main(["--model", folder, "--custom-dtype", "fp32", "--prompt-token-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5",
                            "--repeats", "2", "--block-size", str(page)]) == 0
     printed = capsys.readouterr().out
     assert f"Response: {plain.greedy_generate(config, tensors, prompt, 5)}" in printed

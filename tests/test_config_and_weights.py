@@ -172,3 +172,13 @@ def test_random_model_command_writes_a_folder_that_loads_and_repeats(tmp_path):
             assert torch.equal(a.get_tensor(name), b.get_tensor(name).to(torch.bfloat16)), name
     assert os.stat(os.path.join(first, "model.safetensors")).st_mode & 0o044 == 0o044
     assert subprocess.run(command + ["--out", first], capture_output=True).returncode == 2          # neither a config nor a named size
+
+
+def test_benchmark_command_takes_the_reference_name_of_its_dtype_option(capsys):
+    """``--custom-dtype`` (/root/reference/benchmark.py:344): source and fp32 are other names of --dtype; fp16 is refused
+    before anything is loaded."""
+    from llmserver_amd.cli import benchmark
+    with pytest.raises(SystemExit) as refused:
+        benchmark.main(["--random-config", "tiny-a", "--custom-dtype", "fp16"])
+    assert refused.value.code == 2
+    assert "fp16" in capsys.readouterr().err
