@@ -6,6 +6,9 @@
 // row's chunks, finds the chunk in which the running sum passes the target and walks only that
 // chunk.  Maximum, sums and running sums are 32-bit and walk the vocabulary in a fixed order.
 #include "common.hpp"
+#include "sampling.h"
+
+#include <mutex>
 
 using namespace lsa;
 
@@ -121,4 +124,52 @@ LSA_EXPORT int lsa_sample(const float* logits, const float* temperature, const f
     if (err) return err;
     sample_pick_kernel<<<n_rows, 64, 0, stream>>>(logits, temperature, uniform, (const ChunkStat*)workspace, out, vocab, chunk_len, chunks);
     LSA_LAUNCH_CHECK();
+}
+
+// ---- the variant that allocates nothing (declared and described in sampling.h) ----
+static __device__ __align__(256) unsigned char scratch[(size_t)LSA_SAMPLE_STATIC_MAX_ROWS * MAX_CHUNKS * sizeof(ChunkStat)];
+
+constexpr int MOST_DEVICES = 64;
+
+// The address of `scratch` on the current device.  In host code the array's name is only a handle for this lookup,
+// never a device address; every GPU has its own copy at its own address, so the answer is kept per device.
+static int static_scratch(void** address) {
+    static std::mutex guard;
+    static void* known[MOST_DEVICES] = {};
+    int device = -1;
+    hipError_t status = hipGetDevice(&device);
+    if (status != hipSuccess) return (int)status;
+    if (device < 0 || device >= MOST_DEVICES) return LSA_SAMPLE_STATIC_BAD_DEVICE;
+    std::lock_guard<std::mutex> lock(guard);
+    if (known[device] == nullptr) {
+        void* found = nullptr;
+        status = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+        if (status != hipSuccess) return (int)status;
+        if (found == nullptr) return (int)hipErrorInvalidSymbol;
+        known[device] = found;
+    }
+    *address = known[device];
+    return 0;
+}
+
+LSA_EXPORT int lsa_sample_static_max_rows(void) { return LSA_SAMPLE_STATIC_MAX_ROWS; }
+
+LSA_EXPORT const char* lsa_sample_static_error(int code) {
+    switch (code) {
+        case 0: return "no error";
+        case LSA_SAMPLE_STATIC_TOO_MANY_ROWS: return "lsa_sample_static takes at most 1024 rows a call (its fixed scratch array holds no more)";
+        case LSA_SAMPLE_STATIC_BAD_DEVICE: return "lsa_sample_static: the current device's index is outside the table of scratch addresses";
+        default: return hipGetErrorString((hipError_t)code);
+    }
+}
+
+LSA_EXPORT int lsa_sample_static(const float* logits, const float* temperature, const float* uniform, int* out, int n_rows,
+                                 int vocab, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (n_rows > LSA_SAMPLE_STATIC_MAX_ROWS) return LSA_SAMPLE_STATIC_TOO_MANY_ROWS;
+    void* stats = nullptr;
+    const int status = static_scratch(&stats);
+    if (status) return status;
+    // Every (row, chunk) entry that the second kernel reads is written by the first: nothing of an earlier call is seen.
+    return lsa_sample(logits, temperature, uniform, out, stats, n_rows, vocab, stream);
 }

@@ -58,7 +58,9 @@ def all_modules(head_dims: Iterable[int] = (64, 128)) -> List[str]:
 def _hash(name: str) -> str:
     source, extra = module_recipe(name)
     digest = hashlib.sha256()
-    for path in (os.path.join(CSRC, source), os.path.join(CSRC, "common.hpp")):
+    own_header = os.path.join(CSRC, os.path.splitext(source)[0] + ".h")          # its entry points' declarations, if it has any
+    paths = [os.path.join(CSRC, source), os.path.join(CSRC, "common.hpp")] + ([own_header] if os.path.isfile(own_header) else [])
+    for path in paths:
         with open(path, "rb") as handle:
             digest.update(handle.read())
     digest.update(" ".join(FLAGS + extra).encode())

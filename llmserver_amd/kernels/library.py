@@ -19,6 +19,8 @@ _SIGNATURES = {
     "lsa_rotary_table": [_P, _P, _P, c_int, c_int, _P],
     "lsa_sample": [_P, _P, _P, _P, _P, c_int, c_int, _P],
     "lsa_sample_chunks": [c_int],
+    "lsa_sample_static": [_P, _P, _P, _P, c_int, c_int, _P],
+    "lsa_sample_static_max_rows": [],
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, c_int,
                             c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, _P],
     "lsa_attention_workgroup_tiles": [],

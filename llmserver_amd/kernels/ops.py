@@ -592,6 +592,21 @@ class HipOps:
         _launched(self._sampling.lsa_sample(_ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), _ptr(workspace), n, vocab,
                                             _stream()), "sample")
 
+    def sample_no_alloc(self, logits, temperature, uniform, out):
+        """:meth:`sample` for callers that must not allocate (a graph under capture, for one): the per-chunk statistics
+        lie in a fixed array inside the library instead of a workspace tensor.  At most
+        ``lsa_sample_static_max_rows()`` rows; calls that overlap on one GPU race on that array."""
+        n, vocab = logits.shape
+        _check(logits, "logits", torch.float32)
+        _check(temperature, "temperature", torch.float32, (n,))
+        _check(uniform, "uniform", torch.float32, (n,))
+        _check(out, "out", torch.int32, (n,))
+        most = self._sampling.lsa_sample_static_max_rows()
+        if n > most:
+            raise ValueError(f"sampling without a workspace takes at most {most} rows, got {n}")
+        _launched(self._sampling.lsa_sample_static(_ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), n, vocab, _stream()),
+                  "sample_static")
+
 
 _default = None
 
