@@ -9,8 +9,13 @@ there are slots for per-request state of fixed size.
 Page layout (one cache, i.e. one layer): keys ``[pages, kv_heads, page_size, head_dim]``, values
 transposed ``[pages, kv_heads, head_dim, page_size]``, so that both attention products read each
 lane's operand as one contiguous vector.  The reference keeps ``[layers, blocks, block_size,
-kv_heads, head_dim]`` for both (/root/reference/utils/kv_cache.py:84-89); its allocator
-semantics are in :mod:`.pages`.
+kv_heads, head_dim]`` for both (utils/kv_cache.py:84-89 in the reference); the pages' states and
+queues are in :mod:`.pages`.
+
+Whoever plans a step asks this manager, never a block table, what the plan would cost: :meth:`pages_needed` and
+:meth:`available_pages` answer per group, :meth:`token_room` says how far a request could grow on a given number
+of pages in every group, :meth:`holds_anything` whether giving a request up would free anything.  A request's record
+can be opened without a state slot (a request that waits computes nothing) and take one later (:meth:`acquire_state`).
 """
 from __future__ import annotations
 
@@ -153,18 +158,36 @@ class CacheManager:
         return LayerCacheView(-1, None, None, self.page_size, call.writes_cache)
 
     # -- requests ------------------------------------------------------------------------
-    def open(self, request_id) -> RequestCache:
+    def open(self, request_id, state: bool = True) -> RequestCache:
+        """A record for a new request: empty block tables and, unless ``state`` is False, a state slot (if any mixer
+        keeps state).  Nothing is opened if no slot is free."""
         if request_id in self.requests:
             raise CacheStateError(f"request {request_id!r} already has a cache")
         record = RequestCache(request_id, len(self.groups))
-        if self.state_specs:
-            if not self.free_state_slots:
-                raise CacheExhaustedError(f"no state slot is free: num_state_slots: {self.num_state_slots}")
-            record.state_slot = self.free_state_slots.pop()
-            for tensor in self.state.values():
-                tensor[record.state_slot].zero_()
+        if state:
+            self._take_slot(record)
         self.requests[request_id] = record
         return record
+
+    def _take_slot(self, record: RequestCache) -> None:
+        if not self.state_specs or record.state_slot >= 0:
+            return
+        if not self.free_state_slots:
+            raise CacheExhaustedError(f"all {self.num_state_slots} state slots are taken")
+        record.state_slot = self.free_state_slots.pop()
+        for tensor in self.state.values():
+            tensor[record.state_slot].zero_()            # a state starts from nothing
+
+    def acquire_state(self, request_id) -> int:
+        """The request is about to compute: give it a state slot (zeroed) if mixers keep state and it has none yet.
+        Returns the slot, -1 for a model without state."""
+        record = self.record(request_id)
+        self._take_slot(record)
+        return record.state_slot
+
+    def state_slots_free(self) -> Optional[int]:
+        """How many more requests can get a state slot; None if no mixer keeps state (then nothing limits them)."""
+        return len(self.free_state_slots) if self.state_specs else None
 
     def has(self, request_id) -> bool:
         return request_id in self.requests
@@ -185,6 +208,24 @@ class CacheManager:
 
     def available_pages(self) -> List[int]:
         return [group.pool.num_available for group in self.groups]
+
+    def token_room(self, request_id, spare_pages: Sequence[int]) -> int:
+        """The number of leading positions of the request that its pages would cover if every group gave it
+        ``spare_pages[group]`` more (what it holds already counts).  Without paged groups nothing bounds it."""
+        record = self.requests.get(request_id)
+        room = None
+        for group in self.groups:
+            have = len(record.tables[group.index]) if record is not None else 0
+            covered = (have + max(0, int(spare_pages[group.index]))) * self.page_size
+            room = covered if room is None else min(room, covered)
+        return (1 << 62) if room is None else room
+
+    def holds_anything(self, request_id) -> bool:
+        """Whether closing the request's record would give anything back: a page in any group, or a state slot."""
+        record = self.requests.get(request_id)
+        if record is None:
+            return False
+        return record.state_slot >= 0 or any(page >= 0 for table in record.tables for page in table)
 
     def ensure(self, request_id, num_tokens: int) -> None:
         """Allocate pages so that positions ``< num_tokens`` have a place in every group.
@@ -229,7 +270,7 @@ class CacheManager:
         """The request ended (or is preempted): everything it holds is given back."""
         record = self.record(request_id)
         for group in self.groups:
-            group.pool.release_table(record.tables[group.index])
+            group.pool.release_all(record.tables[group.index])
         if record.state_slot >= 0:
             self.free_state_slots.append(record.state_slot)
             record.state_slot = -1
@@ -238,7 +279,7 @@ class CacheManager:
     # -- prefix caching (complete pages of prompt tokens) ------------------------------------
     def digest(self, parent: str, tokens: Sequence[int]) -> str:
         """Chained sha256 over (parent digest, page tokens, model, adapter), root parent "root"
-        (/root/reference/utils/engine.py:193-195)."""
+        (utils/engine.py:193-195)."""
         payload = json.dumps([parent, list(tokens), self.model_identity, "none"], separators=(",", ":")).encode("utf-8")
         return hashlib.sha256(payload).hexdigest()
 
@@ -253,7 +294,7 @@ class CacheManager:
 
     def share_prefix(self, request_id, prompt: Sequence[int], digests: Optional[List[str]] = None) -> int:
         """Attach the longest chain of cached complete pages; always leaves at least one prompt
-        token to compute (/root/reference/utils/engine.py:197-208).  May be called again while
+        token to compute (utils/engine.py:197-208).  May be called again while
         the request has computed nothing itself: the chain is then continued.  Returns the
         tokens newly covered."""
         if not self.prefix_caching_possible:
@@ -266,17 +307,17 @@ class CacheManager:
             digests = self.prefix_digests(prompt)
         covered = 0
         for digest in digests[have:]:
-            if any(group.pool.find(digest) is None for group in self.groups):
+            if any(group.pool.lookup(digest) is None for group in self.groups):
                 break
             for group in self.groups:
-                group.pool.share(digest, record.tables[group.index])
+                group.pool.adopt(digest, record.tables[group.index])
             covered += self.page_size
         record.num_computed += covered
         return covered
 
     def register_prefix(self, request_id, prompt: Sequence[int], old_computed: int, new_computed: int) -> None:
         """Register pages of prompt tokens that became complete between two counts of computed
-        tokens (/root/reference/utils/engine.py:383-401)."""
+        tokens (utils/engine.py:383-401)."""
         if not self.prefix_caching_possible:
             return
         record = self.record(request_id)
@@ -286,8 +327,8 @@ class CacheManager:
             tokens = prompt[block * self.page_size:(block + 1) * self.page_size]
             for group in self.groups:
                 table = record.tables[group.index]
-                parent = "root" if block == 0 else group.pool.page_digest[table[block - 1]]
-                group.pool.register(table[block], self.digest(parent, tokens))
+                parent = "root" if block == 0 else group.pool.digest[table[block - 1]]
+                group.pool.publish(table[block], self.digest(parent, tokens))
 
     def check_invariants(self) -> None:
         for group in self.groups:
@@ -298,8 +339,8 @@ class CacheManager:
                     if page >= 0:
                         held[page] = held.get(page, 0) + 1
             for page in range(group.pool.num_pages):
-                assert group.pool.references[page] == held.get(page, 0), (
-                    f"group {group.index} page {page}: {group.pool.references[page]} references, {held.get(page, 0)} holders")
+                assert group.pool.holders[page] == held.get(page, 0), (
+                    f"group {group.index} page {page}: the pool counts {group.pool.holders[page]} holders, {held.get(page, 0)} tables list it")
         slots = [record.state_slot for record in self.requests.values() if record.state_slot >= 0]
         assert len(slots) == len(set(slots)), "a state slot is held twice"
         assert not set(slots) & set(self.free_state_slots), "a held state slot is on the free list"

@@ -1,155 +1,217 @@
-"""Page allocator of one cache group: free list, reference counts, complete-page prefix hashes.
+"""The pages of one cache group and who has them.
 
-Semantics follow the reference's paged cache (/root/reference/utils/kv_cache.py:93-189):
-pages come off the head of a FIFO free list; a page whose last reference goes away returns to
-the tail of the free list, unless it holds a registered complete page of prompt tokens, in
-which case it stays "idle" in least-recently-used order and can be shared again by digest; an
-allocation that finds the free list empty evicts the oldest idle page, and fails with
-:class:`CacheExhaustedError` only if there is none.
+Every page is in exactly one of three states.  FREE: nobody lists it and its content is worth nothing.  HELD: at
+least one block table lists it (``holders`` counts the tables).  IDLE: nobody lists it, but it still holds a complete
+page of prompt tokens that was published under a digest, so a later request with the same prefix can adopt it.
+FREE and IDLE pages stand in two queues that are threaded through one pair of link arrays (a page is never in
+both): new pages come from the front of the FREE queue and given-back pages join its end, so a page that was just
+given back is the last to be written again; when no page is FREE the page that has been IDLE longest is recycled.
+
+What the reference's paged cache does with a free deque, a set of allocated blocks, a set of cacheable blocks, two
+digest maps and an ordered dict of idle blocks (utils/kv_cache.py:93-189) is one state and one digest per page here;
+the outcomes its tests pin (order of reuse, eviction of the oldest idle block, errors on double frees) are the same.
 """
 from __future__ import annotations
 
-from collections import OrderedDict, deque
-from typing import List, Optional
+import enum
+from typing import Dict, List, Optional
 
 
 class CacheExhaustedError(BufferError):
-    """No page is free and none can be evicted (/root/reference/utils/kv_cache.py:516)."""
+    """No page is free and none can be recycled (utils/kv_cache.py:516 in the reference)."""
 
 
 class CacheStateError(RuntimeError):
-    """A page or slot is used in a way its state forbids (/root/reference/utils/kv_cache.py:519)."""
+    """A page or slot is used in a way its state forbids (utils/kv_cache.py:519 in the reference)."""
+
+
+class PageState(enum.IntEnum):
+    FREE = 0
+    IDLE = 1
+    HELD = 2
+
+
+class _Queue:
+    """A first-in first-out queue of page numbers, linked through arrays it shares with its sibling."""
+
+    def __init__(self, following: List[int], preceding: List[int]):
+        self.following, self.preceding = following, preceding
+        self.first = self.last = -1
+        self.count = 0
+
+    def join(self, page: int) -> None:
+        self.following[page], self.preceding[page] = -1, self.last
+        if self.last >= 0:
+            self.following[self.last] = page
+        else:
+            self.first = page
+        self.last = page
+        self.count += 1
+
+    def leave(self, page: int) -> None:
+        before, after = self.preceding[page], self.following[page]
+        if before >= 0:
+            self.following[before] = after
+        else:
+            self.first = after
+        if after >= 0:
+            self.preceding[after] = before
+        else:
+            self.last = before
+        self.following[page] = self.preceding[page] = -1
+        self.count -= 1
+
+    def __iter__(self):
+        page = self.first
+        while page >= 0:
+            yield page
+            page = self.following[page]
 
 
 class PagePool:
     def __init__(self, num_pages: int, page_size: int):
-        if num_pages <= 0:
-            raise ValueError(f"num_pages must be positive: {num_pages}")
-        if page_size <= 0:
-            raise ValueError(f"page_size must be positive: {page_size}")
+        if num_pages <= 0 or page_size <= 0:
+            raise ValueError(f"a pool needs a positive number of pages of a positive size, got {num_pages} pages of {page_size}")
         self.num_pages, self.page_size = num_pages, page_size
-        self.free_pages = deque(range(num_pages))
-        self.references = [0] * num_pages
-        self.allocated = set()
-        self.cacheable = set()
-        self.page_digest = {}
-        self.digest_to_page = {}
-        self.idle_lru: "OrderedDict[int, str]" = OrderedDict()
+        self.state = [PageState.FREE] * num_pages
+        self.holders = [0] * num_pages                         # block tables that list the page
+        self.digest: List[Optional[str]] = [None] * num_pages  # what the page's tokens (and all before them) hash to, once complete
+        self.by_digest: Dict[str, int] = {}                    # the one page that may be adopted under a digest
+        following, preceding = [-1] * num_pages, [-1] * num_pages
+        self._free, self._idle = _Queue(following, preceding), _Queue(following, preceding)
+        for page in range(num_pages):
+            self._free.join(page)
 
-    # -- counts ------------------------------------------------------------------------
+    # -- counts ----------------------------------------------------------------------------
     @property
     def num_free(self) -> int:
-        return len(self.free_pages)
+        return self._free.count
 
     @property
     def num_idle(self) -> int:
-        return len(self.idle_lru)
+        return self._idle.count
 
     @property
     def num_available(self) -> int:
-        """Pages an allocation can get: free ones and idle cached ones (/root/reference/utils/engine.py:420)."""
-        return len(self.free_pages) + len(self.idle_lru)
+        """Pages that :meth:`allocate` can hand out: the free ones and the idle ones it may recycle."""
+        return self._free.count + self._idle.count
 
-    def _check_id(self, page: int):
-        if page < 0 or page >= self.num_pages:
-            raise ValueError(f"Page id {page} is invalid, num_pages is {self.num_pages}")
+    def _state_of(self, page: int) -> PageState:
+        if not 0 <= page < self.num_pages:
+            raise ValueError(f"there is no page {page} in a pool of {self.num_pages}")
+        return self.state[page]
 
-    # -- allocate / retain / release -------------------------------------------------------
+    def is_published(self, page: int) -> bool:
+        digest = self.digest[page]
+        return digest is not None and self.by_digest.get(digest) == page
+
+    def published_pages(self) -> set:
+        return set(self.by_digest.values())
+
+    # -- taking and giving back --------------------------------------------------------------
+    def _forget(self, page: int) -> None:
+        digest, self.digest[page] = self.digest[page], None
+        if digest is not None and self.by_digest.get(digest) == page:
+            del self.by_digest[digest]
+
     def allocate(self) -> int:
-        if not self.free_pages:
-            if not self.idle_lru:
-                raise CacheExhaustedError(f"Cache is out of pages: num_pages: {self.num_pages}, free: 0")
-            self._discard(next(iter(self.idle_lru)))
-        page = self.free_pages.popleft()
-        self.allocated.add(page)
-        self.references[page] = 1
+        """A page for one block table to write into."""
+        if self._free.count:
+            page = self._free.first
+            self._free.leave(page)
+        elif self._idle.count:
+            page = self._idle.first                  # idle longest: its cached tokens are given up
+            self._idle.leave(page)
+            self._forget(page)
+        else:
+            raise CacheExhaustedError(f"all {self.num_pages} pages of the pool are held")
+        self.state[page], self.holders[page] = PageState.HELD, 1
         return page
 
-    def retain(self, page: int) -> None:
-        self._check_id(page)
-        if page not in self.allocated:
-            raise CacheStateError(f"Page {page} cannot be retained, it is not allocated")
-        if self.references[page] == 0:
-            self.idle_lru.pop(page, None)
-        self.references[page] += 1
+    def hold(self, page: int) -> None:
+        """One more block table lists ``page``."""
+        state = self._state_of(page)
+        if state == PageState.FREE:
+            raise CacheStateError(f"page {page} is free: there is nothing on it to hold on to")
+        if state == PageState.IDLE:
+            self._idle.leave(page)
+            self.state[page] = PageState.HELD
+        self.holders[page] += 1
 
     def release(self, page: int) -> None:
-        self._check_id(page)
-        if page not in self.allocated:
-            raise CacheStateError(f"Page {page} cannot be freed, it is not allocated")
-        if self.references[page] == 0:
-            raise CacheStateError(f"Page {page} cannot be freed, it has no active references")
-        self.references[page] -= 1
-        if self.references[page] > 0:
+        """One block table lists ``page`` no longer."""
+        if self._state_of(page) != PageState.HELD:
+            raise CacheStateError(f"page {page} is given back, but nobody holds it")
+        self.holders[page] -= 1
+        if self.holders[page]:
             return
-        digest = self.page_digest.get(page)
-        if page in self.cacheable and digest is not None and self.digest_to_page.get(digest) == page:
-            self.idle_lru[page] = digest
-            return
-        self._discard(page)
+        if self.is_published(page):
+            self.state[page] = PageState.IDLE
+            self._idle.join(page)
+        else:
+            self._forget(page)
+            self.state[page] = PageState.FREE
+            self._free.join(page)
 
-    def _discard(self, page: int) -> None:
-        self.idle_lru.pop(page, None)
-        digest = self.page_digest.pop(page, None)
-        if digest is not None and self.digest_to_page.get(digest) == page:
-            del self.digest_to_page[digest]
-        self.allocated.discard(page)
-        self.cacheable.discard(page)
-        self.free_pages.append(page)
-
-    def release_table(self, table: List[int]) -> None:
-        """Give back every page of a block table (entries < 0 were given back earlier); validates first."""
-        seen = set()
-        for page in table:
-            if page < 0:
-                continue
-            if page not in self.allocated:
-                raise CacheStateError(f"Page {page} cannot be freed, it is not allocated")
-            if self.references[page] == 0:
-                raise CacheStateError(f"Page {page} cannot be freed, it has no active references")
-            if page in seen:
-                raise ValueError(f"Duplicate page id {page} found")
-            seen.add(page)
-        for page in table:
-            if page >= 0:
-                self.release(page)
+    def release_all(self, table: List[int]) -> None:
+        """Give back every page a block table lists (negative entries were given back earlier) and empty the table.
+        Nothing is given back if any entry is wrong."""
+        listed = [page for page in table if page >= 0]
+        if len(set(listed)) != len(listed):
+            raise ValueError(f"a block table lists a page twice: {sorted(listed)}")
+        for page in listed:
+            if self._state_of(page) != PageState.HELD:
+                raise CacheStateError(f"page {page} is given back, but nobody holds it")
+        for page in listed:
+            self.release(page)
         table.clear()
 
-    # -- prefix caching ------------------------------------------------------------------
-    def register(self, page: int, digest: str) -> None:
-        """Mark a complete page of prompt tokens shareable under ``digest``
-        (/root/reference/utils/engine.py:387-401)."""
-        if page not in self.allocated:
-            raise CacheStateError(f"Page {page} cannot be cached, it isn't currently allocated")
-        self.cacheable.add(page)
-        self.page_digest[page] = digest
-        self.digest_to_page.setdefault(digest, page)
+    # -- complete pages of prompt tokens, shared by digest -------------------------------------------
+    def publish(self, page: int, digest: str) -> None:
+        """``page`` is complete; its tokens and everything before them hash to ``digest``.  The first page published
+        under a digest is the one later requests adopt (utils/engine.py:387-401 in the reference)."""
+        if self._state_of(page) != PageState.HELD:
+            raise CacheStateError(f"page {page} cannot be published: nobody holds it")
+        if self.digest[page] != digest:
+            self._forget(page)
+            self.digest[page] = digest
+        self.by_digest.setdefault(digest, page)
 
-    def find(self, digest: str) -> Optional[int]:
-        page = self.digest_to_page.get(digest)
-        if page is None or page not in self.allocated or page not in self.cacheable:
-            return None
-        if self.page_digest.get(page) != digest:
+    def lookup(self, digest: str) -> Optional[int]:
+        page = self.by_digest.get(digest)
+        if page is None or self.state[page] == PageState.FREE or self.digest[page] != digest:
             return None
         return page
 
-    def share(self, digest: str, table: List[int]) -> Optional[int]:
-        """Append the page registered under ``digest`` to ``table`` and retain it
-        (/root/reference/utils/kv_cache.py:124-135)."""
-        page = self.find(digest)
+    def adopt(self, digest: str, table: List[int]) -> Optional[int]:
+        """Append the page published under ``digest`` to ``table``; None if there is none."""
+        page = self.lookup(digest)
         if page is None:
             return None
         if page in table:
-            raise ValueError("One request must not list the same physical page twice")
-        self.retain(page)
+            raise ValueError(f"page {page} is already in this block table")
+        self.hold(page)
         table.append(page)
         return page
 
+    # -- self-check ----------------------------------------------------------------------------
     def check_invariants(self) -> None:
-        """Every page is in exactly one of: free list, idle, referenced."""
-        free = list(self.free_pages)
-        assert len(free) == len(set(free)), "a page is on the free list twice"
+        """Every page is in the one place its state names, and the digests point both ways."""
+        queued = {PageState.FREE: list(self._free), PageState.IDLE: list(self._idle)}
+        assert len(queued[PageState.FREE]) == self._free.count and len(queued[PageState.IDLE]) == self._idle.count, "a queue lost count"
+        seen = queued[PageState.FREE] + queued[PageState.IDLE]
+        assert len(seen) == len(set(seen)), "a page stands in a queue twice"
+        for state, pages in queued.items():
+            for page in pages:
+                assert self.state[page] == state, f"page {page} stands in the {state.name} queue but is {self.state[page].name}"
         for page in range(self.num_pages):
-            states = (page in self.free_pages) + (page in self.idle_lru) + (self.references[page] > 0)
-            assert states == 1, f"page {page} is in {states} states"
-            assert (page in self.allocated) == (page not in self.free_pages)
+            state = self.state[page]
+            assert (self.holders[page] > 0) == (state == PageState.HELD), f"page {page} is {state.name} with {self.holders[page]} holders"
+            if state != PageState.HELD:
+                assert page in seen, f"page {page} is {state.name} but in no queue"
+            if state == PageState.FREE:
+                assert self.digest[page] is None, f"free page {page} still has a digest"
+            if state == PageState.IDLE:
+                assert self.is_published(page), f"idle page {page} is not published"
+        for digest, page in self.by_digest.items():
+            assert self.digest[page] == digest and self.state[page] != PageState.FREE, f"digest of page {page} points nowhere"

@@ -72,6 +72,8 @@ class Qwen3Config(ModelConfig):
                    f"query heads: {self.num_attention_heads}, KV heads: {self.num_key_value_heads}")
         if self.head_dim % 2 != 0:
             reject(f"rotate-half position encoding needs an even head_dim: {self.head_dim}")
+        if self.head_dim % 16 != 0 or not 16 <= self.head_dim <= 256:
+            reject(f"the attention kernels take head sizes 16, 32, ..., 256; got {self.head_dim}")
         use_sliding = raw.get("use_sliding_window")
         if use_sliding is None:
             use_sliding = raw.get("sliding_window") is not None

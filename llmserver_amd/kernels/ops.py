@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import torch
 
-from ..parts.attention import group_tiling
+from ..parts.attention import AttentionTuning, group_tiling
 from . import build, library
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -87,6 +87,29 @@ class HipOps:
         self._library_faster = {}   # (kind, rows, out, in, scaled, float32 result) -> bool
         self._flush = None
         self._replay_overhead = None
+        self._tuning = None
+
+    @property
+    def attention_tuning(self) -> AttentionTuning:
+        """What the attention plan should know of this GPU: four wavefronts in flight per compute unit (more and shorter
+        key ranges cost more in the merge than they gain), and what a 32-key step of the prompt-portion kernel
+        costs with four and with eight tiles to a workgroup (measured on an MI355X: with every compute unit busy 2.0 ns
+        per tile-row against 2.75 ns for twice the tiles; alone on the chip 1.37 against 1.40 us a step)."""
+        if self._tuning is None:
+            units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+            self._tuning = AttentionTuning(target_waves=4 * units, step_ns_four_tiles=2.0, step_ns_most_tiles=2.75,
+                                           lone_step_us_four_tiles=1.37, lone_step_us_most_tiles=1.40)
+        return self._tuning
+
+    @staticmethod
+    def check_cache_geometry(cache_specs, page_size: int) -> None:
+        """Refuse, before anything is allocated, a cache that the attention kernels cannot read."""
+        if page_size % 4:
+            raise ValueError(f"the attention kernel reads values four keys at a time: page_size must be a multiple of 4, got {page_size}")
+        for spec in cache_specs.values():
+            head_dim = getattr(spec, "head_dim", None)
+            if head_dim is not None:
+                build.attention_module(True, head_dim)      # raises with the sizes the kernels take
 
     @staticmethod
     def required_modules(head_dims, dtype):

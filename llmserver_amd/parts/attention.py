@@ -20,7 +20,8 @@ whose partial results a second kernel merges by log-sum-exp, the reference's spl
 """
 from __future__ import annotations
 
-from typing import Optional
+import dataclasses
+from typing import Optional, Tuple
 
 import numpy as np
 
@@ -30,8 +31,39 @@ from .linear import Linear
 TILE_ROWS = 16          # rows of (token, group head) pairs one wavefront handles (MFMA N dimension)
 KEY_ALIGN = 32          # key ranges of split items start at multiples of this
 MAX_SPLITS = 128        # key ranges per tile (the merge kernel's limit, which the kernel namespace checks)
-MIN_KEYS_PER_SPLIT = 64     # shorter key ranges than this are not worth a wavefront of their own (measured at batch 1 to 8)
-TARGET_WAVES = 1024     # wavefronts wanted in flight on 256 CUs (measured: more and shorter items cost more in the merge than they gain)
+MIN_KEYS_PER_SPLIT = 64     # shorter key ranges than this are not worth a wavefront of their own
+
+
+@dataclasses.dataclass(frozen=True)
+class AttentionTuning:
+    """What the plan needs to know of the machine and its kernels; the kernel namespace of a step supplies it
+    (``ops.attention_tuning``), these defaults stand where it does not.
+
+    ``target_waves``: wavefronts wanted in flight; rows with few tokens and long contexts are cut into key ranges
+    until there are about that many.  The other four describe the prompt-portion kernel, whose workgroups take four
+    tiles or ``most`` tiles: nanoseconds of a 32-key step per tile-row when every compute unit is busy, and
+    microseconds of such a step when a workgroup has the machine to itself (then the longest workgroup bounds the
+    launch)."""
+    target_waves: int = 1024
+    step_ns_four_tiles: float = 1.0
+    step_ns_most_tiles: float = 1.0
+    lone_step_us_four_tiles: float = 1.0
+    lone_step_us_most_tiles: float = 1.0
+
+
+DEFAULT_TUNING = AttentionTuning()
+TARGET_WAVES = DEFAULT_TUNING.target_waves
+
+
+@dataclasses.dataclass(frozen=True)
+class AttentionNames:
+    """Checkpoint names of an attention layer's tensors, relative to the layer.  ``qkv`` lists the tensors whose rows,
+    stacked in this order, are the query, key and value projections: three tensors, two (queries; keys and values
+    together) or one that holds all three.  The defaults are the names most decoder checkpoints use."""
+    qkv: Tuple[str, ...] = ("q_proj", "k_proj", "v_proj")
+    out: str = "o_proj"
+    q_norm: str = "q_norm"
+    k_norm: str = "k_norm"
 
 
 def group_tiling(group_size: int):
@@ -72,14 +104,14 @@ def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: i
 MIN_TILES_FOR_WORKGROUPS = 16      # rows with at least this many tiles go to the prompt-portion kernel
 
 
-def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, heads, window, most: int) -> int:
+def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, heads, window, most: int,
+                              tuning: AttentionTuning = DEFAULT_TUNING) -> int:
     """4 or ``most`` tiles per workgroup of the prompt-portion kernel, whichever the step's rows finish sooner with.
 
-    A workgroup walks its keys in steps of 32.  With all compute units busy, eight tiles per workgroup get more out of
-    every step (measured on Qwen3-8B shapes: 2.75 ns a step against 2 x 2.0 ns for the same tokens in two workgroups
-    of four; setting up and draining a workgroup costs about 8 steps more), but a step of theirs takes longer
-    (1.40 against 1.37 us), and the workgroup with the most steps bounds the launch from below: one short prompt
-    finishes sooner with four, long rows and many rows with eight."""
+    A workgroup walks its keys in steps of 32.  With all compute units busy, more tiles per workgroup get more out of
+    every step (setting up and draining a workgroup costs about 8 steps more), but a step of theirs takes longer, and
+    the workgroup with the most steps bounds the launch from below: one short prompt finishes sooner with four, long
+    rows and many rows with ``most``.  The costs of a step are the tuning's."""
     if most <= 4:
         return most
     def estimate(per_workgroup, ns_per_step, us_per_step_alone):
@@ -96,7 +128,8 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
             total += int(steps.sum()) + 8 * len(steps)
             longest = max(longest, int(steps.max()))
         return max(total * heads * ns_per_step * 1e-3, longest * us_per_step_alone)
-    return most if estimate(most, 2.75, 1.40) < estimate(4, 2.0, 1.37) else 4
+    return most if estimate(most, tuning.step_ns_most_tiles, tuning.lone_step_us_most_tiles) \
+        < estimate(4, tuning.step_ns_four_tiles, tuning.lone_step_us_four_tiles) else 4
 
 
 WORKGROUP_RANGES = 4    # key ranges of a tile that one workgroup (four wavefronts) walks and merges itself
@@ -137,7 +170,8 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, 
 
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
-                         workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: int = 0) -> AttentionPlan:
+                         workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: int = 0,
+                         tuning: AttentionTuning = DEFAULT_TUNING) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
@@ -160,7 +194,7 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     items, slots, merges, tiles = [], [], [], []
     n_slots = 0
     per_workgroup = _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window,
-                                              int(workgroup_tiles)) if workgroup_tiles and fixed_splits is None else 0
+                                              int(workgroup_tiles), tuning) if workgroup_tiles and fixed_splits is None else 0
     for row in range(len(row_len)):
         n, ctx = int(row_len[row]), int(row_ctx[row])
         first_pos = ctx - n
@@ -212,7 +246,7 @@ class GQAttention(Mixer):
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  qk_norm_eps: Optional[float] = None, bias: bool = False, out_bias: Optional[bool] = None,
-                 window: Optional[int] = None, scale: Optional[float] = None):
+                 window: Optional[int] = None, scale: Optional[float] = None, names: AttentionNames = AttentionNames()):
         if n_heads % n_kv_heads:
             raise ValueError(f"Number of query heads must be divisible by the number of KV heads: query heads: {n_heads}, KV heads: {n_kv_heads}")
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
@@ -221,9 +255,13 @@ class GQAttention(Mixer):
         self.qk_norm_eps = qk_norm_eps
         self.window = window
         self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
-        self.qkv = Linear(width, ("q_proj", "k_proj", "v_proj"),
-                          (n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * head_dim), bias)
-        self.o = Linear(n_heads * head_dim, ("o_proj",), (width,), bias if out_bias is None else out_bias)
+        q_rows, kv_rows = n_heads * head_dim, n_kv_heads * head_dim
+        stacked = {3: (q_rows, kv_rows, kv_rows), 2: (q_rows, 2 * kv_rows), 1: (q_rows + 2 * kv_rows,)}
+        if len(names.qkv) not in stacked:
+            raise ValueError(f"queries, keys and values come in one, two or three checkpoint tensors, not {len(names.qkv)}")
+        self.names = names
+        self.qkv = Linear(width, names.qkv, stacked[len(names.qkv)], bias)
+        self.o = Linear(q_rows, (names.out,), (width,), bias if out_bias is None else out_bias)
         self.q_norm_weight = None
         self.k_norm_weight = None
 
@@ -233,19 +271,22 @@ class GQAttention(Mixer):
     def param_specs(self):
         specs = {**self.qkv.param_specs(), **self.o.param_specs()}
         if self.qk_norm_eps is not None:
-            specs["q_norm.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
-            specs["k_norm.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
+            specs[f"{self.names.q_norm}.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
+            specs[f"{self.names.k_norm}.weight"] = ParamSpec((self.head_dim,), VECTOR, "norm")
         return specs
 
     def assign(self, name, tensor):
-        if name == "q_norm.weight":
+        owner = name.rsplit(".", 1)[0]
+        if owner == self.names.q_norm:
             self.q_norm_weight = tensor
-        elif name == "k_norm.weight":
+        elif owner == self.names.k_norm:
             self.k_norm_weight = tensor
-        elif name.startswith("o_proj."):
+        elif owner == self.names.out:
             self.o.assign(name, tensor)
-        else:
+        elif owner in self.names.qkv:
             self.qkv.assign(name, tensor)
+        else:
+            raise KeyError(name)
 
     def finalize(self):
         self.qkv.finalize()
@@ -259,8 +300,9 @@ class GQAttention(Mixer):
         if ctx.has_plan(key):
             return
         fixed = None
+        tuning = getattr(ctx.ops, "attention_tuning", None) or DEFAULT_TUNING
         if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
-            fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys)
+            fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves)
         # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:
         #  * short contexts (the step says so, and keeps saying so for as long as its shape is replayed): four ranges a tile;
         #  * so many rows that a tile gets four ranges anyway;
@@ -275,7 +317,8 @@ class GQAttention(Mixer):
         per_workgroup = getattr(ctx.ops, "attention_workgroup_tiles", None)
         per_workgroup = per_workgroup(ctx.dtype, self.head_dim) if per_workgroup is not None else 0
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
-                                    fixed_splits=fixed, workgroup_tiles=per_workgroup, merge_in_workgroup=in_workgroup)
+                                    target_waves=tuning.target_waves, fixed_splits=fixed, workgroup_tiles=per_workgroup,
+                                    merge_in_workgroup=in_workgroup, tuning=tuning)
         ctx.set_plan(key, {
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
             "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),

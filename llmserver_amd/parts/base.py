@@ -64,12 +64,22 @@ class Norm(Part):
     ``add_norm(resid, delta, ctx, rows=None)`` computes ``s = resid + delta`` in 32-bit (``delta``
     may be None), stores ``s`` back into ``resid`` and returns ``norm(s)``; with ``rows`` (int32
     device tensor) only those token rows are normalised and returned, ``resid`` is left alone.
-    A norm with ``weight`` and ``eps`` attributes (an RMSNorm) may be handed ``delta`` as float32
-    partial sums ``[parts, T, H]`` by a projection that was told this norm follows it.
+
+    ``row_scale_form()`` is how a norm tells the projections around it that it can be folded into them: a norm of
+    the form ``s * rsqrt(mean(s^2) + eps) * weight`` returns ``(weight, eps)`` and must then also accept ``delta`` as
+    float32 partial sums ``[parts, T, H]`` (a projection that was told this norm follows it may leave its result so);
+    any other norm returns None and always runs in a kernel of its own.
     """
 
     def add_norm(self, resid, delta, ctx, rows=None):
         raise NotImplementedError
+
+    def row_scale_form(self):
+        return None
+
+    def defer(self, resid, delta, ctx) -> "PendingNorm":
+        """The same normalisation, left to whoever consumes it (a projection may fold it in)."""
+        return PendingNorm(self, resid, delta, ctx)
 
 
 class StreamUpdate:
@@ -112,9 +122,10 @@ class PendingNorm:
 
     def row_scale(self):
         """``(weighted stream, (square_sums, eps))`` if a projection may apply the norm as a row scale, else None."""
-        if self.prepared is None or self.prepared.weighted is None or self._done is not None or not hasattr(self.norm, "eps"):
+        form = self.norm.row_scale_form()
+        if self.prepared is None or self.prepared.weighted is None or self._done is not None or form is None:
             return None
-        return self.prepared.weighted, (self.prepared.square_sums, self.norm.eps)
+        return self.prepared.weighted, (self.prepared.square_sums, form[1])
 
 
 class ResidualSink:

@@ -40,7 +40,7 @@ class PreNormBlock(Block):
         :class:`StreamUpdate`); otherwise the norm runs first, in its own kernel.  A consumer that
         ends with a projection is told the norm that follows its output (``following``), so that
         this projection may in turn add its result to the stream and prepare that norm."""
-        if consumer.accepts_pending_norm and hasattr(norm, "defer"):
+        if consumer.accepts_pending_norm:
             pending = norm.defer(resid, delta, ctx)
             kwargs = {}
             if following is not None and consumer.takes_sink:

@@ -80,15 +80,15 @@ class Linear(Part):
                 x, row_scale = scaled            # the norm becomes a scale of the product's rows
             else:
                 x = x.tensor()
-        if sink is not None and fused and self.bias is None and not self.out_float32 \
-                and getattr(sink.norm, "weight", None) is not None and hasattr(sink.norm, "eps"):
+        following = sink.norm.row_scale_form() if sink is not None and fused and self.bias is None and not self.out_float32 else None
+        if following is not None:
             # The product may leave its result as partial sums, which the kernel of the sum and the norm adds up on
             # its way: that is the way of 17 rows and more, and of fewer where it has been measured to be faster.
             partial_sums = getattr(ops, "linear_partial_sums", None)
             split_few_rows = partial_sums is not None and row_scale is None and getattr(ops, "partial_sums_are_faster", None) is not None \
                 and ops.partial_sums_are_faster(x, self.weight)
             if not split_few_rows:
-                done = ops.linear_into_stream(x, self.weight, sink.stream(), sink.norm.weight, row_scale=row_scale)
+                done = ops.linear_into_stream(x, self.weight, sink.stream(), following[0], row_scale=row_scale)
                 if done is not None:
                     return StreamUpdate(sink.norm, *done)
             sums = None

@@ -6,27 +6,48 @@ the activation kernel.
 """
 from __future__ import annotations
 
+import dataclasses
+from typing import Tuple
+
 from .base import FeedForward, PendingNorm
 from .linear import Linear
+
+
+@dataclasses.dataclass(frozen=True)
+class GatedMLPNames:
+    """Checkpoint names of the layer's tensors.  ``gate_up``: the gate and the up projection, or one tensor that holds
+    the gate's rows followed by the up projection's."""
+    gate_up: Tuple[str, ...] = ("gate_proj", "up_proj")
+    down: str = "down_proj"
 
 
 class GatedMLP(FeedForward):
     accepts_pending_norm = True
     takes_sink = True
 
-    def __init__(self, width: int, intermediate: int, activation: str = "silu", bias: bool = False):
+    def __init__(self, width: int, intermediate: int, activation: str = "silu", bias: bool = False,
+                 names: GatedMLPNames = GatedMLPNames()):
         if activation not in ("silu", "swish"):
             raise ValueError(f"Unsupported activation {activation!r}; supported: ['silu', 'swish']")
         self.width = width
         self.intermediate = intermediate
-        self.gate_up = Linear(width, ("gate_proj", "up_proj"), (intermediate, intermediate), bias)
-        self.down = Linear(intermediate, ("down_proj",), (width,), bias)
+        if len(names.gate_up) not in (1, 2):
+            raise ValueError(f"gate and up projection come in one or two checkpoint tensors, not {len(names.gate_up)}")
+        self.names = names
+        self.gate_up = Linear(width, names.gate_up, (intermediate, intermediate) if len(names.gate_up) == 2 else (2 * intermediate,), bias)
+        self.down = Linear(intermediate, (names.down,), (width,), bias)
 
     def param_specs(self):
         return {**self.gate_up.param_specs(), **self.down.param_specs()}
 
     def assign(self, name, tensor):
-        (self.down if name.startswith("down_proj.") else self.gate_up).assign(name, tensor)
+        owner = name.rsplit(".", 1)[0]
+        if owner == self.names.down:
+            self.down.assign(name, tensor)
+        elif owner in self.names.gate_up:
+            self.gate_up.assign(name, tensor)
+        else:
+            raise KeyError(name)
 
     def finalize(self):
         self.gate_up.finalize()

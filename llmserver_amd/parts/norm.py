@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import VECTOR, Norm, ParamSpec, PendingNorm
+from .base import VECTOR, Norm, ParamSpec
 
 
 class RMSNorm(Norm):
@@ -31,6 +31,5 @@ class RMSNorm(Norm):
         ctx.ops.add_rmsnorm(resid, delta, self.weight, self.eps, out, rows)
         return out
 
-    def defer(self, resid, delta, ctx) -> PendingNorm:
-        """The same normalisation, left to whoever consumes it (a projection may fuse it)."""
-        return PendingNorm(self, resid, delta, ctx)
+    def row_scale_form(self):
+        return self.weight, self.eps

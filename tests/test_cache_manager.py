@@ -4,7 +4,7 @@ import random
 
 import pytest
 
-from llmserver_amd.cache import CacheExhaustedError, CacheManager, CacheStateError, PagePool
+from llmserver_amd.cache import CacheExhaustedError, CacheManager, CacheStateError, PagePool, PageState
 from llmserver_amd.parts import PagedKVSpec, StateSpec
 
 FULL = PagedKVSpec(2, 16)
@@ -36,38 +36,59 @@ def test_pool_rejects_bad_ids_and_double_frees():
     with pytest.raises(CacheStateError):
         pool.release(page)               # freed twice
     with pytest.raises(CacheStateError):
-        pool.retain(page)
+        pool.hold(page)
     with pytest.raises(ValueError):
         PagePool(0, 2)
 
 
-def test_release_table_validates_before_it_frees_anything():
+def test_release_all_validates_before_it_frees_anything():
     pool = PagePool(4, 2)
     table = [pool.allocate(), pool.allocate()]
     with pytest.raises(ValueError):
-        pool.release_table(table + [table[0]])
+        pool.release_all(table + [table[0]])
+    with pytest.raises(CacheStateError):
+        pool.release_all(table + [3])          # page 3 was never handed out
     assert pool.num_free == 2
-    pool.release_table(table)
+    table.insert(1, -1)                        # an entry a window has passed was given back earlier
+    pool.release_all(table)
     assert table == [] and pool.num_free == 4
+    pool.check_invariants()
+
+
+def test_every_page_is_in_one_state():
+    pool = PagePool(3, 2)
+    a, b = pool.allocate(), pool.allocate()
+    pool.publish(a, "ha")
+    pool.release(a)
+    assert [pool.state[p] for p in range(3)] == [PageState.IDLE, PageState.HELD, PageState.FREE]
+    pool.hold(a)                               # an idle page can be taken up again: its tokens are still there
+    pool.hold(a)
+    assert pool.state[a] == PageState.HELD and pool.holders[a] == 2 and pool.num_idle == 0
+    pool.release(a)
+    pool.release(a)
+    pool.publish(b, "ha")                      # a second page with the same tokens: the first stays the one to adopt
+    pool.release(b)
+    assert pool.state[b] == PageState.FREE and pool.lookup("ha") == a
+    pool.check_invariants()
 
 
 def test_registered_pages_idle_then_are_evicted_oldest_first():
     pool = PagePool(3, 2)
     a, b, c = pool.allocate(), pool.allocate(), pool.allocate()
-    pool.register(a, "ha")
-    pool.register(b, "hb")
+    pool.publish(a, "ha")
+    pool.publish(b, "hb")
     pool.release(b)
     pool.release(a)
     pool.release(c)
     assert (pool.num_free, pool.num_idle, pool.num_available) == (1, 2, 3)
     table = []
-    assert pool.share("ha", table) == a and pool.references[a] == 1 and pool.num_idle == 1
+    assert pool.adopt("ha", table) == a and pool.holders[a] == 1 and pool.num_idle == 1
     assert pool.allocate() == c
-    assert pool.allocate() == b and pool.find("hb") is None      # b was the oldest idle page: evicted, digest forgotten
+    assert pool.allocate() == b and pool.lookup("hb") is None    # b was the oldest idle page: recycled, digest forgotten
     with pytest.raises(CacheExhaustedError):
         pool.allocate()
     with pytest.raises(ValueError):
-        pool.share("ha", table)          # same page twice in one table
+        pool.adopt("ha", table)          # same page twice in one table
     pool.check_invariants()
 
 
@@ -111,15 +132,42 @@ def test_ensure_is_all_or_nothing():
 def test_state_slots_are_acquired_zeroed_and_released():
     m = manager({0: FULL, 1: StateSpec((3,))}, slots=2)
     a, b = m.open("a"), m.open("b")
-    assert {a.state_slot, b.state_slot} == {0, 1}
+    assert {a.state_slot, b.state_slot} == {0, 1} and m.state_slots_free() == 0
     with pytest.raises(CacheExhaustedError):
         m.open("c")
+    assert not m.has("c")
     freed = a.state_slot
     m.close("a")
     assert m.open("c").state_slot == freed
     m.check_invariants()
+
+
+def test_a_record_can_wait_without_a_slot_and_take_one_when_it_computes():
+    m = manager({0: FULL, 1: StateSpec((3,))}, slots=1)
+    waiting = [m.open(name, state=False) for name in ("a", "b", "c")]        # more records than slots: nobody computes yet
+    assert [r.state_slot for r in waiting] == [-1, -1, -1] and m.state_slots_free() == 1
+    assert not m.holds_anything("a")
+    assert m.acquire_state("a") == 0 and m.acquire_state("a") == 0            # asked twice, one slot
+    assert m.holds_anything("a") and m.state_slots_free() == 0
+    with pytest.raises(CacheExhaustedError):
+        m.acquire_state("b")
+    m.close("a")
+    assert m.acquire_state("b") == 0
+    m.check_invariants()
+    assert manager({0: FULL}).state_slots_free() is None                      # no mixer keeps state: nothing to run out of
+
+
+def test_what_a_plan_would_cost_is_answered_per_group():
+    m = manager({0: FULL, 1: WINDOW}, page_size=4, pages=[8, 3])
+    assert m.pages_needed("nobody", 9) == [3, 3] and m.token_room("nobody", [2, 1]) == 4
+    m.open("a")
+    m.ensure("a", 6)
+    assert m.pages_needed("a", 6) == [0, 0] and m.pages_needed("a", 13) == [2, 2]
+    assert m.available_pages() == [6, 1]
+    assert m.token_room("a", [6, 1]) == 12 and m.token_room("a", [0, 0]) == 8    # the scarcer group bounds it
+    assert m.holds_anything("a") and not m.holds_anything("nobody")
     with pytest.raises(CacheStateError):
-        m.open("c")
+        m.open("a")                      # a request has one record
     with pytest.raises(KeyError):
         m.close("nobody")
 
@@ -130,7 +178,7 @@ def test_prefix_pages_are_shared_leaving_one_token_to_compute():
     m.open("a")
     m.ensure("a", 10)
     m.register_prefix("a", prompt, 0, 10)
-    assert len(m.groups[0].pool.cacheable) == 2                     # 10 tokens: two complete pages
+    assert len(m.groups[0].pool.published_pages()) == 2                     # 10 tokens: two complete pages
     for length, shared in ((4, 0), (8, 1), (10, 2)):
         rid = f"r{length}"
         m.open(rid)

@@ -1,6 +1,6 @@
 """The scheduler's decisions and the engine's loop on the host (CPU).  The model's forward is
 replaced by a script that returns one-hot logits, the reference's own way of testing its engine
-(/root/reference/tests/test_engine.py:11-55); cache, step builder and sampler are the real ones
+(tests/test_engine.py:11-55 there); cache, step builder and sampler are the real ones
 (with the torch twins of the kernels).  Decision vectors marked "reference" are the outcomes the
 reference's tests hold for the same situations."""
 import asyncio
@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from llmserver_amd.cache import CacheExhaustedError
-from llmserver_amd.engine import (STREAM_END, Engine, Request, RequestFinishReason, RequestStateError, RequestStatus,
+from llmserver_amd.engine import (STREAM_END, Engine, EngineConfig, Request, RequestFinishReason, RequestStateError, RequestStatus,
                                   Scheduler, load_model)
 from helpers import model_folder
 from torch_ops import TorchOps
@@ -19,54 +19,103 @@ def request(name, prompt=None):
     return Request(name, "Hello", prompt or [9707], 20)
 
 
-def decoding(name, prompt=None):
+def decoding(name, prompt=None, generated=7):
+    """A request that has been through its prompt and holds its first generated token."""
     r = request(name, prompt)
-    r.start_prefill()
-    r.advance_prefill(len(r.prompt_token_ids))
-    r.complete_prefill()
+    r.admit()
+    assert r.computed(len(r.prompt_token_ids))
+    r.accept(generated)
     return r
+
+
+class Pages:
+    """What the scheduler asks of a cache manager, for one group of pages of ``page`` tokens: ``free`` pages are
+    available, ``held`` says how many pages a request has already."""
+
+    def __init__(self, free, page, held=None, slots=None):
+        self.free, self.page, self.held, self.slots = free, page, dict(held or {}), slots
+
+    def available_pages(self):
+        return [self.free]
+
+    def pages_needed(self, request_id, num_tokens):
+        return [max(0, -(-num_tokens // self.page) - self.held.get(request_id, 0))]
+
+    def token_room(self, request_id, spare):
+        return (self.held.get(request_id, 0) + max(0, spare[0])) * self.page
+
+    def state_slots_free(self):
+        return self.slots
 
 
 # ---------------------------------------------------------------- request state machine
 def test_request_walks_through_its_states():
     r = request("a", [1, 2, 3])
     with pytest.raises(RequestStateError):
-        r.advance_prefill(1)
-    r.start_prefill()
+        r.computed(1)                       # it has not been admitted
+    r.admit()
+    with pytest.raises(RequestStateError):
+        r.admit()
     with pytest.raises(ValueError):
-        r.advance_prefill(4)
-    r.advance_prefill(2)
+        r.computed(4)
+    assert r.next_tokens(2) == [1, 2] and not r.computed(2)
+    assert (r.status, r.tokens_ahead) == (RequestStatus.PREFILL, 1)
     with pytest.raises(RequestStateError):
-        r.complete_prefill()
-    r.advance_prefill(1)
-    r.complete_prefill()
-    r.append_generated_token(7)
-    r.complete_decode()
-    assert (r.status, r.num_computed_tokens) == (RequestStatus.DECODING, 4)
+        r.accept(7)                         # the end of the sequence has not been reached: there are no logits to sample
+    assert r.computed(1) and r.status == RequestStatus.DECODING
+    r.accept(7)
+    assert r.next_tokens(1) == [7] and r.computed(1)
+    assert (r.status, r.num_computed_tokens, r.sequence_length) == (RequestStatus.DECODING, 4, 4)
     r.finish("length")
-    assert r.finish_reason == RequestFinishReason.LENGTH
+    assert r.finish_reason == RequestFinishReason.LENGTH and not r.is_alive
+    for event in (lambda: r.finish("eos"), r.cancel, r.preempt, r.admit):
+        with pytest.raises(RequestStateError):
+            event()
+
+
+def test_a_preempted_request_is_computed_again_over_all_it_has_and_emits_nothing_twice():
+    r = decoding("a", [20], generated=60)
+    r.computed(1)
+    r.accept(51)
+    r.preempt()
+    assert (r.status, r.num_computed_tokens, r.preemption_count, r.tokens_ahead) == (RequestStatus.WAITING, 0, 1, 3)
+    r.admit()
+    assert r.next_tokens(2) == [20, 60] and not r.computed(2)     # the reference's re-prefill: tests/test_engine.py:507
+    assert r.next_tokens(1) == [51] and r.computed(1)             # ... and its decode step, which gives the next token
+    assert r.status == RequestStatus.DECODING and r.generated_token_ids == [60, 51]
+    r.preempt()
+    r.admit()
+    assert r.next_tokens(3) == [20, 60, 51] and r.computed(3)     # or all of it in one portion
+    r.accept(52)
+    assert r.generated_token_ids == [60, 51, 52]
+
+
+def test_cached_tokens_move_the_mark_of_a_waiting_request_only():
+    r = request("a", [1, 2, 3, 4, 5])
+    with pytest.raises(ValueError):
+        r.reuse(5)                          # one token at least must be computed
+    r.reuse(4)
+    assert r.tokens_ahead == 1 and r.next_tokens(1) == [5]
+    r.forget_reused()
+    assert r.tokens_ahead == 5
+    r.admit()
     with pytest.raises(RequestStateError):
-        r.finish("eos")
-
-
-def test_preempted_decoder_prefills_prompt_plus_all_but_the_last_generated_token():
-    r = decoding("a", [20])
-    r.append_generated_token(60)
-    r.append_generated_token(51)
-    r.preempt_for_compute()
-    assert (r.status, r.num_computed_tokens, r.preemption_count, r.needs_decode_resume) == (RequestStatus.WAITING, 0, 1, True)
-    assert r.prefill_token_ids == [20, 60]                        # reference: tests/test_engine.py:507
-    r.start_prefill()
-    r.advance_prefill(2)
-    r.complete_prefill()
-    assert not r.needs_decode_resume and r.generated_token_ids == [60, 51]
+        r.reuse(2)
 
 
 # ---------------------------------------------------------------- scheduler decisions
-def plan_commit(scheduler, free=100, page=2):
-    out = scheduler.plan(free, page)
-    scheduler.commit(out)
-    return out
+def plan_commit(scheduler, free=100, page=2, held=None):
+    plan = scheduler.plan(Pages(free, page, held))
+    scheduler.commit(plan)
+    return plan
+
+
+def counts(plan):
+    return [count for _, count in plan.portions]
+
+
+def who(plan):
+    return [r for r, _ in plan.portions]
 
 
 def test_budget_is_shared_by_decodes_and_portions():
@@ -74,9 +123,9 @@ def test_budget_is_shared_by_decodes_and_portions():
     d, first, second = decoding("d"), request("first", [10, 11, 12]), request("second", [20, 21])
     s.running.append(d)
     s.waiting.extend([first, second])
-    out = plan_commit(s)
-    assert out.decode_requests == [d] and out.prefill_requests == [first, second]
-    assert out.prefill_token_counts == [3, 1] and out.num_scheduled_tokens == 5          # reference [3, 1]
+    plan = plan_commit(s)
+    assert plan.decodes == [d] and who(plan) == [first, second]
+    assert counts(plan) == [3, 1] and plan.tokens == 5                                      # reference [3, 1]
     assert s.running == [d, first, second] and not s.waiting
 
 
@@ -84,35 +133,35 @@ def test_prompt_longer_than_the_budget_is_cut_and_computed_tokens_are_not_counte
     s = Scheduler(max_batch_size=1, max_num_batched_tokens=3)
     r = request("long", [10, 11, 12, 13])
     s.waiting.append(r)
-    assert plan_commit(s).prefill_token_counts == [3]
-    r.advance_prefill(3)
-    assert plan_commit(s).prefill_token_counts == [1]                                      # reference [3] then [1]
+    assert counts(plan_commit(s)) == [3]
+    r.computed(3)
+    assert counts(plan_commit(s)) == [1]                                                    # reference [3] then [1]
     s = Scheduler(max_batch_size=2, max_num_batched_tokens=4)
     partial = request("partial", [10, 11, 12, 13, 14])
-    partial.num_computed_tokens = 2                                                        # a cached prefix
+    partial.reuse(2)                                                                        # a cached prefix
     s.running.append(decoding("d"))
     s.waiting.append(partial)
-    assert plan_commit(s).prefill_token_counts == [3]
+    assert counts(plan_commit(s, held={"partial": 1})) == [3]
 
 
 def test_chunk_size_caps_each_portion_and_running_prefills_keep_their_slot():
     s = Scheduler(max_batch_size=2, max_num_batched_tokens=4, prefill_chunk_size=2)
     a, b = request("a", [1, 2, 3, 4, 5]), request("b", [6, 7, 8, 9, 10])
     s.waiting.extend([a, b])
-    assert plan_commit(s).prefill_token_counts == [2, 2]
-    a.advance_prefill(2)
-    b.advance_prefill(2)
-    out = plan_commit(s)
-    assert out.prefill_requests == [a, b] and out.prefill_token_counts == [2, 2] and s.running == [a, b]
+    assert counts(plan_commit(s)) == [2, 2]
+    a.computed(2)
+    b.computed(2)
+    plan = plan_commit(s)
+    assert who(plan) == [a, b] and counts(plan) == [2, 2] and s.running == [a, b]
 
 
 def test_plan_changes_nothing_and_waiting_steps_count_committed_steps():
     s = Scheduler(max_batch_size=1, max_num_batched_tokens=1)
     rs = [request(f"r{i}") for i in range(3)]
     s.waiting.extend(rs)
-    out = s.plan(10, 2)
+    plan = s.plan(Pages(10, 2))
     assert list(s.waiting) == rs and not s.running and [r.waiting_steps for r in rs] == [0, 0, 0]
-    s.commit(out)
+    assert s.commit(plan) == [rs[0]]
     assert [r.waiting_steps for r in rs] == [0, 1, 1]
     plan_commit(s, 10)
     s.running.remove(rs[0])
@@ -123,26 +172,53 @@ def test_plan_changes_nothing_and_waiting_steps_count_committed_steps():
 def test_admission_keeps_one_spare_page_per_running_request():
     for free, admitted in ((2, 0), (3, 1)):                                               # reference: headroom cases
         s = Scheduler(max_batch_size=2, max_num_batched_tokens=2)
-        d = decoding("d", [10, 11])
-        d.block_table = [0]
+        d = decoding("d", [10, 11])                                                       # two tokens in one page; the third needs another
         w = request("w", [20])
         s.running.append(d)
         s.waiting.append(w)
-        out = s.plan(free, 2)
-        assert out.decode_requests == [d] and out.num_admitted_requests == admitted
+        plan = s.plan(Pages(free, 2, held={"d": 1}))
+        assert plan.decodes == [d] and plan.admitted == admitted and plan.fits
     s = Scheduler(max_batch_size=1, max_num_batched_tokens=5)
     s.waiting.append(request("long", [1, 2, 3, 4, 5]))
-    assert s.plan(1, 2).prefill_token_counts == [2]                                        # shrunk to the free page
+    assert counts(s.plan(Pages(1, 2))) == [2]                                             # shrunk to the free page
+
+
+def test_a_plan_that_overdraws_the_pages_says_by_how_much():
+    s = Scheduler(max_batch_size=2, max_num_batched_tokens=4)
+    a, b = decoding("a", [1, 2]), decoding("b", [3, 4])
+    s.running.extend([a, b])
+    s.waiting.append(request("w"))
+    plan = s.plan(Pages(1, 2, held={"a": 1, "b": 1}))          # both need a second page, one is free
+    assert plan.short == [1] and not plan.fits and plan.admitted == 0 and plan.decodes == [a, b]
+    assert s.plan(Pages(2, 2, held={"a": 1, "b": 1})).fits
+
+
+def test_state_slots_are_places_too():
+    s = Scheduler(max_batch_size=4, max_num_batched_tokens=8)
+    s.waiting.extend(request(f"r{i}") for i in range(3))
+    assert s.plan(Pages(100, 2, slots=2)).admitted == 2 and s.plan(Pages(100, 2, slots=None)).admitted == 3
+
+
+def test_a_preempted_request_comes_back_only_when_all_of_it_fits():
+    s = Scheduler(max_batch_size=2, max_num_batched_tokens=8, prefill_chunk_size=2)
+    back = request("back", [1, 2, 3, 4, 5, 6])
+    back.preemption_count = 1
+    s.running.append(decoding("d", [9]))
+    s.waiting.append(back)
+    assert s.plan(Pages(3, 2, held={"d": 1})).admitted == 0          # 3 free, one kept for d: two pages hold four of its six tokens
+    assert s.plan(Pages(4, 2, held={"d": 1})).admitted == 1
+    back.preemption_count = 0
+    assert counts(s.plan(Pages(3, 2, held={"d": 1}))) == [2]          # a new request starts on whatever portion fits
 
 
 def test_nothing_fits_raises_and_bad_limits_are_refused():
     s = Scheduler(max_batch_size=1, max_num_batched_tokens=1)
     s.waiting.append(request("w"))
     with pytest.raises(CacheExhaustedError):
-        s.plan(0, 2)
-    assert s.plan(1, 2).num_admitted_requests == 1
-    empty = Scheduler(max_batch_size=1, max_num_batched_tokens=1).plan(1, 2)
-    assert empty.num_scheduled_tokens == 0
+        s.plan(Pages(0, 2))
+    assert s.plan(Pages(1, 2)).admitted == 1
+    empty = Scheduler(max_batch_size=1, max_num_batched_tokens=1).plan(Pages(1, 2))
+    assert empty.tokens == 0 and not empty.requests
     for args in ((0, 2), (2, 0), (3, 2)):
         with pytest.raises(ValueError):
             Scheduler(*args)
@@ -188,9 +264,9 @@ def test_recompute_preemption_resumes_without_duplicate_output():
     assert second.output_queue.drain() == [60, 51]
     assert engine.step()                                # the later request is the victim; the first decodes and finishes
     assert first.status == RequestStatus.FINISHED and first.generated_token_ids == [50, 51, 51]
-    assert second.status == RequestStatus.WAITING and second.prefill_token_ids == [20, 60] and second.block_table == []
-    assert engine.step()                                # re-prefill of prompt + generated[:-1]; its last row is not sampled
-    assert second.status == RequestStatus.DECODING and second.num_computed_tokens == 2
+    assert second.status == RequestStatus.WAITING and second.tokens_ahead == 3 and not engine.kv_cache.has(second.request_id)
+    assert engine.step()                                # computed again: the budget of two tokens takes [20, 60], nothing to sample yet
+    assert second.status == RequestStatus.PREFILL and second.num_computed_tokens == 2
     assert second.generated_token_ids == [60, 51] and second.output_queue.empty()
     assert script.calls[3]["tokens"] == [[20, 60]] and script.calls[3]["n_out"] == 0
     assert not engine.step()
@@ -212,8 +288,8 @@ def test_victim_is_least_preempted_then_least_waited_then_latest_admitted(first,
     for r, (count, steps) in zip(requests, (first, second)):
         r.preemption_count, r.waiting_steps = count, steps
     out = engine.schedule_step()
-    assert out.decode_requests == [requests[1 - victim]] and list(engine.scheduler.waiting) == [requests[victim]]
-    assert requests[victim].preemption_count == (first, second)[victim][0] + 1 and requests[victim].block_table == []
+    assert out.decodes == [requests[1 - victim]] and list(engine.scheduler.waiting) == [requests[victim]]
+    assert requests[victim].preemption_count == (first, second)[victim][0] + 1 and not engine.kv_cache.has(requests[victim].request_id)
 
 
 def test_a_single_request_that_cannot_grow_raises():
@@ -232,7 +308,7 @@ def test_only_complete_pages_of_prompt_tokens_become_shareable(length, complete)
     engine, _ = scripted_engine([[50]], max_batch_size=1, max_num_batched_tokens=8, kv_cache_num_blocks=4, kv_cache_block_size=4)
     r = engine.add_request(None, list(range(10, 10 + length)))
     engine.step()
-    assert engine.kv_cache.groups[0].pool.cacheable == set(r.block_table[:complete])
+    assert engine.kv_cache.groups[0].pool.published_pages() == set(engine.kv_cache.record(r.request_id).tables[0][:complete])
 
 
 @pytest.mark.parametrize("length, shared", [(4, 0), (8, 1), (10, 2)])
@@ -243,9 +319,11 @@ def test_second_request_reuses_the_longest_cached_prefix(length, shared):
     first = engine.add_request(None, prompt)
     engine.step()
     second = engine.add_request(None, prompt)
-    assert second.block_table == first.block_table[:shared] and second.num_computed_tokens == shared * 4
-    assert all(engine.kv_cache.groups[0].pool.references[p] == 2 for p in second.block_table)
+    assert not engine.kv_cache.has(second.request_id)       # a request that waits holds nothing; it looks when it is admitted
     engine.step()                       # one mixed step: the first request's decode token beside the second's portion
+    tables = [engine.kv_cache.record(r.request_id).tables[0] for r in (first, second)]
+    assert tables[1][:shared] == tables[0][:shared] and not set(tables[1][shared:]) & set(tables[0])
+    assert all(engine.kv_cache.groups[0].pool.holders[p] == 2 for p in tables[1][:shared])
     call = script.calls[-1]
     assert call["requests"] == [first.request_id, second.request_id]
     index = call["requests"].index(second.request_id)
@@ -331,7 +409,7 @@ def test_requests_that_arrive_together_share_what_the_first_of_them_computed():
     call = script.calls[1]
     assert call["requests"] == [first.request_id, second.request_id]
     assert call["tokens"][1] == prompt[8:] and call["start"][1] == 8
-    assert second.block_table[:2] == first.block_table[:2]
+    assert engine.kv_cache.record(second.request_id).tables[0][:2] == engine.kv_cache.record(first.request_id).tables[0][:2]
     assert engine.step_profile["prefix_hit_tokens"] == 8
     engine.kv_cache.check_invariants()
 
@@ -358,10 +436,11 @@ def test_so_few_pages_that_requests_take_turns_still_ends(seed):
     assert min(engine.kv_cache.available_pages()) == pages and not engine.kv_cache.requests
 
 
-def test_waiting_requests_give_their_cached_prefix_back_when_pages_run_short():
+def test_waiting_requests_hold_no_pages_so_cached_prefixes_never_starve_a_running_request():
     """One place, five pages.  A finished request leaves two cached pages; a waiting request with the same prefix
-    holds them (so they cannot be evicted) while the running request grows to need all five pages: the waiting one
-    gives them back instead of the engine giving up, and computes its prompt itself when its turn comes."""
+    would like them, while the running request grows to need all five pages.  A request that waits holds nothing (it
+    looks its prefix up when a place is free), so the cached pages are recycled for the running request instead of
+    the engine giving up, and the waiting one computes its prompt itself when its turn comes."""
     engine, script = scripted_engine([], max_new_tokens=6, max_batch_size=1, max_num_batched_tokens=8, kv_cache_num_blocks=5,
                                      kv_cache_block_size=2)
     first = engine.add_request(None, [7, 8, 9, 10, 11], max_new_tokens=1)
@@ -369,13 +448,36 @@ def test_waiting_requests_give_their_cached_prefix_back_when_pages_run_short():
     assert engine.kv_cache.groups[0].pool.num_idle == 2
     running = engine.add_request(None, [20, 21, 22, 23, 24])
     waiting = engine.add_request(None, [7, 8, 9, 10, 12])
-    assert len(waiting.block_table) == 2 and waiting.num_computed_tokens == 4 and engine.step_profile["prefix_hit_tokens"] == 4
-    while running.status != RequestStatus.FINISHED:        # ten tokens in the cache: five pages, two are the waiting request's
+    while running.status != RequestStatus.FINISHED:        # ten tokens in the cache: five pages, two of them were the cached ones
         assert engine.step()
         engine.kv_cache.check_invariants()
+        assert waiting.status != RequestStatus.WAITING or not engine.kv_cache.has(waiting.request_id)
     assert running.generated_token_ids == [0] * 6 and engine.step_profile["preemptions"] == 0
-    assert waiting.block_table == [] or waiting.status != RequestStatus.WAITING
     while engine.step():
         pass
     assert waiting.status == RequestStatus.FINISHED and len(waiting.generated_token_ids) == 6
+    assert engine.step_profile["prefix_hit_tokens"] == 0
     assert min(engine.kv_cache.available_pages()) == 5 and not engine.kv_cache.requests
+
+
+def test_an_offered_prefix_is_given_back_if_the_request_is_not_admitted_after_all():
+    """Two places; the budget of a step is used up by the first waiting request, so the second, which was offered the
+    cached pages of its prefix, is not admitted: it gives them back and holds nothing over the step."""
+    engine, script = scripted_engine([], max_new_tokens=2, max_batch_size=2, max_num_batched_tokens=4, kv_cache_num_blocks=8,
+                                     kv_cache_block_size=2)
+    seed = engine.add_request(None, [7, 8, 9, 10, 11], max_new_tokens=1)
+    while engine.step():
+        pass
+    assert seed.status == RequestStatus.FINISHED and engine.kv_cache.groups[0].pool.num_idle == 2
+    long, follower = engine.add_request(None, [30, 31, 32, 33, 34, 35]), engine.add_request(None, [7, 8, 9, 10, 12])
+    engine.step()                                           # four tokens of `long`; nothing is left for `follower`
+    assert follower.status == RequestStatus.WAITING and follower.num_computed_tokens == 0
+    assert not engine.kv_cache.has(follower.request_id) and engine.kv_cache.groups[0].pool.num_idle == 2
+    engine.step()                                           # two tokens of `long`, and `follower` joins behind its cached prefix
+    assert script.calls[-1]["requests"] == [long.request_id, follower.request_id]
+    assert script.calls[-1]["tokens"][1] == [12] and script.calls[-1]["start"][1] == 4
+    assert engine.step_profile["prefix_hit_tokens"] == 4
+    while engine.step():
+        pass
+    engine.kv_cache.check_invariants()
+    assert not engine.kv_cache.requests

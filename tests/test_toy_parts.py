@@ -19,8 +19,8 @@ from llmserver_amd.cache import CacheManager
 from llmserver_amd.config import ModelConfig, field, register_architecture
 from llmserver_amd.engine import ModelRunner, StepEntry, load_model
 from llmserver_amd.models.decoder import DecoderModel, LayerCall
-from llmserver_amd.parts import (MATRIX, FeedForward, GatedMLP, GQAttention, Linear, Mixer, NoPosition, ParamSpec, PositionEncoding,
-                                 PreNormBlock, RMSNorm, RotaryPosition, StateSpec, TokenEmbedding)
+from llmserver_amd.parts import (MATRIX, AttentionNames, FeedForward, GatedMLP, GatedMLPNames, GQAttention, Linear, Mixer, NoPosition,
+                                 ParamSpec, PositionEncoding, PreNormBlock, RMSNorm, RotaryPosition, StateSpec, TokenEmbedding)
 from llmserver_amd.weights import RandomInit, write_random_model
 from torch_ops import TorchOps
 
@@ -128,6 +128,7 @@ class ToyConfig(ModelConfig):
     layer_order: object = field("layer_order", object)       # per call: [block, cache, writes]
     ffn_experts: object = field("ffn_experts", object, None)        # per block: 0 = dense, n = top-one of n experts
     position_kinds: object = field("position_kinds", object, None)  # per block: "rope", "harmonic" or "none"
+    fused_names: bool = field("fused_names", bool, False)           # a checkpoint that stores q, k, v in one tensor, and other names
     tie_word_embeddings: bool = field("tie_word_embeddings", bool, False)
 
     @property
@@ -135,7 +136,15 @@ class ToyConfig(ModelConfig):
         return len(self.layer_kinds)
 
 
+FUSED_ATTENTION = AttentionNames(qkv=("wqkv",), out="wo", q_norm="qn", k_norm="kn")
+FUSED_MLP = GatedMLPNames(gate_up=("w13",), down="w2")
+FUSED_BLOCK = ("attention_norm", "attention", "ffn_norm", "feed_forward")
+FUSED_MODEL = ("tok_embeddings", "layers", "norm")
+
+
 def build_toy(config: ToyConfig) -> DecoderModel:
+    fused = config.fused_names
+    attention_names, mlp_names = (FUSED_ATTENTION, FUSED_MLP) if fused else (AttentionNames(), GatedMLPNames())
     positions = {"rope": RotaryPosition(config.head_dim, config.rope_theta), "harmonic": HarmonicPosition(config.head_dim),
                  "none": NoPosition()}
     blocks = []
@@ -145,15 +154,18 @@ def build_toy(config: ToyConfig) -> DecoderModel:
         else:
             position = positions[config.position_kinds[index] if config.position_kinds else "rope"]
             mixer = GQAttention(config.hidden_size, config.num_attention_heads, config.num_key_value_heads, config.head_dim,
-                                position, qk_norm_eps=config.rms_norm_eps, window=kind or None)
+                                position, qk_norm_eps=config.rms_norm_eps, window=kind or None, names=attention_names)
         n_experts = config.ffn_experts[index] if config.ffn_experts else 0
-        ffn = TopOneExperts(config.hidden_size, config.intermediate_size, n_experts) if n_experts else GatedMLP(config.hidden_size, config.intermediate_size)
+        ffn = TopOneExperts(config.hidden_size, config.intermediate_size, n_experts) if n_experts \
+            else GatedMLP(config.hidden_size, config.intermediate_size, names=mlp_names)
+        block_names = {"names": FUSED_BLOCK} if fused else {}
         blocks.append(PreNormBlock(RMSNorm(config.hidden_size, config.rms_norm_eps), mixer,
-                                   RMSNorm(config.hidden_size, config.rms_norm_eps), ffn))
+                                   RMSNorm(config.hidden_size, config.rms_norm_eps), ffn, **block_names))
     order = [LayerCall(b, c, bool(w)) for b, c, w in config.layer_order]
-    head = Linear(config.hidden_size, ("lm_head",), (config.vocab_size,), out_float32=True)
+    head = Linear(config.hidden_size, ("output" if fused else "lm_head",), (config.vocab_size,), out_float32=True)
+    model_names = {"names": FUSED_MODEL} if fused else {}
     return DecoderModel(config, TokenEmbedding(config.vocab_size, config.hidden_size), blocks,
-                        RMSNorm(config.hidden_size, config.rms_norm_eps), head, config.tie_word_embeddings, order)
+                        RMSNorm(config.hidden_size, config.rms_norm_eps), head, config.tie_word_embeddings, order, **model_names)
 
 
 register_architecture("toy_parts", ToyConfig, build_toy, replace=True)
@@ -171,12 +183,38 @@ TOYS = {
     "experts": dict(BASE, layer_kinds=[0, 0, 0], layer_order=[[i, i, 1] for i in range(3)], ffn_experts=[0, 3, 2]),
     # the framework's rotation, another table of frequencies, no rotation at all
     "positions": dict(BASE, layer_kinds=[0, 0, 0], layer_order=[[i, i, 1] for i in range(3)], position_kinds=["rope", "harmonic", "none"]),
+    # a checkpoint with q, k and v in one tensor, gate and up in one tensor and names of its own; a window of 13 beside all keys
+    "fused": dict(BASE, layer_kinds=[0, 13, 0], layer_order=[[i, i, 1] for i in range(3)], fused_names=True),
 }
 DISCONTINUOUS = {"experts"}       # a router's choice can flip under bfloat16 rounding: compared in float32 only
 
 
+def usual_names(raw, tensors):
+    """The tensors of a checkpoint with fused projections and names of its own, under the names the plain implementation
+    reads: the stacked matrices are cut back into their projections."""
+    if not raw.get("fused_names"):
+        return tensors
+    q_rows, kv_rows = raw["num_attention_heads"] * raw["head_dim"], raw["num_key_value_heads"] * raw["head_dim"]
+    renamed = {"model.embed_tokens.weight": tensors["tok_embeddings.weight"], "model.norm.weight": tensors["norm.weight"],
+               "lm_head.weight": tensors["output.weight"]}
+    for layer in range(len(raw["layer_kinds"])):
+        old, new = f"layers.{layer}", f"model.layers.{layer}"
+        wqkv, w13 = tensors[f"{old}.attention.wqkv.weight"], tensors[f"{old}.feed_forward.w13.weight"]
+        renamed.update({
+            f"{new}.input_layernorm.weight": tensors[f"{old}.attention_norm.weight"],
+            f"{new}.post_attention_layernorm.weight": tensors[f"{old}.ffn_norm.weight"],
+            f"{new}.self_attn.q_proj.weight": wqkv[:q_rows], f"{new}.self_attn.k_proj.weight": wqkv[q_rows:q_rows + kv_rows],
+            f"{new}.self_attn.v_proj.weight": wqkv[q_rows + kv_rows:], f"{new}.self_attn.o_proj.weight": tensors[f"{old}.attention.wo.weight"],
+            f"{new}.self_attn.q_norm.weight": tensors[f"{old}.attention.qn.weight"],
+            f"{new}.self_attn.k_norm.weight": tensors[f"{old}.attention.kn.weight"],
+            f"{new}.mlp.gate_proj.weight": w13[:raw["intermediate_size"]], f"{new}.mlp.up_proj.weight": w13[raw["intermediate_size"]:],
+            f"{new}.mlp.down_proj.weight": tensors[f"{old}.feed_forward.w2.weight"]})
+    return renamed
+
+
 def plain_toy(raw, tensors, tokens):
     """The toy models over a whole sequence, from the plain implementation's functions."""
+    tensors = usual_names(raw, tensors)
     config = dict(raw, num_hidden_layers=len(raw["layer_kinds"]))
     ids = torch.as_tensor(tokens)
     positions = torch.arange(len(tokens))
@@ -231,6 +269,9 @@ def run_toy(name, device, dtype, ops, tol):
     cache = CacheManager(model.cache_specs(), page, 36, num_state_slots=2, device=device, dtype=model.dtype)
     if name == "windows":
         assert sorted(str(g.spec.window) for g in cache.groups) == ["20", "9", "None"]
+    if name == "fused":
+        assert sorted(str(g.spec.window) for g in cache.groups) == ["13", "None"]
+        assert "layers.1.attention.wqkv.weight" in tensors and model.blocks[1].mixer.qkv.weight.shape == (8 * 16, 48)
     if name == "state":
         assert cache.state_specs and not cache.prefix_caching_possible
     runner = ModelRunner(model, cache, ops)
