@@ -197,3 +197,105 @@ def test_q_and_k_norms_act_per_head_before_rotation():
     b = plain.attention_block(x, scaled, p, config0, torch.arange(4))
     assert torch.allclose(a, b, atol=1e-9)
     assert base.shape == (4, 24)
+
+
+# ---------------------------------------------------------------- the attention block against a construction from library routines
+def library_attention_block(x, tensors, p, config, positions, weight_after_rotation=False, bias_after_norm=False, scale=None):
+    """The block rebuilt from library routines only (``F.linear``, ``F.rms_norm``, ``F.scaled_dot_product_attention``
+    with the library's own default scale) and an explicit rotation; the two switches build the plausible mistakes."""
+    n_q, n_kv, d, eps = config["num_attention_heads"], config["num_key_value_heads"], config["head_dim"], config["rms_norm_eps"]
+    seq = x.shape[0]
+    angles = positions.to(torch.float32)[:, None] * (1.0 / config["rope_theta"] ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    angles = torch.cat([angles, angles], -1).to(D64)
+
+    def rotate(t):                       # [heads, seq, d]; pairs (i, i + d/2)
+        half = d // 2
+        return t * torch.cos(angles) + torch.cat([-t[..., half:], t[..., :half]], -1) * torch.sin(angles)
+
+    def heads(name, n, norm_weight):
+        bias = tensors.get(f"{p}.{name}.bias")
+        y = F.linear(x, tensors[f"{p}.{name}.weight"], None if bias_after_norm else bias).view(seq, n, d).transpose(0, 1)
+        if norm_weight is None:
+            return y
+        if weight_after_rotation:
+            y = rotate(F.rms_norm(y, (d,), None, eps)) * norm_weight
+        else:
+            y = rotate(F.rms_norm(y, (d,), norm_weight, eps))
+        if bias_after_norm and bias is not None:
+            y = y + bias.view(n, 1, d)
+        return y
+
+    q = heads("q_proj", n_q, tensors[f"{p}.q_norm.weight"])
+    k = heads("k_proj", n_kv, tensors[f"{p}.k_norm.weight"])
+    v = heads("v_proj", n_kv, None)
+    group = n_q // n_kv
+    out = F.scaled_dot_product_attention(q[None], k.repeat_interleave(group, 0)[None], v.repeat_interleave(group, 0)[None],
+                                         is_causal=True, scale=scale)[0]
+    return F.linear(out.transpose(0, 1).reshape(seq, n_q * d), tensors[f"{p}.o_proj.weight"], tensors.get(f"{p}.o_proj.bias"))
+
+
+def lopsided_norm_tensors(bias=False):
+    """Norm weights far from one and different in the two halves of a head (a rotation mixes element i with element
+    i + d/2, so a weight applied after the rotation gives another result), and, on request, large biases."""
+    tensors = tiny_tensors(CONFIG)
+    p = "model.layers.0.self_attn"
+    tensors[f"{p}.q_norm.weight"] = torch.tensor([3.0, 0.2, 1.5, 0.1, 0.3, 2.5, 0.4, 4.0], dtype=D64)
+    tensors[f"{p}.k_norm.weight"] = torch.tensor([0.2, 2.0, 0.3, 3.0, 2.5, 0.1, 1.8, 0.5], dtype=D64)
+    if bias:
+        g = torch.Generator().manual_seed(5)
+        for name, rows in (("q_proj", 48), ("k_proj", 16), ("v_proj", 16), ("o_proj", 24)):
+            tensors[f"{p}.{name}.bias"] = torch.randn(rows, generator=g, dtype=D64)
+    return tensors, p
+
+
+def test_scores_are_scaled_by_the_library_s_default_one_over_root_d():
+    """``scale=None`` makes the library divide by sqrt(head_dim); the plain block is given no scale either."""
+    tensors, p = lopsided_norm_tensors()
+    x, positions = torch.randn(7, 24, dtype=D64), torch.arange(7)
+    got = plain.attention_block(x, tensors, p, CONFIG, positions)
+    assert torch.allclose(got, library_attention_block(x, tensors, p, CONFIG, positions), atol=1e-7)
+    for wrong in (1.0, 1.0 / 8, 8 ** -0.25):
+        assert not torch.allclose(got, library_attention_block(x, tensors, p, CONFIG, positions, scale=wrong), atol=1e-3)
+
+
+def test_q_and_k_norm_weights_are_applied_before_the_rotation():
+    tensors, p = lopsided_norm_tensors()
+    x, positions = torch.randn(7, 24, dtype=D64), torch.arange(3, 10)       # away from position 0, where nothing turns
+    got = plain.attention_block(x, tensors, p, CONFIG, positions)
+    assert torch.allclose(got, library_attention_block(x, tensors, p, CONFIG, positions), atol=1e-7)
+    after = library_attention_block(x, tensors, p, CONFIG, positions, weight_after_rotation=True)
+    assert (got - after).abs().max() > 1e-2
+
+
+def test_biases_belong_to_the_projections():
+    """q, k and v biases are added by the projection, so the per-head norm sees them; the output bias is added last."""
+    tensors, p = lopsided_norm_tensors(bias=True)
+    x, positions = torch.randn(6, 24, dtype=D64), torch.arange(6)
+    got = plain.attention_block(x, tensors, p, CONFIG, positions)
+    assert torch.allclose(got, library_attention_block(x, tensors, p, CONFIG, positions), atol=1e-7)
+    assert (got - library_attention_block(x, tensors, p, CONFIG, positions, bias_after_norm=True)).abs().max() > 1e-2
+    without = {name: tensor for name, tensor in tensors.items() if not name.endswith(".bias")}
+    silent = dict(tensors)
+    silent[f"{p}.o_proj.weight"] = torch.zeros_like(tensors[f"{p}.o_proj.weight"])
+    assert torch.allclose(plain.attention_block(x, silent, p, CONFIG, positions), tensors[f"{p}.o_proj.bias"].expand(6, 24))
+    assert (got - plain.attention_block(x, without, p, CONFIG, positions)).abs().max() > 1e-2
+
+
+ROPE_THETA_CASES = [          # (config.json keys, theta): utils/architecture.py:23-30 in the reference
+    ({"rope_theta": 5.0, "rope_parameters": {"rope_theta": 7.0}}, 5.0),          # the top-level key wins
+    ({"rope_parameters": {"rope_theta": 7.0}}, 7.0),
+    ({"rope_scaling": {"rope_theta": 9.0}, "rope_parameters": {"rope_theta": 7.0}}, 9.0),   # rope_scaling is looked at first
+    ({"rope_scaling": None, "rope_parameters": {"rope_theta": 7.0}}, 7.0),
+    ({"rope_parameters": {"rope_type": "default"}}, 10000.0),
+    ({}, 10000.0),
+]
+
+
+@pytest.mark.parametrize("keys, theta", ROPE_THETA_CASES)
+def test_where_rope_theta_is_looked_up(keys, theta):
+    """The plain implementation and the engine's typed configuration read the same places in the same order."""
+    from llmserver_amd.config import config_from_dict
+    assert plain.rope_theta_of(keys) == theta
+    raw = dict(model_type="qwen3", vocab_size=50, hidden_size=24, intermediate_size=40, num_hidden_layers=1,
+               num_attention_heads=3, num_key_value_heads=1, head_dim=16, rms_norm_eps=1e-5, **keys)
+    assert config_from_dict(raw).rope_theta == theta

@@ -16,11 +16,20 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 pytestmark = pytest.mark.gpu
 
 TOLERANCE = {"float32": dict(atol=3e-5, rtol=1e-4), "bfloat16": None}
+# bfloat16 keeps 8 bits, and a few roundings of that size meet through two or three layers: the error of a position's
+# logits is measured against those logits' own size (their largest magnitude; the tiny models' logits are a few tenths,
+# so an absolute bound would hide a wrong key or page).  The errors of a run are a smooth spread; a fault is not.
+BF16_WORST, BF16_MEDIAN = 0.03, 0.01
 
 
-def bf16_atol(expected):
-    """bfloat16 keeps 8 bits: a few roundings of that size through two or three layers."""
-    return 0.02 * max(1.0, float(np.abs(expected).max()))
+def bf16_error(got, expected):
+    return float(np.abs(got - expected).max()) / float(np.abs(expected).max())
+
+
+def check_bf16(errors, what):
+    errors = np.asarray(errors)
+    print(f"  {what}: bfloat16 error relative to the logits: median {np.median(errors):.4f} worst {errors.max():.4f}", flush=True)
+    assert np.median(errors) <= BF16_MEDIAN and errors.max() <= BF16_WORST, (what, float(np.median(errors)), float(errors.max()))
 
 
 def build_trace(case):
@@ -58,7 +67,7 @@ def run_trace(case, dtype, steps, tmp_path, max_tokens, page_size):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("case, page_size", [("A", 16), ("B", 8), ("C", 4)])
+@pytest.mark.parametrize("case, page_size", [("A", 16), ("B", 8), ("C", 4), ("D", 16)])
 def test_all_schedules_match_the_plain_implementation(case, page_size, dtype, tmp_path):
     print(f"replay case {case} {dtype} page {page_size}", flush=True)
     steps, meta = build_trace(case)
@@ -66,24 +75,29 @@ def test_all_schedules_match_the_plain_implementation(case, page_size, dtype, tm
     assert max_tokens <= 256
     results = run_trace(case, dtype, steps, tmp_path, max_tokens, page_size)
     assert len(results) == sum(n for n, _ in meta.values())
-    worst = 0.0
+    errors = []
     for (rid, position), logits in results.items():
         n, seed = meta[rid]
         expected = plain_logits(case, n, seed)[position].numpy()
         if dtype == "float32":
             np.testing.assert_allclose(logits, expected, err_msg=f"{rid} position {position}", **TOLERANCE["float32"])
         else:
-            error = float(np.abs(logits - expected).max())
-            worst = max(worst, error)
-            assert error <= bf16_atol(expected), f"{rid} position {position}: {error}"
+            errors.append(bf16_error(logits, expected))
+    if errors:
+        check_bf16(errors, f"case {case} against the plain implementation")
     # the same request cut differently agrees with itself at least as well as with the oracle
+    errors = []
     for rid in ("a", "b", "c"):
         n, _ = meta[f"w-{rid}"]
         for position in range(n):
             for other in ("t-", "p-"):
                 a, b = results[(f"w-{rid}", position)], results[(f"{other}{rid}", position)]
-                limit = 1e-4 if dtype == "float32" else bf16_atol(a)
-                assert float(np.abs(a - b).max()) <= limit, (rid, other, position)
+                if dtype == "float32":
+                    assert float(np.abs(a - b).max()) <= 1e-4, (rid, other, position)
+                else:
+                    errors.append(bf16_error(b, a))
+    if errors:
+        check_bf16(errors, f"case {case} between two cuts of the same request")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -96,12 +110,15 @@ def test_long_decoding_and_first_tokens(dtype, tmp_path):
     assert len(steps) == 301 and all(len(s["entries"][0]["tokens"]) == 1 for s in steps)
     results = run_trace(case, dtype, steps, tmp_path, 320, 8)
     expected = plain_logits(case, 301, 31).numpy()
+    errors = []
     for position in range(301):
         got = results[("long", position)]
         if dtype == "float32":
             np.testing.assert_allclose(got, expected[position], err_msg=f"position {position}", **TOLERANCE["float32"])
         else:
-            assert float(np.abs(got - expected[position]).max()) <= bf16_atol(expected[position]), position
+            errors.append(bf16_error(got, expected[position]))
+    if errors:
+        check_bf16(errors, "long decoding")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -135,7 +152,7 @@ def test_unusual_steps(dtype, tmp_path):
     assert done.returncode == 0, done.stderr[-3000:]
     assert done.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
     assert sorted(os.listdir(out)) == ["0.f32", "2.f32", "4.f32", "5.f32", "6.f32", "7.f32"]       # steps 1 and 3 want nothing
-    fed, place = {}, {}
+    fed, place, errors = {}, {}, []
     for step in steps:
         wanted = sum(len(e["want"]) for e in step["entries"])
         rows = np.fromfile(out / f"{step['step']}.f32", dtype="<f4").reshape(wanted, vocab) if wanted else None
@@ -148,9 +165,11 @@ def test_unusual_steps(dtype, tmp_path):
                 if dtype == "float32":
                     np.testing.assert_allclose(rows[row], expected, err_msg=f"step {step['step']} {entry['id']} place {want}", **TOLERANCE["float32"])
                 else:
-                    assert float(np.abs(rows[row] - expected).max()) <= bf16_atol(expected), (step["step"], entry["id"], want)
+                    errors.append(bf16_error(rows[row], expected))
                 row += 1
             place[entry["id"]] = start + len(entry["tokens"])
         for name in step["end"]:
             place.pop(name, None)
             fed.pop(name, None)
+    if errors:
+        check_bf16(errors, "unusual steps")

@@ -23,7 +23,16 @@ TINY_C = dict(model_type="qwen3", num_hidden_layers=2, hidden_size=72, num_atten
 TINY_C_INIT = RandomInit(seed=5, std=0.05, norm_noise=0.2)
 TINY_C_PAGE = 12
 
-CASES = {"A": (TINY_A, TINY_A_INIT, TINY_A_PAGE), "B": (TINY_B, TINY_B_INIT, TINY_B_PAGE), "C": (TINY_C, TINY_C_INIT, TINY_C_PAGE)}
+# A head size that is a multiple of 64: in bfloat16 steps of single tokens the attention kernel then normalises, rotates and
+# writes the new key and value itself.  One KV head for five query heads.
+TINY_D = dict(model_type="qwen3", num_hidden_layers=2, hidden_size=80, num_attention_heads=5, num_key_value_heads=1,
+              head_dim=64, intermediate_size=176, vocab_size=200, rope_theta=2e5, rms_norm_eps=2e-6,
+              attention_bias=False, tie_word_embeddings=True)
+TINY_D_INIT = RandomInit(seed=37, std=0.05, norm_noise=0.15)
+TINY_D_PAGE = 16
+
+CASES = {"A": (TINY_A, TINY_A_INIT, TINY_A_PAGE), "B": (TINY_B, TINY_B_INIT, TINY_B_PAGE), "C": (TINY_C, TINY_C_INIT, TINY_C_PAGE),
+         "D": (TINY_D, TINY_D_INIT, TINY_D_PAGE)}
 
 
 def make_config(raw) -> Qwen3Config:
