@@ -4,12 +4,16 @@
 
 Default workload: the Qwen3-8B-sized configuration (36 layers, hidden 4096, 32 query heads, 8 KV
 heads, head size 128, intermediate 12288, vocabulary 151936, untied head), bfloat16, a batch of 8
-requests decoding at a context of 4,096 tokens.  A "step" is one decode step of the whole batch:
-build the batch, run the model against the paged cache, sample greedily, return the token ids.
-Prints ONE JSON line: ``value`` is decoded tokens per second; ``prefill`` times one 2,048-token
-prompt; ``roofline`` relates the bytes a decode step has to read (every weight once, plus the
-cache of the live requests) to the published HBM bandwidth; ``points`` holds batch 1 and 64.
-Token ids are seeded uniform random numbers (synthetic data), weights seeded normal.
+requests decoding at a context of 4,096 tokens.  A "step" is one decode step of the whole batch
+through ``Engine.step()``: the scheduler plans it, the batch is laid out, the model runs against the
+paged cache, tokens are sampled greedily and every request moves on.  Prints ONE JSON line: ``value``
+is decoded tokens per second; ``prefill`` times one engine step that takes a 2,048-token prompt from
+its arrival to its first token; ``roofline`` relates the bytes a decode step has to read (every
+weight once, plus the cache of the live requests) to the published HBM bandwidth; ``points`` holds
+batch 1 and 64 of the same model (tokens per second, with the step's milliseconds and its share of
+the HBM peak beside them) and, unless ``--no-extra-points``, the two other workloads the baseline
+names: 64 mixed requests with a shared prefix on Qwen3-1.7B sizes, and batch 16 behind 8,192 tokens
+on Qwen3-32B sizes.  Token ids are seeded uniform random numbers (synthetic data), weights seeded normal.
 """
 from __future__ import annotations
 
@@ -24,21 +28,21 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
-QWEN3_8B = dict(model_type="qwen3", num_hidden_layers=36, hidden_size=4096, num_attention_heads=32,
-                num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1e6,
-                rms_norm_eps=1e-6, attention_bias=False, tie_word_embeddings=False, max_position_embeddings=40960)
-FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+MODEL = "qwen3-8b"
 
 
 def log(*args):
     print(*args, file=sys.stderr, flush=True)
 
 
-def weight_bytes(config, elem):
-    c = config
-    per_layer = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
+def layer_weights(c):
+    return c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
         + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
-    return elem * (c.num_hidden_layers * per_layer + c.vocab_size * c.hidden_size)
+
+
+def weight_bytes(config, elem):
+    """What a decode step reads of the weights: every layer's matrices and the head (the embedding table only by row)."""
+    return elem * (config.num_hidden_layers * layer_weights(config) + config.vocab_size * config.hidden_size)
 
 
 def kv_bytes_per_token(config, elem):
@@ -47,99 +51,105 @@ def kv_bytes_per_token(config, elem):
 
 def prefill_flops(config, tokens):
     c = config
-    per_layer = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
-        + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
-    gemm = 2.0 * tokens * per_layer * c.num_hidden_layers + 2.0 * c.vocab_size * c.hidden_size
+    gemm = 2.0 * tokens * layer_weights(c) * c.num_hidden_layers + 2.0 * c.vocab_size * c.hidden_size
     attention = 2.0 * c.num_attention_heads * c.head_dim * tokens * (tokens + 1) * c.num_hidden_layers
     return gemm + attention
 
 
-class DecodeBench:
-    """Holds B requests at a given context in the engine's cache and steps them."""
-
-    def __init__(self, model, page_size, batch, context, final_context, prompt_chunk=2048, seed=0):
-        import torch
-
-        from llmserver_amd.cache import CacheManager
-        from llmserver_amd.engine import ModelRunner, StepEntry
-        from llmserver_amd.sampling import Sampler
-
-        self.torch, self.StepEntry = torch, StepEntry
-        self.batch = batch
-        pages = batch * (-(-(final_context + 8) // page_size)) + 8
-        self.cache = CacheManager(model.cache_specs(), page_size, pages, device=model.device, dtype=model.dtype)
-        self.runner = ModelRunner(model, self.cache)
-        self.sampler = Sampler(self.runner.ops, model.device)
-        generator = torch.Generator().manual_seed(seed)
-        self.ids = [f"r{i}" for i in range(batch)]
-        self.last = []
-        vocab = model.config.vocab_size
-        for rid in self.ids:
-            self.cache.open(rid)
-        # Fill every request's cache up to `context` tokens with real prefill steps.
-        for rid in self.ids:
-            done = 0
-            while done < context:
-                n = min(prompt_chunk, context - done)
-                tokens = torch.randint(0, vocab, (n,), generator=generator).tolist()
-                self.runner.step([StepEntry(rid, tokens, [])])
-                done += n
-        self.last = torch.randint(0, vocab, (batch,), generator=generator).tolist()
-        torch.cuda.synchronize()
-
-    def step(self, more_follow=True):
-        entries = [self.StepEntry(rid, [token], [0]) for rid, token in zip(self.ids, self.last)]
-        logits = self.runner.step(entries)
-        sampled = self.sampler.launch(logits, [0.0] * self.batch, [0.0] * self.batch)
-        # As the engine does while it knows that all requests go on: the next step is laid out on the host while the
-        # GPU runs this one, and started with the sampled tokens still on the device.
-        if more_follow and self.runner.prepare_ahead(self.ids):
-            self.runner.launch_ahead(sampled.device)
-        self.last = sampled.tolist()
-
-    def run(self, steps, warmup):
-        """Seconds for exactly ``steps`` decode steps: the last warm-up step starts nothing that the timed steps would
-        find done, and the last timed step starts nothing that would run beyond them."""
-        torch = self.torch
-        for index in range(warmup):
-            self.step(more_follow=index + 1 < warmup)
-        torch.cuda.synchronize()
-        start = time.perf_counter()
-        for index in range(steps):
-            self.step(more_follow=index + 1 < steps)
-        torch.cuda.synchronize()
-        return time.perf_counter() - start
-
-    def close(self):
-        for rid in self.ids:
-            self.cache.close(rid)
-        del self.runner, self.cache
-        self.torch.cuda.empty_cache()
+def random_model(name, layers, dtype, seed=0):
+    from llmserver_amd.cli.benchmark import RANDOM_CONFIGS
+    from llmserver_amd.config import config_from_dict
+    from llmserver_amd.kernels import default_ops
+    from llmserver_amd.weights import RandomInit, random_model_on_device
+    raw = dict(RANDOM_CONFIGS[name], model_type="qwen3")
+    full = raw["num_hidden_layers"]
+    raw["num_hidden_layers"] = min(full, layers) if layers else full
+    config = config_from_dict(raw)
+    default_ops().preload([config.head_dim], dtype)
+    elem = 2 if str(dtype).endswith("bfloat16") else 4
+    log(f"[bench] {name}: drawing random weights, {weight_bytes(config, elem) / 1e9:.2f} GB")
+    model = random_model_on_device(config, "cuda:0", dtype, RandomInit(seed=seed, std=0.02))
+    model.name = f"{name}-random"
+    return model, config, full
 
 
-def time_prefill(model, page_size, tokens, repeats=3, seed=1):
+def decode_through_engine(model, page_size, batch, context, steps, warmup, seed=0):
+    """Seconds for exactly ``steps`` decoding steps of ``batch`` requests through ``Engine.step()``, the last of which
+    ends at a context of ``context`` tokens.  The requests' prompts are prefilled by the engine itself first."""
     import torch
 
-    from llmserver_amd.cache import CacheManager
-    from llmserver_amd.engine import ModelRunner, StepEntry
+    from llmserver_amd.engine import Engine, RequestStatus
+    prompt_tokens = context - steps - warmup
+    pages = batch * (-(-(context + 8) // page_size)) + 16
+    engine = Engine(model, None, max_new_tokens=steps + warmup + 8, max_batch_size=batch, max_num_batched_tokens=max(4096, batch * page_size),
+                    kv_cache_num_blocks=pages, kv_cache_block_size=page_size, stream_text=False, max_completed_requests=0,
+                    ignore_eos=True, enable_prefix_caching=True)
+    generator = torch.Generator().manual_seed(seed)
+    vocab = model.config.vocab_size
+    prompts = [torch.randint(0, vocab, (prompt_tokens,), generator=generator).tolist() for _ in range(batch)]
+    # Every prompt goes through the engine once on its own, which leaves its complete pages in the cache; the requests
+    # that are timed then find them, compute the last few tokens of their prompts in one common step, and decode in step.
+    for prompt in prompts:
+        engine.add_request(None, prompt_token_ids=prompt, max_new_tokens=1)
+        while engine.step():
+            pass
+    requests = [engine.add_request(None, prompt_token_ids=prompt) for prompt in prompts]
+    engine.step()
+    assert all(request.status == RequestStatus.DECODING for request in requests), "the prompts' pages were not found in the cache"
+    produced = len(requests[0].generated_token_ids)
+    assert produced == 1 and all(len(request.generated_token_ids) == produced for request in requests)
 
-    cache = CacheManager(model.cache_specs(), page_size, -(-tokens // page_size) + 4, device=model.device, dtype=model.dtype)
-    runner = ModelRunner(model, cache)
+    def run(count):
+        # The last of these steps starts nothing ahead of time: what is timed is exactly these steps' work.
+        for index in range(count):
+            engine.launch_ahead = index + 1 < count
+            engine.step()
+        torch.cuda.synchronize()
+
+    run(warmup + 1 - produced)                          # the step that finished the prompts gave the first token
+    start = time.perf_counter()
+    run(steps)
+    elapsed = time.perf_counter() - start
+    assert all(len(request.generated_token_ids) == warmup + 1 + steps for request in requests)
+    assert all(request.sequence_length == context + 1 for request in requests)       # the last step ran at `context` tokens
+    profile = dict(engine.step_profile)
+    for request in requests:
+        engine.cancel_request(request.request_id)
+    del engine
+    torch.cuda.empty_cache()
+    return elapsed, profile
+
+
+def prefill_through_engine(model, page_size, tokens, repeats=3, seed=1):
+    """Seconds of the one engine step that takes a prompt of ``tokens`` tokens to its first token (best of ``repeats``)."""
+    import torch
+
+    from llmserver_amd.engine import Engine
+    engine = Engine(model, None, max_new_tokens=1, max_batch_size=1, max_num_batched_tokens=tokens,
+                    kv_cache_num_blocks=-(-tokens // page_size) + 8, kv_cache_block_size=page_size, stream_text=False,
+                    max_completed_requests=0, ignore_eos=True, enable_prefix_caching=False)
     generator = torch.Generator().manual_seed(seed)
     best = float("inf")
     for attempt in range(repeats + 1):
-        prompt = torch.randint(0, model.config.vocab_size, (tokens,), generator=generator).tolist()
-        cache.open("p")
+        request = engine.add_request(None, prompt_token_ids=torch.randint(0, model.config.vocab_size, (tokens,), generator=generator).tolist())
         torch.cuda.synchronize()
         start = time.perf_counter()
-        logits = runner.step([StepEntry("p", prompt, [tokens - 1])])
-        int(torch.argmax(logits[0]))
+        more = engine.step()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - start
-        cache.close("p")
+        assert not more and len(request.generated_token_ids) == 1
         if attempt:
             best = min(best, elapsed)
+    del engine
+    torch.cuda.empty_cache()
     return best
+
+
+def decode_point(model, config, elem, page_size, batch, context, steps, warmup):
+    seconds, _ = decode_through_engine(model, page_size, batch, context, steps, warmup)
+    ms = 1000.0 * seconds / steps
+    step_bytes = weight_bytes(config, elem) + batch * (context - steps / 2.0) * kv_bytes_per_token(config, elem)
+    return batch * steps / seconds, ms, step_bytes / (ms * 1e-3) / 1e9
 
 
 def main() -> int:
@@ -149,79 +159,102 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
-    parser.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the configuration has, if memory or time needs it")
+    parser.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has, if memory or time needs it (0: all)")
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--page-size", type=int, default=16)
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points")
+    parser.add_argument("--no-extra-points", action="store_true", help="skip the Qwen3-1.7B-sized mixed workload and the Qwen3-32B-sized batch")
     parser.add_argument("--no-prefill", action="store_true")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
+    if args.context - args.steps - args.warmup < 1:
+        parser.error("--context must exceed --steps + --warmup")
 
     import torch
 
-    from llmserver_amd.config import config_from_dict
     from llmserver_amd.engine.loading import parse_dtype
-    from llmserver_amd.kernels import default_ops
-    from llmserver_amd.weights import RandomInit, random_model_on_device
 
-    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
-    config = config_from_dict(raw)
     dtype = parse_dtype(args.dtype)
     short = "bf16" if dtype == torch.bfloat16 else "fp32"
     elem = 2 if dtype == torch.bfloat16 else 4
-    default_ops().preload([config.head_dim], dtype)
-    log(f"[bench] drawing random weights: {weight_bytes(config, elem) / 1e9:.2f} GB")
-    model = random_model_on_device(config, "cuda:0", dtype, RandomInit(seed=0, std=0.02))
-    model.name = "qwen3-8b-random"
+    model, config, full_layers = random_model(MODEL, args.layers, dtype)
 
-    start_context = args.context - args.steps - args.warmup
-    if start_context < 1:
-        parser.error("--context must exceed --steps + --warmup")
-
-    def decode_rate(batch, steps, warmup):
-        log(f"[bench] decode batch {batch}: filling {batch} x {args.context - steps - warmup} tokens of cache")
-        bench = DecodeBench(model, args.page_size, batch, args.context - steps - warmup, args.context)
-        log(f"[bench] decode batch {batch}: timing {steps} steps")
-        elapsed = bench.run(steps, warmup)
-        bench.close()
-        return elapsed
-
-    elapsed = decode_rate(args.batch, args.steps, args.warmup)
-    ms_per_step = 1000.0 * elapsed / args.steps
-    value = args.batch * args.steps / elapsed
-    mean_context = args.context - args.steps / 2.0
-    step_bytes = weight_bytes(config, elem) + args.batch * mean_context * kv_bytes_per_token(config, elem)
-    achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
+    log(f"[bench] decode batch {args.batch}: {args.batch} prompts of {args.context - args.steps - args.warmup} tokens, then {args.warmup} + {args.steps} steps")
+    value, ms_per_step, achieved = decode_point(model, config, elem, args.page_size, args.batch, args.context, args.steps, args.warmup)
     result = {
         "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen3-8B-sized, random weights)", "value": round(value, 2),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short, "data": "synthetic",
-        "config": {"model": "qwen3-8b-sized", "layers": config.num_hidden_layers, "layers_full": FULL_LAYERS,
+        "config": {"model": "qwen3-8b-sized", "layers": config.num_hidden_layers, "layers_full": full_layers,
                    "hidden": config.hidden_size, "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
                    "head_dim": config.head_dim, "intermediate": config.intermediate_size, "vocab": config.vocab_size,
                    "global_batch": args.batch, "seq_len": args.context, "prefill_tokens": args.prefill_tokens,
-                   "page_size": args.page_size, "weights": "random N(0,0.02)", "parallelism": "single-gpu"},
+                   "page_size": args.page_size, "weights": "random N(0,0.02)", "timed_through": "Engine.step",
+                   "parallelism": "single-gpu"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
     if not args.no_prefill:
         log(f"[bench] prefill of {args.prefill_tokens} tokens")
-        seconds = time_prefill(model, args.page_size, args.prefill_tokens)
+        seconds = prefill_through_engine(model, args.page_size, args.prefill_tokens)
         flops = prefill_flops(config, args.prefill_tokens)
         result["prefill"] = {"value": round(args.prefill_tokens / seconds, 1), "tokens": args.prefill_tokens,
                              "ms": round(1000.0 * seconds, 3),
                              "frac": round(flops / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)}
+    points = {}
     if not args.no_points:
-        points = {}
         for batch, steps in ((1, min(args.steps, 64)), (64, min(args.steps, 32))):
-            seconds = decode_rate(batch, steps, min(args.warmup, 4))
-            points[f"decode_b{batch}"] = round(batch * steps / seconds, 2)
+            log(f"[bench] decode batch {batch}")
+            rate, ms, gbs = decode_point(model, config, elem, args.page_size, batch, args.context, steps, min(args.warmup, 4))
+            points[f"decode_b{batch}"] = round(rate, 2)
+            points[f"decode_b{batch}_ms_per_step"] = round(ms, 4)
+            points[f"decode_b{batch}_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
+    del model
+    torch.cuda.empty_cache()
+    if not args.no_points and not args.no_extra_points and dtype == torch.bfloat16 and not args.layers:
+        points.update(extra_points(dtype, elem, args.page_size))
+    if points:
         result["points"] = points
     print(json.dumps(result), flush=True)
     return 0
+
+
+def extra_points(dtype, elem, page_size):
+    """The two other workloads the baseline names, each on a random model of its own size."""
+    import torch
+
+    from llmserver_amd.cli.benchmark import mixed_workload
+    from llmserver_amd.engine import Engine
+    points = {}
+    # 64 concurrent requests, prompts of 16 to 2,048 tokens, half of them behind one shared prefix of 512 tokens, 256 new
+    # tokens each, continuous batching with chunked prefill (Qwen3-1.7B sizes).
+    model, config, _ = random_model("qwen3-1.7b", 0, dtype)
+    requests, high, new_tokens = 64, 2048, 256
+    engine = Engine(model, None, max_new_tokens=new_tokens, max_batch_size=requests, max_num_batched_tokens=16384,
+                    kv_cache_num_blocks=requests * (-(-(high + new_tokens) // page_size)) + 8, kv_cache_block_size=page_size,
+                    stream_text=False, max_completed_requests=0, ignore_eos=True, enable_prefix_caching=True)
+    engine.warmup_graphs(max_context=high + new_tokens)
+    entry = mixed_workload(engine, config.vocab_size, requests, 16, high, 512, 0.5, new_tokens)
+    log(f"[bench] mixed workload: {entry}")
+    points["mixed_1p7b_64req_generated_tok_s"] = round(entry["generated_tok_s"], 1)
+    points["mixed_1p7b_64req_total_s"] = round(entry["total_s"], 3)
+    points["mixed_1p7b_64req_prefix_hit_tokens"] = int(entry["prefix_hit_tokens"])
+    points["mixed_1p7b_64req_prompt_tokens"] = int(entry["prompt_tokens_total"])
+    del engine, model
+    torch.cuda.empty_cache()
+    # Batch 16 behind prompts of 8,192 tokens (Qwen3-32B sizes): the decoding steps up to a context of 8,192 + 64.
+    model, config, _ = random_model("qwen3-32b", 0, dtype)
+    batch, context, steps, warmup = 16, 8192 + 64, 48, 4
+    rate, ms, gbs = decode_point(model, config, elem, page_size, batch, context, steps, warmup)
+    points["decode_32b_b16_ctx8192"] = round(rate, 2)
+    points["decode_32b_b16_ctx8192_ms_per_step"] = round(ms, 4)
+    points["decode_32b_b16_ctx8192_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
+    del model
+    torch.cuda.empty_cache()
+    return points
 
 
 if __name__ == "__main__":

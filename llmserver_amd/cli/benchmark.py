@@ -69,6 +69,33 @@ def run_once(engine, prompts, new_tokens):
     return time.perf_counter() - start, [list(r.generated_token_ids) for r in requests]
 
 
+def mixed_workload(engine, vocab, requests, low, high, shared_prefix_tokens, shared_fraction, output_tokens, seed=0) -> dict:
+    """``requests`` concurrent requests with prompt lengths uniform in [low, high], a fraction of them starting with
+    one shared random prefix, ``output_tokens`` greedy tokens each, under continuous batching with chunked prefill.
+    A short run first loads what a first run loads; the counters are the timed run's."""
+    import random
+    rng = random.Random(seed)
+    prefix = build_prompts(vocab, shared_prefix_tokens, 1, "shared-prefix", seed)[0]
+    prompts = []
+    for index in range(requests):
+        length = rng.randint(low, high)
+        body = build_prompts(vocab, length, 1, f"mixed-{index}", seed)[0]
+        if index < shared_fraction * requests and length > shared_prefix_tokens:
+            body = prefix + body[shared_prefix_tokens:]
+        prompts.append(body)
+    rng.shuffle(prompts)
+    run_once(engine, build_prompts(vocab, 64, min(4, engine.scheduler.max_batch_size), "warm-mixed", seed), 4)
+    for key in ("steps", "decode_steps", "prefill_steps", "tokens", "prefix_hit_tokens", "preemptions"):
+        engine.step_profile[key] = 0
+    seconds, _ = run_once(engine, prompts, output_tokens)
+    prompt_total = sum(len(p) for p in prompts)
+    return {"workload": "mixed", "requests": requests, "prompt_tokens_total": prompt_total, "output_tokens": output_tokens,
+            "total_s": seconds, "generated_tok_s": requests * output_tokens / seconds,
+            "processed_tok_s": (prompt_total + requests * output_tokens) / seconds,
+            "prefix_hit_tokens": engine.step_profile["prefix_hit_tokens"], "steps": engine.step_profile["steps"],
+            "preemptions": engine.step_profile["preemptions"]}
+
+
 def one_prompt(args, model, load_seconds) -> int:
     """One prompt, ``--repeats`` fresh requests: the reference's single-prompt statistics
     (/root/reference/benchmark.py:68-88)."""
@@ -96,7 +123,7 @@ def one_prompt(args, model, load_seconds) -> int:
                     max_num_batched_tokens=max(args.max_num_batched_tokens, 1), prefill_chunk_size=args.prefill_chunk_size,
                     kv_cache_num_blocks=blocks, kv_cache_block_size=args.block_size, stream_text=False, max_completed_requests=0,
                     ignore_eos=False, temperature=args.temperature, seed=args.seed, enable_prefix_caching=False)
-    run_once(engine, [prompt_ids], min(args.max_new_tokens, 4))               # graphs and kernel choices, before the clock
+    run_once(engine, [prompt_ids], min(args.max_new_tokens, 4))               # graphs are captured before the clock starts
     results = []
     for _ in range(args.repeats):
         torch.cuda.synchronize()
@@ -198,33 +225,13 @@ def main(argv=None) -> int:
                     ignore_eos=True, temperature=args.temperature, seed=args.seed, enable_prefix_caching=True)
     results = []
     if args.mixed_requests:
-        import random
-        rng = random.Random(args.seed)
-        prefix = build_prompts(vocab, args.shared_prefix_tokens, 1, "shared-prefix", args.seed)[0]
-        prompts = []
-        for index in range(args.mixed_requests):
-            length = rng.randint(low, high)
-            body = build_prompts(vocab, length, 1, f"mixed-{index}", args.seed)[0]
-            if index < args.shared_fraction * args.mixed_requests and length > args.shared_prefix_tokens:
-                body = prefix + body[args.shared_prefix_tokens:]
-            prompts.append(body)
-        rng.shuffle(prompts)
-        # A server captures its decode graphs (and measures its kernel choices) at start-up, before requests come
-        # (/root/reference/server.py:332): so does this workload, which stands for one.
+        # A server captures its decode graphs at start-up, before requests come (server.py:332 in the reference):
+        # so does this workload, which stands for one.
         engine.warmup_graphs(max_context=high + args.output_tokens)
-        run_once(engine, build_prompts(vocab, 64, min(4, max_batch), "warm-mixed", args.seed), 4)
-        for key in ("steps", "decode_steps", "prefill_steps", "tokens", "prefix_hit_tokens", "preemptions"):
-            engine.step_profile[key] = 0
-        seconds, generated = run_once(engine, prompts, args.output_tokens)
-        prompt_total = sum(len(p) for p in prompts)
-        entry = {"workload": "mixed", "requests": args.mixed_requests, "prompt_tokens_total": prompt_total,
-                 "output_tokens": args.output_tokens, "total_s": seconds,
-                 "generated_tok_s": args.mixed_requests * args.output_tokens / seconds,
-                 "processed_tok_s": (prompt_total + args.mixed_requests * args.output_tokens) / seconds,
-                 "prefix_hit_tokens": engine.step_profile["prefix_hit_tokens"], "steps": engine.step_profile["steps"],
-                 "preemptions": engine.step_profile["preemptions"]}
-        print(f"mixed: {args.mixed_requests} requests, {prompt_total} prompt tokens ({entry['prefix_hit_tokens']} served from cached prefix pages), "
-              f"{args.output_tokens} new tokens each: {seconds:.3f} s, {entry['generated_tok_s']:.1f} generated tok/s, "
+        entry = mixed_workload(engine, vocab, args.mixed_requests, low, high, args.shared_prefix_tokens, args.shared_fraction,
+                               args.output_tokens, args.seed)
+        print(f"mixed: {args.mixed_requests} requests, {entry['prompt_tokens_total']} prompt tokens ({entry['prefix_hit_tokens']} served from cached prefix pages), "
+              f"{args.output_tokens} new tokens each: {entry['total_s']:.3f} s, {entry['generated_tok_s']:.1f} generated tok/s, "
               f"{entry['processed_tok_s']:.1f} processed tok/s, {entry['steps']} steps, {entry['preemptions']} preemptions", flush=True)
         results.append(entry)
         prompt_lengths = []
@@ -234,8 +241,8 @@ def main(argv=None) -> int:
             try:
                 if batch * (prompt_length + args.output_tokens) > wanted * args.block_size:
                     raise MemoryError("KV cache too small for this configuration")
-                # One whole run first, as the reference warms up (/root/reference/benchmark_cuda.py:208): every graph the
-                # timed runs replay is captured and every choice of a kernel is measured before the clock starts.
+                # One whole run first, as the reference warms up (benchmark_cuda.py:208 there): every graph the timed
+                # runs replay is captured before the clock starts.
                 run_once(engine, build_prompts(vocab, prompt_length, batch, f"warm-{prompt_length}-{batch}", args.seed), args.output_tokens)
                 ttft, total, tokens = [], [], None
                 for repeat in range(args.repeats):

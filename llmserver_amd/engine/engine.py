@@ -370,6 +370,42 @@ class Engine:
             return 0
         return self.runner.graph_count()
 
+    def calibrate(self, save_to: Optional[str] = None, portions=(24, 32, 48, 64, 96, 128)) -> int:
+        """Measure, for this model's shapes, which products go through a hand-written kernel and which through the
+        library, for every number of decoding rows up to ``max_batch_size`` and for prompt portions of the given sizes;
+        an idle engine only, never part of serving.  The findings join the kernel namespace's table of choices (and the
+        file ``save_to``, if given, which ``LLMSERVER_AMD_CHOICES`` can name in later runs).  Returns how many shapes
+        were measured.  Graphs captured before are dropped: they may hold the other choice."""
+        measuring = getattr(self.runner.ops, "measuring", None)
+        if measuring is None or self.active_requests:
+            return 0
+        most = self.scheduler.max_batch_size
+        sizes = [(rows, 1) for rows in range(1, most + 1)]
+        sizes += [(1, tokens) for tokens in portions if tokens <= self.max_num_batched_tokens]
+        graphs, self.runner.use_graphs = self.runner.use_graphs, False
+        try:
+            with measuring() as choices:
+                before = len(choices.measured)
+                for rows, tokens in sizes:
+                    if rows * -(-tokens // self.block_size) > min(self.kv_cache.available_pages() or [1 << 30]):
+                        continue
+                    names = [f"calibrate-{i}" for i in range(rows)]
+                    try:
+                        for name in names:
+                            self.kv_cache.open(name)
+                        self.runner.step([StepEntry(name, [0] * tokens, [tokens - 1]) for name in names])
+                    finally:
+                        for name in names:
+                            if name in self.kv_cache.requests:
+                                self.kv_cache.close(name)
+                measured = len(choices.measured) - before
+                if save_to:
+                    choices.save(save_to)
+        finally:
+            self.runner.use_graphs = graphs
+            self.runner.drop_graphs()
+        return measured
+
     def prepare_next_step(self, sampled, pending=None) -> bool:
         """If the next step can only be a decoding step of known requests (nobody can join, nobody is still behind
         its sequence), let the runner lay it out before this step's tokens are back; and if it brings exactly the

@@ -13,6 +13,7 @@ import torch
 
 from ..parts.attention import AttentionTuning, group_tiling
 from . import build, library
+from .choices import ChoiceTable, choice_key
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 SKINNY_GEMM_ROWS = 16       # up to this many rows the hand-written weight-streaming products, with the sums, norms and the
@@ -80,11 +81,15 @@ class HipOps:
         # Whether projections whose result is added to the residual stream may leave it as partial sums at 17 to 128 rows.
         self.split_products = True
         self._split_parts = {}      # (rows, out, in) -> partial sums the split product writes for that size
-        # The few-row products win on most shapes but not on all (on Qwen3-32B's gate/up the library is a third faster):
-        # the first time a size is met outside a graph capture, the few-row kernel is timed against the library's
-        # product plus the kernels it would have absorbed, and the faster is kept for that size.
-        self.choose_by_measurement = True
-        self._library_faster = {}   # (kind, rows, out, in, scaled, float32 result) -> bool
+        # The few-row products win on most shapes but not on all (on Qwen3-32B's gate/up the library is a third faster).
+        # Which way a shape goes is looked up in a table per GPU model (see choices.py); a shape the table does not
+        # know goes the hand-written way.  Nothing is timed unless somebody asks for it (``measuring()``).
+        self.consult_choices = True
+        properties = torch.cuda.get_device_properties(torch.cuda.current_device())
+        # (the marketing name is the same for several chips; the architecture and the number of compute units tell them apart)
+        self.device_kind = f"{str(getattr(properties, 'gcnArchName', properties.name)).split(':')[0]}-{properties.multi_processor_count}cu"
+        self.choices = ChoiceTable.load(self.device_kind)
+        self._measuring = False
         self._flush = None
         self._replay_overhead = None
         self._tuning = None
@@ -182,24 +187,24 @@ class HipOps:
         """Whether, for these sizes, the library's product (with a norm kernel before it if ``scaled``, and the
         activation kernel after it if ``kind`` is "gated") beats the kernel of this repository that does it all;
         ``kind`` "partial": the product in partial sums and the norm kernel that adds them up, against the library's
-        product and the plain norm kernel.  Measured once."""
-        if not self.choose_by_measurement:
+        product and the plain norm kernel.  Looked up in the table of choices; measured only inside ``measuring()``."""
+        if not self.consult_choices:
             return False
         rows, width = x.shape
-        # Beyond the few-row kernels one measurement stands for eight neighbouring numbers of rows (portions of
-        # prompts come in every length, and each measurement takes a few milliseconds).
-        key = (kind, rows if rows <= 16 else -(-rows // 8) * 8, weight.shape[0], width, bool(scaled), bool(out_float32))
-        known = self._library_faster.get(key)
+        # Beyond the few-row kernels one entry stands for eight neighbouring numbers of rows (portions of prompts
+        # come in every length).
+        key = choice_key(kind, rows if rows <= 16 else -(-rows // 8) * 8, weight.shape[0], width, scaled, out_float32)
+        known = self.choices.get(key)
         if known is not None:
             return known
-        if torch.cuda.is_current_stream_capturing():
-            return False                                  # nothing can be timed while a graph is recorded
+        if not self._measuring or torch.cuda.is_current_stream_capturing():
+            return False                                  # unknown shape: this repository's kernel
         sums = torch.ones((rows, 16), device=x.device, dtype=torch.float32) if scaled else None
         row_scale = (sums, 1e-6) if scaled else None
         stream = torch.zeros_like(x) if scaled else None
         norm_weight = torch.ones(width, device=x.device, dtype=torch.float32) if scaled else None
         normed = torch.empty_like(x) if scaled else None
-        saved, self.choose_by_measurement = self.choose_by_measurement, False
+        saved, self.consult_choices = self.consult_choices, False
         try:
             if kind == "partial":
                 stream = torch.zeros((rows, weight.shape[0]), device=x.device, dtype=x.dtype)
@@ -233,32 +238,47 @@ class HipOps:
                         self.add_rmsnorm(stream, None, norm_weight, 1e-6, normed)
                     return torch.mm(x, weight.t(), out_dtype=torch.float32) if out_float32 else torch.mm(x, weight.t())
             if few() is None:
-                self._library_faster[key] = False         # no case for this repository's kernel: nothing to choose
-                return False
+                return False                              # no case for this repository's kernel: nothing to choose
             faster = self._second_is_faster(few, library)
         finally:
-            self.choose_by_measurement = saved
-        self._library_faster[key] = faster
+            self.consult_choices = saved
+        self.choices.record(key, faster)
         return faster
+
+    def measuring(self):
+        """A context in which shapes that the table of choices does not know are timed the first time they are met
+        (a few milliseconds each) and entered into ``self.choices``; afterwards the buffer that the timing uses to
+        empty the caches is given back.  Never entered by a step that serves a request."""
+        import contextlib
+
+        @contextlib.contextmanager
+        def context():
+            saved, self._measuring = self._measuring, True
+            try:
+                yield self.choices
+            finally:
+                self._measuring = saved
+                self._flush = None
+        return context()
 
     def partial_sums_are_faster(self, x, weight) -> bool:
         """For a projection of few rows into the residual stream: whether the product in partial sums plus the kernel
         that adds them up and normalises beats the few-row kernel that does it all (long inner dimensions at 9 to 16
         rows, where every workgroup of the few-row kernel moves as many activations as weights); measured once."""
         rows, width = x.shape
-        if not self.choose_by_measurement or not self.split_products or not self.fuse_stream_updates \
+        if not self.consult_choices or not self.split_products or not self.fuse_stream_updates \
                 or not 8 < rows <= self.skinny_rows or not self._few_rows(x, weight):
             return False
-        key = ("stream", rows, weight.shape[0], width, False, False)
-        known = self._library_faster.get(key)
+        key = choice_key("stream", rows, weight.shape[0], width, False, False)
+        known = self.choices.get(key)
         if known is not None:
             return known
-        if torch.cuda.is_current_stream_capturing():
+        if not self._measuring or torch.cuda.is_current_stream_capturing():
             return False
         resid = torch.zeros((rows, weight.shape[0]), device=x.device, dtype=x.dtype)
         norm_weight = torch.ones(weight.shape[0], device=x.device, dtype=torch.float32)
         normed = torch.empty_like(resid)
-        saved, self.choose_by_measurement = self.choose_by_measurement, False
+        saved, self.consult_choices = self.consult_choices, False
         try:
             def few():
                 return self.linear_into_stream(x, weight, resid, norm_weight)
@@ -270,8 +290,8 @@ class HipOps:
             else:
                 faster = self._second_is_faster(few, split)
         finally:
-            self.choose_by_measurement = saved
-        self._library_faster[key] = faster
+            self.consult_choices = saved
+        self.choices.record(key, faster)
         return faster
 
     def _row_scale_args(self, row_scale, rows):

@@ -18,13 +18,13 @@ TOL = {torch.float32: dict(atol=2e-5, rtol=1e-5), torch.bfloat16: dict(atol=2e-2
 
 @pytest.fixture(scope="module")
 def ops():
-    """The kernels themselves are under test here: the choice between a few-row kernel and the library by
-    measurement, which serving makes, is switched off (it has a test of its own below)."""
+    """The kernels themselves are under test here: the table that sends some shapes to the library instead of a
+    few-row kernel, which serving consults, is switched off (it has a test of its own below)."""
     from llmserver_amd.kernels import default_ops
     ops = default_ops()
-    ops.choose_by_measurement = False
+    ops.consult_choices = False
     yield ops
-    ops.choose_by_measurement = True
+    ops.consult_choices = True
 
 
 class Ctx:
@@ -618,42 +618,53 @@ def test_gated_product_beyond_few_rows(ops, rows, inter, k):
     assert ops._gemm.lsa_gemm_split_gated(x.data_ptr(), w.data_ptr(), x.data_ptr(), 16, inter, k, None) == -1
 
 
-def test_few_row_kernel_or_library_by_measurement(ops):
-    """Serving times a few-row kernel against the library's product (plus the kernels it would have absorbed) the
-    first time it meets a size, keeps the faster and asks no more; either way the product is right; while a graph is
-    recorded nothing is timed and the few-row kernel stands."""
-    print("few-row kernel or library by measurement", flush=True)
+def test_few_row_kernel_or_library_by_table(ops, tmp_path):
+    """A shape goes the way the table of choices says; a shape the table does not know goes the few-row kernel's way
+    and nothing is timed, unless the caller is inside ``measuring()``: then it is timed once, entered into the table
+    and can be saved.  Either way the product is right.  While a graph is recorded nothing is timed."""
+    from llmserver_amd.kernels.choices import ChoiceTable, choice_key
+    print("few-row kernel or library by table", flush=True)
     torch.manual_seed(5)
     x = torch.randn(8, 512, device=DEV).to(torch.bfloat16)
     w = (torch.randn(1024, 512, device=DEV) / 512 ** 0.5).to(torch.bfloat16)
     expected = (x.double() @ w.double().t()).float()
-    ops.choose_by_measurement = True
+    plain_key, gated_key = choice_key("plain", 8, 1024, 512, False, False), choice_key("gated", 8, 1024, 512, False, False)
+    saved_table, ops.choices = ops.choices, ChoiceTable(ops.choices.device_name)
+    ops.consult_choices = True
     try:
-        ops._library_faster.clear()
         for _ in range(2):
             torch.testing.assert_close(ops.linear(x, w).float(), expected, atol=2e-2, rtol=1e-2)
-        assert list(ops._library_faster) == [("plain", 8, 1024, 512, False, False)]
+        assert not ops.choices.entries and ops._flush is None      # an unknown shape: no timing, no entry
+        with ops.measuring():
+            for _ in range(2):
+                torch.testing.assert_close(ops.linear(x, w).float(), expected, atol=2e-2, rtol=1e-2)
+        assert list(ops.choices.entries) == [plain_key] == list(ops.choices.measured)
+        assert ops._flush is None                                    # the buffer that empties the caches is given back
+        path = str(tmp_path / "choices.json")
+        assert ops.choices.save(path) == 1
+        again = ChoiceTable.load(ops.choices.device_name, [path])
+        assert again.entries == ops.choices.entries and ChoiceTable.load("another GPU", [path]).entries == {}
         for forced in (True, False):
-            ops._library_faster[("plain", 8, 1024, 512, False, False)] = forced
+            ops.choices.entries[plain_key] = forced
             torch.testing.assert_close(ops.linear(x, w).float(), expected, atol=2e-2, rtol=1e-2)
-        ops._library_faster[("gated", 8, 1024, 512, False, False)] = True
+        ops.choices.entries[gated_key] = True
         assert ops.linear_gated(x, w) is None and ops.linear_gated(x, w, pairs_per_workgroup=8) is not None
-        ops._library_faster[("gated", 8, 1024, 512, False, False)] = False
+        ops.choices.entries[gated_key] = False
         assert ops.linear_gated(x, w) is not None
-        ops._library_faster.clear()
+        ops.choices = ChoiceTable(ops.choices.device_name)
         graph = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             ops.linear(x, w)                              # (warm-up on the side stream, as graph capture wants it)
         torch.cuda.current_stream().wait_stream(side)
-        ops._library_faster.clear()
-        with torch.cuda.graph(graph):
-            captured = ops.linear(x, w)
-        assert not ops._library_faster                    # nothing was measured during the capture
+        with ops.measuring():
+            with torch.cuda.graph(graph):
+                captured = ops.linear(x, w)
+        assert not ops.choices.entries                    # nothing was measured during the capture
         graph.replay()
         torch.cuda.synchronize()
         torch.testing.assert_close(captured.float(), expected, atol=2e-2, rtol=1e-2)
     finally:
-        ops._library_faster.clear()
-        ops.choose_by_measurement = False
+        ops.choices = saved_table
+        ops.consult_choices = False
