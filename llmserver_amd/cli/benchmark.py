@@ -1,5 +1,5 @@
 """Benchmark of the engine on token-id prompts, in the manner of the reference's
-``benchmark_cuda.py`` (/root/reference/benchmark_cuda.py:1-13, 475-496): option names and
+``benchmark_cuda.py`` (benchmark_cuda.py:1-13, 475-496): option names and
 meanings follow it where it has them.
 
     python benchmark.py --model DIR --prompt-tokens 128,1024 --batch-sizes 1,8,32 --output-tokens 128
@@ -7,7 +7,7 @@ meanings follow it where it has them.
     python benchmark.py --model DIR --prompt-token-ids 151644,872,198 --max-new-tokens 32 --repeats 3
 
 With ``--prompt`` (text, if the model folder has a ``tokenizer.json``) or ``--prompt-token-ids`` it benchmarks one prompt
-in the manner of the reference's ``benchmark.py`` (/root/reference/benchmark.py:68-88, 339-341): model load, time to
+in the manner of the reference's ``benchmark.py`` (benchmark.py:68-88, 339-341): model load, time to
 the first token, generation and decode throughput, medians over ``--repeats``.
 
 For each (prompt length, batch size):
@@ -16,7 +16,7 @@ For each (prompt length, batch size):
   * decode tok/s = batch * (output_tokens - 1) / (total_s - ttft_s)
 EOS is ignored, decoding is greedy unless ``--temperature`` is given, and every (prompt length,
 batch size, repeat) gets its own seeded random token ids, so prefix caching cannot help
-(/root/reference/benchmark_cuda.py:13, 32-38).  ``--random-config`` draws seeded random weights
+(benchmark_cuda.py:13, 32-38).  ``--random-config`` draws seeded random weights
 on the device instead of reading a folder.
 """
 from __future__ import annotations
@@ -98,7 +98,7 @@ def mixed_workload(engine, vocab, requests, low, high, shared_prefix_tokens, sha
 
 def one_prompt(args, model, load_seconds) -> int:
     """One prompt, ``--repeats`` fresh requests: the reference's single-prompt statistics
-    (/root/reference/benchmark.py:68-88)."""
+    (benchmark.py:68-88)."""
     import os
 
     import torch
@@ -168,7 +168,7 @@ def main(argv=None) -> int:
     parser.add_argument("--repeats", type=int, default=3)
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--custom-dtype", default=None, choices=("source", "fp32", "fp16"),
-                        help="the reference's name of --dtype (/root/reference/benchmark.py:344): source = bfloat16 as stored, fp32 = float32; fp16 is not built")
+                        help="the reference's name of --dtype (benchmark.py:344): source = bfloat16 as stored, fp32 = float32; fp16 is not built")
     parser.add_argument("--device", default="cuda")
     parser.add_argument("--block-size", type=int, default=16)
     parser.add_argument("--max-num-batched-tokens", type=int, default=16384)
@@ -217,7 +217,7 @@ def main(argv=None) -> int:
         prompt_lengths, batches = [high], [args.max_batch_size or args.mixed_requests]
     max_batch, max_length = max(batches), max(prompt_lengths) + args.output_tokens
     bytes_per_block = CacheManager.bytes_per_token(model.cache_specs(), model.dtype) * args.block_size
-    wanted = max_batch * math.ceil(max_length / args.block_size) + 8          # /root/reference/benchmark_cuda.py:107-111
+    wanted = max_batch * math.ceil(max_length / args.block_size) + 8          # benchmark_cuda.py:107-111
     wanted = min(wanted, int(torch.cuda.mem_get_info()[0] * 0.8 // max(1, bytes_per_block)))
     engine = Engine(model, None, max_new_tokens=1, max_batch_size=max_batch,
                     max_num_batched_tokens=max(args.max_num_batched_tokens, max_batch), prefill_chunk_size=args.prefill_chunk_size,

@@ -2,9 +2,9 @@
 
 A configuration is read from the architecture's own ``config.json`` keys and nothing else; no
 size or constant that ``config.json`` gives is repeated in code.  The reference builds an untyped
-kwargs dict from a library config object (/root/reference/utils/architecture.py:90-107); here the
+kwargs dict from a library config object (utils/architecture.py:90-107); here the
 file is parsed directly into a frozen dataclass whose ``validate`` gives every refusal a reason
-(/root/reference/utils/architecture.py:50-86).
+(utils/architecture.py:50-86).
 """
 from __future__ import annotations
 
@@ -17,7 +17,7 @@ from typing import Any, ClassVar, Mapping
 class UnsupportedModelError(ValueError):
     """A model folder describes something this engine does not implement.
 
-    Same role as /root/reference/utils/architecture.py:19.
+    Same role as utils/architecture.py:19.
     """
 
 

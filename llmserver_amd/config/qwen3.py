@@ -1,11 +1,11 @@
 """Qwen3 dense decoder configuration, read from the keys of its ``config.json``.
 
-Keys and defaults follow what the reference reads (/root/reference/utils/architecture.py:72-107):
+Keys and defaults follow what the reference reads (utils/architecture.py:72-107):
 ``head_dim`` defaults to ``hidden_size // num_attention_heads`` (line 88) and need not multiply
 back to the hidden size; ``rope_theta`` may sit at top level or inside ``rope_parameters`` /
 ``rope_scaling`` and defaults to 10000.0 (lines 23-30); ``rms_norm_eps`` has no default (106);
 ``num_key_value_heads``, when the file leaves it out, is the number of query heads (plain multi-head attention).
-The refusals are the reference's (72-86, /root/reference/utils/attention.py:186-187).
+The refusals are the reference's (72-86, utils/attention.py:186-187).
 """
 from __future__ import annotations
 

@@ -1,7 +1,7 @@
 """One registry from an architecture's name to its configuration class and model builder.
 
 The reference keeps a tuple of verified ``model_type`` strings and refuses the rest with a
-message that says what is supported (/root/reference/utils/architecture.py:16,48-54).  Here the
+message that says what is supported (utils/architecture.py:16,48-54).  Here the
 name maps to ``(config class, builder)``; a builder takes the typed config and returns a model
 assembled from parts.  Registering another architecture is one call and changes no file here.
 """

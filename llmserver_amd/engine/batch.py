@@ -5,8 +5,8 @@ prompt or one decoded token, cut anywhere.  All of them are laid end to end as `
 Per token: id, absolute position, request row.  Per row: where its tokens start, how many there
 are, and the context length after the step.  Per cache group: the rows' block tables.  Every
 integer array is staged in one pinned host buffer and reaches the GPU in one copy, the
-reference's static-header idea (/root/reference/utils/cuda_graph.py:29-34, 86-95) extended to
-mixed batches, which the reference never forms (/root/reference/utils/batch.py:4-81).
+reference's static-header idea (utils/cuda_graph.py:29-34, 86-95) extended to
+mixed batches, which the reference never forms (utils/batch.py:4-81).
 """
 from __future__ import annotations
 

@@ -1,5 +1,5 @@
 """From a model folder to a model on the device, in the reference's manner
-(/root/reference/utils/model_loader.py:18-86): the configuration picks the architecture, the
+(utils/model_loader.py:18-86): the configuration picks the architecture, the
 architecture's builder assembles the parts, the weights are streamed in by name."""
 from __future__ import annotations
 

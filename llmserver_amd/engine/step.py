@@ -3,7 +3,7 @@
 It runs only the tokens it is given, as one flat batch, against the cache earlier steps left:
 portions of prompts beside single decoded tokens, cut anywhere.  The reference runs two kinds of
 forward per engine step, padded prefill batches and a decode batch
-(/root/reference/utils/engine.py:437-443, /root/reference/utils/model.py:76-158); here there is
+(utils/engine.py:437-443, utils/model.py:76-158); here there is
 one pass, and one code path serves generation, the benchmark and trace replay.
 
 A step that brings one token per request is launch-bound, so it is captured once into a HIP
@@ -11,7 +11,7 @@ graph per (rows, block-table width, wanted rows) and replayed afterwards: the ke
 everything that changes from the staged arrays, whose addresses and shapes stay the same.  Decoding
 steps are filled up with rows of nobody's to one of a few sizes, so that few graphs serve every batch.  The
 reference replays its decode pass from a CUDA graph in the same way
-(/root/reference/utils/cuda_graph.py:51-99).
+(utils/cuda_graph.py:51-99).
 
 Such a step can be laid out on the host while the GPU still runs the step before it (``prepare_ahead``: everything but
 the token ids is known then), and started before the host has seen those tokens (``launch_ahead``: the ids are copied

@@ -1,5 +1,5 @@
 """Python entry points in the reference's manner: ``model_loader(...)`` then ``Engine(...)``
-(/root/reference/utils/model_loader.py:18, /root/reference/utils/engine.py:47)."""
+(utils/model_loader.py:18, utils/engine.py:47)."""
 from __future__ import annotations
 
 from typing import List, Sequence

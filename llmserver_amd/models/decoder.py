@@ -3,8 +3,8 @@
 The order is data: ``order`` is a list of :class:`LayerCall`, each naming a block and the cache
 it uses.  A block may be named twice (its weights are shared) and a call may read the cache that
 another call writes.  The plain stacked model is ``[LayerCall(i, i) for i in range(L)]``
-(/root/reference/utils/model.py:124-132).  Rows whose logits are wanted are selected before the
-final norm and the head (/root/reference/utils/model.py:147-158).
+(utils/model.py:124-132).  Rows whose logits are wanted are selected before the
+final norm and the head (utils/model.py:147-158).
 """
 from __future__ import annotations
 
@@ -77,7 +77,7 @@ class DecoderModel:
         specs.update({f"{self.norm_name}.{k}": v for k, v in self.final_norm.param_specs().items()})
         for k, v in self.head.param_specs().items():
             # Tied when the configuration says so or the checkpoint holds no head
-            # (/root/reference/utils/model_loader.py:56-59).
+            # (utils/model_loader.py:56-59).
             specs[k] = dataclasses.replace(v, optional=True)
         return specs
 

@@ -1,10 +1,10 @@
 """Qwen3 dense decoder put together from parts, layer by layer, from its typed configuration.
 
-Layer kinds and tensor names as the reference has them (/root/reference/utils/model.py:7-54,
-/root/reference/utils/attention.py:33-39, /root/reference/utils/layers.py:188-191,
-/root/reference/utils/model_loader.py:54-67): pre-norm blocks of grouped-query attention with
+Layer kinds and tensor names as the reference has them (utils/model.py:7-54,
+utils/attention.py:33-39, utils/layers.py:188-191,
+utils/model_loader.py:54-67): pre-norm blocks of grouped-query attention with
 per-head q/k RMSNorm and rotate-half RoPE, and a SwiGLU feed-forward; one eps for every norm
-(/root/reference/utils/model.py:10-12, /root/reference/utils/attention.py:38-39).
+(utils/model.py:10-12, utils/attention.py:38-39).
 """
 from __future__ import annotations
 

@@ -1,22 +1,22 @@
 """Grouped-query causal attention over a paged cache, with optional per-head q/k RMSNorm,
 rotate-half position encoding and an optional window.
 
-Formulas in execution order (/root/reference/utils/attention.py:114-160, 183-197):
+Formulas in execution order (utils/attention.py:114-160, 183-197):
 ``q,k,v = x Wq^T, x Wk^T, x Wv^T`` as one stacked product (54-66, 124-126); per head
 ``q^ = q * rsqrt(mean_d(q^2) + eps) * w_q`` and the same for k, before the rotation (157-158;
-fused form /root/reference/utils/fused_ops.py:90-134); rotation of q and k by the absolute
+fused form utils/fused_ops.py:90-134); rotation of q and k by the absolute
 position; rotated k and raw v of every new token go to the cache before attention reads it
-(/root/reference/utils/kv_cache.py:335-349), so a token sees itself; query head ``h`` uses KV head
-``h // G`` (/root/reference/utils/attention.py:77,188); scores ``q.k * scale`` with
-``scale = head_dim^-0.5`` by default (/root/reference/utils/architecture.py:105), causal within
-the request, softmax and accumulation in 32-bit (/root/reference/utils/attention.py:75-96,197);
+(utils/kv_cache.py:335-349), so a token sees itself; query head ``h`` uses KV head
+``h // G`` (utils/attention.py:77,188); scores ``q.k * scale`` with
+``scale = head_dim^-0.5`` by default (utils/architecture.py:105), causal within
+the request, softmax and accumulation in 32-bit (utils/attention.py:75-96,197);
 output projection (299-300).
 
 The attention kernel works through a list of work items made on the host once a step
 (:func:`build_attention_plan`): an item is 16 rows of (token, head-of-the-group) pairs against
 a contiguous range of keys.  Rows with few tokens and many keys are cut into several items
 whose partial results a second kernel merges by log-sum-exp, the reference's split-KV idea
-(/root/reference/utils/paged_attention.py:78-115).
+(utils/paged_attention.py:78-115).
 """
 from __future__ import annotations
 

@@ -1,7 +1,7 @@
 """Pre-norm residual block: ``h += mixer(norm_in(h)); h += ffn(norm_post(h))``.
 
-Order of the parts as in /root/reference/utils/model.py:15-35.  The block keeps the reference's
-fused dataflow (/root/reference/utils/model.py:87-100): the residual stream and the update that
+Order of the parts as in utils/model.py:15-35.  The block keeps the reference's
+fused dataflow (utils/model.py:87-100): the residual stream and the update that
 is still to be added travel as a pair, so every "add, then normalise" is one kernel.
 """
 from __future__ import annotations

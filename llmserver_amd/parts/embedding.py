@@ -1,4 +1,4 @@
-"""Token embedding lookup ``h0 = E[ids]`` without scaling (/root/reference/utils/model.py:56-59,110)."""
+"""Token embedding lookup ``h0 = E[ids]`` without scaling (utils/model.py:56-59,110)."""
 from __future__ import annotations
 
 from .base import MATRIX, ParamSpec, Part

@@ -1,10 +1,10 @@
 """Linear projection ``y = x W^T (+ b)`` with ``W [out, in]`` as checkpoints store it.
 
 The matrix product itself is a library call, as in the reference's engine, which runs every
-projection through the vendor GEMM behind ``nn.Linear`` (/root/reference/utils/attention.py:33-37,
-/root/reference/utils/layers.py:188-191).  Several checkpoint matrices can be stacked along the
-output dimension into one product (/root/reference/utils/attention.py:54-66,
-/root/reference/utils/layers.py:194-203).
+projection through the vendor GEMM behind ``nn.Linear`` (utils/attention.py:33-37,
+utils/layers.py:188-191).  Several checkpoint matrices can be stacked along the
+output dimension into one product (utils/attention.py:54-66,
+utils/layers.py:194-203).
 """
 from __future__ import annotations
 

@@ -1,7 +1,7 @@
 """Gated feed-forward ``down(silu(gate(x)) * up(x))``.
 
-Gate and up are one stacked product, gate first (/root/reference/utils/layers.py:194-218;
-/root/reference/utils/fused_ops.py:59-61, 80-88).  Sigmoid and the product run in 32-bit inside
+Gate and up are one stacked product, gate first (utils/layers.py:194-218;
+utils/fused_ops.py:59-61, 80-88).  Sigmoid and the product run in 32-bit inside
 the activation kernel.
 """
 from __future__ import annotations

@@ -1,9 +1,9 @@
 """RMSNorm fused with the residual sum.
 
 ``y = s * rsqrt(mean(s^2) + eps) * w`` with ``s = resid + delta`` and everything in 32-bit inside
-(/root/reference/utils/layers.py:131-138; fused form /root/reference/utils/fused_ops.py:23-26,
+(utils/layers.py:131-138; fused form utils/fused_ops.py:23-26,
 65-78).  ``s`` is rounded to the activation dtype once, when it is stored back as the new
-residual stream (/root/reference/utils/fused_ops.py:73).
+residual stream (utils/fused_ops.py:73).
 """
 from __future__ import annotations
 

@@ -2,9 +2,9 @@
 
 ``inv_freq_i = theta^(-2i/d)`` for ``i = 0..d/2-1``, ``angle = position * inv_freq`` in 32-bit,
 ``x' = x*cos + rotate_half(x)*sin`` with ``rotate_half(x) = cat(-x[d/2:], x[:d/2])``
-(/root/reference/utils/layers.py:140-177).  Positions are absolute token positions
-(/root/reference/utils/batch.py:30,80).  The table of inverse frequencies is made once on the
-host with the reference's expression (/root/reference/utils/layers.py:158); the rotation itself
+(utils/layers.py:140-177).  Positions are absolute token positions
+(utils/batch.py:30,80).  The table of inverse frequencies is made once on the
+host with the reference's expression (utils/layers.py:158); the rotation itself
 happens inside the mixer's fused kernel, which gets the table and the positions of the step's
 tokens, so a position depends on nothing but the token's own index.
 """

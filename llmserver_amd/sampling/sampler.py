@@ -1,6 +1,6 @@
 """Greedy and temperature sampling over the step's float32 logits.
 
-The reference's engine samples with ``argmax`` only (/root/reference/utils/engine.py:295-297).
+The reference's engine samples with ``argmax`` only (utils/engine.py:295-297).
 Temperature sampling draws from ``softmax(logits / temperature)`` (computed in 32-bit) by
 inverting the cumulative distribution at a uniform number; the numbers come from a generator
 seeded per request, so a request's tokens do not depend on what shares its batch.

@@ -3,10 +3,10 @@
 Matrices follow the compute dtype (bfloat16 for serving, float32 on the 32-bit path); small
 per-channel vectors are held in float32, which keeps a vector stored in 32-bit as it is and
 widens a bfloat16 one without loss; integer tables become int32.  The reference loads each
-module strictly, so a missing or unexpected name raises (/root/reference/utils/model_loader.py:
+module strictly, so a missing or unexpected name raises (utils/model_loader.py:
 49-52); here every problem of the folder is collected first and reported in one error.  The
 output head is tied to the embedding when the configuration says so or the checkpoint has no
-head (/root/reference/utils/model_loader.py:56-59).
+head (utils/model_loader.py:56-59).
 """
 from __future__ import annotations
 

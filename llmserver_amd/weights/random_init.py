@@ -1,7 +1,7 @@
 """Seeded random weights: writes a model folder from a configuration and a seed.
 
 The reference's loader has no such mode; its tests seed a generator and draw every parameter
-from a normal distribution (/root/reference/tests/test_paged_decode.py:273-277).  Here each
+from a normal distribution (tests/test_paged_decode.py:273-277).  Here each
 tensor is drawn from a generator seeded by (seed, tensor name), so the values do not depend on
 the order of tensors: matrices ``N(0, std)``, norm weights ``1 + N(0, norm_noise)``, biases
 ``N(0, bias_std)``.

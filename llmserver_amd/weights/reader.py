@@ -1,6 +1,6 @@
 """Reads a model folder's safetensors files one tensor at a time, by tensor name.
 
-Same job as /root/reference/utils/weights.py:15-55: a folder holds either one
+Same job as utils/weights.py:15-55: a folder holds either one
 ``model.safetensors`` or shards listed in ``model.safetensors.index.json["weight_map"]``; files
 are memory-mapped and tensors handed out singly, so a large model never has a second full copy
 in host memory.  Only local folders are read (there is no download path).

@@ -26,25 +26,25 @@ def read_folder(folder, dtype=torch.float64):
 
 
 def head_dim_of(config):
-    """/root/reference/utils/architecture.py:88"""
+    """utils/architecture.py:88"""
     return config.get("head_dim") or config["hidden_size"] // config["num_attention_heads"]
 
 
 def rope_theta_of(config):
-    """/root/reference/utils/architecture.py:23-30"""
+    """utils/architecture.py:23-30"""
     parameters = config.get("rope_scaling") or config.get("rope_parameters") or {}
     theta = config.get("rope_theta")
     return parameters.get("rope_theta", 10000.0) if theta is None else theta
 
 
 def rms_norm(x, weight, eps):
-    """y = x * rsqrt(mean(x^2, last dim) + eps) * w  (/root/reference/utils/layers.py:133-138)."""
+    """y = x * rsqrt(mean(x^2, last dim) + eps) * w  (utils/layers.py:133-138)."""
     variance = x.pow(2).mean(dim=-1, keepdim=True)
     return weight * (x * torch.rsqrt(variance + eps))
 
 
 def inverse_frequencies(head_dim, theta, dtype=torch.float64):
-    """inv_freq_i = 1 / theta^(2i/d), i = 0..d/2-1  (/root/reference/utils/layers.py:145,158).
+    """inv_freq_i = 1 / theta^(2i/d), i = 0..d/2-1  (utils/layers.py:145,158).
 
     The reference evaluates this in float32; the float32 values are kept so that the oracle's
     angles are the ones the formula defines at the reference's precision of the table."""
@@ -57,7 +57,7 @@ ANGLE_DTYPE = torch.float32     # precision of pos * inv_freq, as in the referen
 
 
 def rope_cos_sin(positions, head_dim, theta, dtype=torch.float64, angle_dtype=None):
-    """angles = pos * inv_freq, duplicated over both halves  (/root/reference/utils/layers.py:160-164).
+    """angles = pos * inv_freq, duplicated over both halves  (utils/layers.py:160-164).
 
     The reference forms the product in float32 (line 160: ``pos_ids.to(torch.float32) * inv_freq``), and a
     float32 angle of a few thousand radians is up to 2e-4 away from the exact product: that rounding is
@@ -70,13 +70,13 @@ def rope_cos_sin(positions, head_dim, theta, dtype=torch.float64, angle_dtype=No
 
 
 def rotate_half(x):
-    """cat(-x[d/2:], x[:d/2])  (/root/reference/utils/layers.py:166-170)."""
+    """cat(-x[d/2:], x[:d/2])  (utils/layers.py:166-170)."""
     half = x.shape[-1] // 2
     return torch.cat([-x[..., half:], x[..., :half]], dim=-1)
 
 
 def apply_rope(x, cos, sin):
-    """x * cos + rotate_half(x) * sin; x [heads, seq, d], cos/sin [seq, d]  (/root/reference/utils/layers.py:172-177)."""
+    """x * cos + rotate_half(x) * sin; x [heads, seq, d], cos/sin [seq, d]  (utils/layers.py:172-177)."""
     return x * cos.unsqueeze(0) + rotate_half(x) * sin.unsqueeze(0)
 
 
@@ -84,8 +84,8 @@ def causal_attention(q, k, v, scale, window=None):
     """q [Hq, S, d], k/v [Hkv, S, d] -> [Hq, S, d].
 
     KV heads repeated per group, scores scaled, causal additive mask, softmax, times V
-    (/root/reference/utils/attention.py:188-198).  ``window`` (not in the reference, which refuses
-    sliding windows at /root/reference/utils/architecture.py:72-76) keeps for query p the keys
+    (utils/attention.py:188-198).  ``window`` (not in the reference, which refuses
+    sliding windows at utils/architecture.py:72-76) keeps for query p the keys
     p-window+1 .. p; None keeps all."""
     n_q, seq, _ = q.shape
     group = n_q // k.shape[0]
@@ -102,7 +102,7 @@ def causal_attention(q, k, v, scale, window=None):
 
 def attention_block(x, tensors, prefix, config, positions, window=None, kv_store=None, kv_from=None, cos_sin=None):
     """Projections, per-head q/k norm before the rotation, rotation, attention, output projection
-    (/root/reference/utils/attention.py:119-128, 155-159, 299-300).
+    (utils/attention.py:119-128, 155-159, 299-300).
 
     ``kv_store`` (a dict) receives this layer's rotated keys and values under ``prefix``;
     ``kv_from`` names a prefix whose stored keys and values are used instead of this layer's own
@@ -128,7 +128,7 @@ def attention_block(x, tensors, prefix, config, positions, window=None, kv_store
             k, v = kv_store[kv_from]
         else:
             kv_store[prefix] = (k, v)
-    out = causal_attention(q, k, v, d ** -0.5, window)           # /root/reference/utils/architecture.py:105
+    out = causal_attention(q, k, v, d ** -0.5, window)           # utils/architecture.py:105
     out = out.permute(1, 0, 2).reshape(seq, n_q * d)
     y = out @ tensors[f"{prefix}.o_proj.weight"].T
     bias = tensors.get(f"{prefix}.o_proj.bias")
@@ -136,14 +136,14 @@ def attention_block(x, tensors, prefix, config, positions, window=None, kv_store
 
 
 def swiglu_mlp(x, tensors, prefix):
-    """down(silu(gate(x)) * up(x))  (/root/reference/utils/layers.py:210-218)."""
+    """down(silu(gate(x)) * up(x))  (utils/layers.py:210-218)."""
     gate = x @ tensors[f"{prefix}.gate_proj.weight"].T
     up = x @ tensors[f"{prefix}.up_proj.weight"].T
     return (torch.nn.functional.silu(gate) * up) @ tensors[f"{prefix}.down_proj.weight"].T
 
 
 def decoder_layer(h, tensors, index, config, positions, window=None):
-    """h += attn(norm_in(h)); h += mlp(norm_post(h))  (/root/reference/utils/model.py:15-35)."""
+    """h += attn(norm_in(h)); h += mlp(norm_post(h))  (utils/model.py:15-35)."""
     prefix = f"model.layers.{index}"
     eps = config["rms_norm_eps"]
     h = h + attention_block(rms_norm(h, tensors[f"{prefix}.input_layernorm.weight"], eps), tensors,
@@ -153,8 +153,8 @@ def decoder_layer(h, tensors, index, config, positions, window=None):
 
 def forward(config, tensors, token_ids, windows=None, layer_order=None, first_position=0):
     """Logits ``[seq, vocab]`` at every position of one whole sequence
-    (/root/reference/utils/model.py:109-158 without cache; tied head rule
-    /root/reference/utils/model_loader.py:56-59).
+    (utils/model.py:109-158 without cache; tied head rule
+    utils/model_loader.py:56-59).
 
     ``windows`` (per layer) and ``layer_order`` (which layer runs when) serve the tests' toy
     arrangements; ``first_position`` shifts all positions."""
@@ -171,7 +171,7 @@ def forward(config, tensors, token_ids, windows=None, layer_order=None, first_po
 
 
 def greedy_generate(config, tensors, prompt, new_tokens):
-    """Argmax continuation, recomputing the whole sequence each step (/root/reference/utils/engine.py:295-297)."""
+    """Argmax continuation, recomputing the whole sequence each step (utils/engine.py:295-297)."""
     tokens = list(prompt)
     for _ in range(new_tokens):
         tokens.append(int(torch.argmax(forward(config, tensors, tokens)[-1])))

@@ -175,7 +175,7 @@ def test_random_model_command_writes_a_folder_that_loads_and_repeats(tmp_path):
 
 
 def test_benchmark_command_takes_the_reference_name_of_its_dtype_option(capsys):
-    """``--custom-dtype`` (/root/reference/benchmark.py:344): source and fp32 are other names of --dtype; fp16 is refused
+    """``--custom-dtype`` (benchmark.py:344): source and fp32 are other names of --dtype; fp16 is refused
     before anything is loaded."""
     from llmserver_amd.cli import benchmark
     with pytest.raises(SystemExit) as refused:

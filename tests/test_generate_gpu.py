@@ -248,3 +248,28 @@ def test_requests_arriving_over_time_with_shared_prefixes_and_few_pages(case, se
             preemptions += engine.step_profile["preemptions"]
             hits += engine.step_profile["prefix_hit_tokens"]
     assert hits > 0
+
+
+def test_calibrate_measures_only_when_asked_and_writes_a_table(tmp_path):
+    """Serving looks kernel choices up; ``Engine.calibrate`` is the one place that measures, and it leaves a file that a
+    later process can be pointed at."""
+    import json
+    from llmserver_amd import Engine, load_model
+    from llmserver_amd.kernels import default_ops
+    from llmserver_amd.kernels.choices import ChoiceTable
+    print("calibrate", flush=True)
+    ops = default_ops()
+    saved, ops.choices = ops.choices, ChoiceTable(ops.device_kind)
+    try:
+        model = load_model(model_folder("B"), "cuda", "bfloat16")
+        engine = Engine(model, None, max_new_tokens=4, max_batch_size=3, max_num_batched_tokens=64, kv_cache_num_blocks=64, kv_cache_block_size=8)
+        assert engine.generate([[1, 2, 3], [4, 5]]) and not ops.choices.entries       # generation measured nothing
+        path = str(tmp_path / "choices.json")
+        measured = engine.calibrate(save_to=path)
+        assert measured > 0 and len(ops.choices.measured) == measured and ops._flush is None
+        stored = json.load(open(path))
+        assert list(stored) == [ops.device_kind] and len(stored[ops.device_kind]) == measured
+        assert engine.generate([[1, 2, 3], [4, 5]])
+        assert engine.calibrate() == 0                                                # everything is known now
+    finally:
+        ops.choices = saved

@@ -173,3 +173,21 @@ def test_unusual_steps(dtype, tmp_path):
             fed.pop(name, None)
     if errors:
         check_bf16(errors, "unusual steps")
+
+
+def test_two_bfloat16_runs_write_the_same_bytes(tmp_path):
+    """Which kernel a shape goes through comes from a table, never from a stopwatch: a second process rounds as the first."""
+    case = "D"
+    vocab = CASES[case][0]["vocab_size"]
+    requests = {"a": random_tokens(vocab, 90, 3), "b": random_tokens(vocab, 40, 4)}
+    steps = traces.mixed(requests, seed=1, budget_tokens=192) + traces.tail_decoded({"c": random_tokens(vocab, 50, 5)}, 20)
+    for index, step in enumerate(steps):
+        step["step"] = index
+    outs = []
+    for run in range(2):
+        (tmp_path / str(run)).mkdir()
+        run_trace(case, "bfloat16", steps, tmp_path / str(run), 256, 16)
+        folder = tmp_path / str(run) / f"out-{case}-bfloat16"
+        outs.append({name: (folder / name).read_bytes() for name in sorted(os.listdir(folder))})
+    assert outs[0].keys() == outs[1].keys() and len(outs[0]) > 10
+    assert all(outs[0][name] == outs[1][name] for name in outs[0])
