@@ -602,21 +602,33 @@ constexpr int KPH = (K_HALF_PIECES + 255) / 256, VPH = (V_HALF_PIECES + 255) / 2
 // The host picks one or two per launch: two pay when the rows are long (the longest workgroup then does not
 // decide the time), one when they are short and there are few workgroups.
 constexpr int MAX_SUB = LSA_ND <= 8 ? 2 : 1;
+// Halves of a workgroup that split the keys between them (see the kernel): two where their buffers leave room in LDS for
+// more than one workgroup.
+constexpr int MAX_HALVES = LSA_ND <= 8 ? 2 : 1;
 // Wavefronts per SIMD wanted (they hide the latency of a step's dependent chain: LDS read, MFMA, softmax, MFMA),
 // as far as the registers of SUB tiles allow.
 #define LSA_TILE_MIN_WAVES(SUB) ((SUB) == 1 ? (LSA_ND <= 8 ? 3 : 1) : (LSA_ND <= 4 ? 3 : 2))
 struct FullStep { static constexpr bool value = true; };        // every key of the step is seen by every pair
 struct MaskedStep { static constexpr bool value = false; };
 
-template <int SUB>
-__global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_tile_kernel(
+// HALVES = 2: the workgroup has eight wavefronts; wavefronts 4 .. 7 take the same tiles as wavefronts 0 .. 3 and the
+// second half of the keys' steps, through LDS buffers of their own, and leave their running maximum, sum and
+// accumulators in LDS at the end, where the first four merge them by log-sum-exp.  The longest workgroup of a launch
+// (the tiles that see the most keys) then walks half as many steps: a launch with few workgroups, which that
+// workgroup bounds, ends sooner.  Both halves make the same number of trips through the loop (one of them may
+// have a step less to compute), so that they meet at the same barriers.
+template <int SUB, int HALVES>
+__global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_tile_kernel(
     const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
     const elem_t* __restrict__ keys, const elem_t* __restrict__ values,
     const int* __restrict__ table, int table_stride,
     const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
     const Item* __restrict__ tiles, Geometry g) {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2][K_TILE_BYTES + V_TILE_BYTES];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int STEP_BYTES = K_TILE_BYTES + V_TILE_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char lds_all[HALVES * 2 * STEP_BYTES];
+    const int half = HALVES > 1 ? (int)(threadIdx.x >> 8) : 0;
+    const int lds_base = half * 2 * STEP_BYTES;                       // this half's two buffers
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
     // Workgroups are handed to the eight XCDs in turn, and each XCD has its own L2: with the KV head
     // running fastest over the workgroup index, an XCD keeps meeting the same few KV heads, whose
     // keys and values then stay in its L2 for all the tiles that read them.
@@ -669,10 +681,16 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
         run_sum[u] = 0.f;
     }
 
-    const int k_begin = tile.k_begin, k_end = tile.k_end;
+    // The steps of 32 keys that cover the tile's keys, and this half's share of them: [k_begin, k_end).
+    const int first_step = (tile.k_begin / 32) * 32;
+    const int all_steps = tile.k_begin < tile.k_end ? (tile.k_end - 1 - first_step) / 32 + 1 : 0;
+    const int trips = (all_steps + HALVES - 1) / HALVES;              // of every wavefront through the loop below
+    const int cut = min(tile.k_end, first_step + 32 * trips);         // where the second half's keys begin
+    const int k_begin = half ? cut : tile.k_begin, k_end = half ? tile.k_end : cut;
+    const int my_steps = half ? all_steps - trips : trips;
     int chunk = -1, pages_cur = 0, pages_next = 0;
-    auto table_chunk = [&](int c) { return row_table[min(64 * c + lane, table_stride - 1)]; };
-    auto enter_chunk = [&](int kt) {
+    auto table_chunk = [&](int c) __attribute__((always_inline)) { return row_table[min(64 * c + lane, table_stride - 1)]; };
+    auto enter_chunk = [&](int kt) __attribute__((always_inline)) {
         const int c = (int)__umulhi((unsigned)kt, g.page_magic) >> 6;
         if (c != chunk) {
             pages_cur = (chunk >= 0 && c == chunk + 1) ? pages_next : table_chunk(c);
@@ -680,7 +698,7 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
             pages_next = table_chunk(c + 1);
         }
     };
-    auto locate = [&](int key, int& slot) {
+    auto locate = [&](int key, int& slot) __attribute__((always_inline)) {
         const int block = (int)__umulhi((unsigned)key, g.page_magic);
         slot = key - block * ps;
         return (size_t)__shfl(pages_cur, block - 64 * chunk, 64) * page_elems;
@@ -701,7 +719,7 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
         v_off[j] = 2u * (unsigned)((q >> 2) * ps + 4 * (q & 3));
     }
     const bool pages_of_16 = (ps & 15) == 0;        // then each half of a step (16 keys) lies inside one page
-    auto issue_loads = [&](Staged& r, int kt) {
+    auto issue_loads = [&](Staged& r, int kt) __attribute__((always_inline)) {
         enter_chunk(kt);
         if (pages_of_16 && kt >= k_begin && kt + 32 <= k_end) {
             // Interior step: one page lookup per half for the whole wavefront (scalar); every piece is then the
@@ -741,9 +759,9 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
             }
         }
     };
-    auto store_lds = [&](int buf, Staged& r, int kt) {
-        unsigned char* kl = lds[buf];
-        unsigned char* vl = lds[buf] + K_TILE_BYTES;
+    auto store_lds = [&](int buf, Staged& r, int kt) __attribute__((always_inline)) {
+        unsigned char* kl = lds_all + lds_base + buf * STEP_BYTES;
+        unsigned char* vl = kl + K_TILE_BYTES;
         const bool edge = kt < k_begin || kt + 32 > k_end;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -772,10 +790,10 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
     // Scores stay as the products left them; the scale (in units of ln 2, so that the exponential is one
     // instruction) goes into the multiply-add that also subtracts the running maximum.  FULL: every key of
     // the step is seen by every pair of the wavefront, nothing is masked.
-    auto compute_step = [&](auto full_tag, int buf, int kt) {
+    auto compute_step = [&](auto full_tag, int buf, int kt) __attribute__((always_inline)) {
         constexpr bool FULL = decltype(full_tag)::value;
-        const unsigned char* kl = lds[buf];
-        const unsigned char* vl = lds[buf] + K_TILE_BYTES;
+        const unsigned char* kl = lds_all + lds_base + buf * STEP_BYTES;
+        const unsigned char* vl = kl + K_TILE_BYTES;
         float sv[SUB][8];
         float tile_max[SUB];
 #pragma unroll
@@ -844,7 +862,7 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
             }
         }
     };
-    auto compute = [&](int buf, int kt) {
+    auto compute = [&](int buf, int kt) __attribute__((always_inline)) {
         if (kt >= wave_hi || kt + 32 <= wave_lo) return;          // nothing for this wavefront's pairs in this step
         // Steps every pair of the wavefront sees completely need no mask.
         const bool full = kt >= k_begin && kt + 32 <= k_end && kt + 31 <= q_pos_min && wave_tokens == SUB * g.tokens_per_tile &&
@@ -854,31 +872,86 @@ __global__ __launch_bounds__(256, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_
         else compute_step(MaskedStep{}, buf, kt);
     };
 
-    if (k_begin < k_end) {
+    if (all_steps > 0) {
         // Loads run two steps ahead of the products: while step i is multiplied out of one LDS
         // buffer, step i+1 sits in registers on its way to the other buffer and step i+2 is being
-        // fetched.  Loads are issued unconditionally (past the end they fetch the last step again),
-        // so that nothing between a load and its use makes the wait stricter than it has to be.
+        // fetched.  Loads are issued unconditionally (past the end they fetch the last step again; a half
+        // without keys fetches the step before its own), so that nothing between a load and its use makes the wait
+        // stricter than it has to be.  The trips through the loop are the same for every wavefront of the workgroup.
         Staged r0, r1;
-        int kt = (k_begin / 32) * 32;
-        const int last = ((k_end - 1) / 32) * 32;
+        int kt = half ? first_step + 32 * trips : first_step;
+        const int last = my_steps > 0 ? kt + 32 * (my_steps - 1) : max(first_step, kt - 32);
+        if (my_steps == 0) kt = last;
         issue_loads(r0, kt);
         issue_loads(r1, min(kt + 32, last));
         store_lds(0, r0, kt);
         __syncthreads();
+        int trip = 0;
         while (true) {
             issue_loads(r0, min(kt + 64, last));
-            compute(0, kt);
-            if (kt + 32 > last) break;
+            if (trip < my_steps) compute(0, kt);
+            if (trip + 1 >= trips) break;
             store_lds(1, r1, kt + 32);
             __syncthreads();
             issue_loads(r1, min(kt + 96, last));
-            compute(1, kt + 32);
-            if (kt + 64 > last) break;
+            if (trip + 1 < my_steps) compute(1, kt + 32);
+            if (trip + 2 >= trips) break;
             store_lds(0, r0, kt + 64);
             __syncthreads();
             kt += 64;
+            trip += 2;
         }
+    }
+    if constexpr (HALVES > 1) {
+        // The second half's wavefronts hand over what they have; the first half's add it to theirs.  The buffers
+        // of keys and values are free once everybody has passed the barrier.
+        __syncthreads();
+        float* handed = reinterpret_cast<float*>(lds_all);
+        constexpr int PER_WAVE = SUB * (ND * 256 + 32);               // floats: accumulators (ND x 64 lanes x 4), then max and sum of 16 pairs
+        static_assert(4 * PER_WAVE * sizeof(float) <= sizeof(lds_all), "the buffers of keys and values hold what the second half hands over");
+        float* mine = handed + (size_t)wave * PER_WAVE;
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) {
+            float total = run_sum[u];
+            total += __shfl_xor(total, 16, 64);
+            total += __shfl_xor(total, 32, 64);
+            run_sum[u] = total;                                       // the pair's whole sum, in every lane of the pair
+        }
+        if (half) {
+#pragma unroll
+            for (int u = 0; u < SUB; ++u) {
+                float* block = mine + u * (ND * 256 + 32);
+#pragma unroll
+                for (int c = 0; c < ND; ++c) *reinterpret_cast<f32x4*>(block + (c * 64 + lane) * 4) = acc[u][c];
+                if (quad == 0) {
+                    block[ND * 256 + col] = run_max[u];
+                    block[ND * 256 + 16 + col] = run_sum[u];
+                }
+            }
+        }
+        __syncthreads();
+        if (half) return;
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) {
+            const float* block = mine + u * (ND * 256 + 32);
+            const float other_max = block[ND * 256 + col], other_sum = block[ND * 256 + 16 + col];
+            const float top = fmaxf(run_max[u], other_max);
+            const float w0 = run_max[u] == NEG_INF ? 0.f : __builtin_amdgcn_exp2f((run_max[u] - top) * scale_log2);
+            const float w1 = other_max == NEG_INF ? 0.f : __builtin_amdgcn_exp2f((other_max - top) * scale_log2);
+            const float total = w0 * run_sum[u] + w1 * other_sum;
+            if (!pair_valid[u]) continue;
+            const float inv = total > 0.f ? 1.f / total : 0.f;
+            elem_t* o = out + ((size_t)(row_start[row] + q0 + u * g.tokens_per_tile + pair_token) * g.n_q + head) * D + 4 * quad;
+#pragma unroll
+            for (int c = 0; c < ND; ++c) {
+                const f32x4 other = *reinterpret_cast<const f32x4*>(block + (c * 64 + lane) * 4);
+                bf16x4 r4;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) r4[r] = (bf16_t)((acc[u][c][r] * w0 + other[r] * w1) * inv);
+                *reinterpret_cast<bf16x4*>(o + 16 * c) = r4;
+            }
+        }
+        return;
     }
 #pragma unroll
     for (int u = 0; u < SUB; ++u) {
@@ -1018,7 +1091,7 @@ LSA_EXPORT int lsa_paged_attention(
     const void* merges, int n_merges, int n_slots, float* part_acc, float* part_ml, const void* tiles, int n_tiles, float scale,
     int window, int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
     int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, int tiles_per_workgroup,
-    int merge_in_workgroup, hipStream_t stream) {
+    int merge_in_workgroup, int tile_halves, hipStream_t stream) {
     if (n_items <= 0 && n_tiles <= 0) return 0;
     // decode_fusion (see DecodeFusion::mode): the caller promises that every row of the step brings one token.
     DecodeFusion fusion = {q_weight, k_weight, cos_sin, norm_eps, decode_fusion};
@@ -1033,14 +1106,15 @@ LSA_EXPORT int lsa_paged_attention(
         // The plan's entries of `tiles` span what a workgroup takes: 4 or 8 tiles.
         if (tiles_per_workgroup != 4 && tiles_per_workgroup != 4 * MAX_SUB) return -1;
         dim3 tgrid(n_tiles * n_kv * gtiles);
-        if (tiles_per_workgroup == 4)
-            paged_attention_tile_kernel<1><<<tgrid, 256, 0, stream>>>(
-                (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
-                row_start, row_len, row_ctx, (const Item*)tiles, g);
-        else
-            paged_attention_tile_kernel<MAX_SUB><<<tgrid, 256, 0, stream>>>(
-                (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
-                row_start, row_len, row_ctx, (const Item*)tiles, g);
+        if (tile_halves != 1 && tile_halves != MAX_HALVES) return -1;
+#define LSA_LAUNCH_TILES(SUB, HALVES) paged_attention_tile_kernel<SUB, HALVES><<<tgrid, 256 * HALVES, 0, stream>>>( \
+                (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride, \
+                row_start, row_len, row_ctx, (const Item*)tiles, g)
+        if (tiles_per_workgroup == 4 && tile_halves == 1) LSA_LAUNCH_TILES(1, 1);
+        else if (tiles_per_workgroup == 4) LSA_LAUNCH_TILES(1, MAX_HALVES);
+        else if (tile_halves == 1) LSA_LAUNCH_TILES(MAX_SUB, 1);
+        else LSA_LAUNCH_TILES(MAX_SUB, MAX_HALVES);
+#undef LSA_LAUNCH_TILES
         const int terr = (int)hipGetLastError();
         if (terr) return terr;
 #else
@@ -1095,6 +1169,14 @@ LSA_EXPORT int lsa_attention_workgroup_tiles() {
     return 4 * MAX_SUB;
 #else
     return 0;
+#endif
+}
+// Halves that a workgroup of the prompt-portion kernel can split a tile's keys between (1: it cannot).
+LSA_EXPORT int lsa_attention_tile_halves() {
+#if LSA_BF16
+    return MAX_HALVES;
+#else
+    return 1;
 #endif
 }
 // Most key ranges a tile's keys may be split into (the merge takes no more slots per tile).

@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import torch
 
-from ..parts.attention import AttentionTuning, group_tiling
+from ..parts.attention import AttentionTuning, TileLaunchCost, group_tiling
 from . import build, library
 from .choices import ChoiceTable, choice_key
 
@@ -97,13 +97,15 @@ class HipOps:
     @property
     def attention_tuning(self) -> AttentionTuning:
         """What the attention plan should know of this GPU: four wavefronts in flight per compute unit (more and shorter
-        key ranges cost more in the merge than they gain), and what a 32-key step of the prompt-portion kernel
-        costs with four and with eight tiles to a workgroup (measured on an MI355X: with every compute unit busy 2.0 ns
-        per tile-row against 2.75 ns for twice the tiles; alone on the chip 1.37 against 1.40 us a step)."""
+        key ranges cost more in the merge than they gain), and what the prompt-portion kernel costs in each of its four
+        forms (measured on an MI355X at head size 128: a launch of one prompt of 512 to 4,096 tokens, of several, and of
+        portions behind long prefixes; eight tiles to a workgroup do more with each key they load but start later, two
+        halves shorten the longest workgroup's walk but make every step dearer)."""
         if self._tuning is None:
             units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-            self._tuning = AttentionTuning(target_waves=4 * units, step_ns_four_tiles=2.0, step_ns_most_tiles=2.75,
-                                           lone_step_us_four_tiles=1.37, lone_step_us_most_tiles=1.40)
+            costs = (((False, 1), TileLaunchCost(3.2, 1.16, 2.0)), ((True, 1), TileLaunchCost(8.7, 1.16, 2.75)),
+                     ((False, 2), TileLaunchCost(3.3, 1.7, 2.42)), ((True, 2), TileLaunchCost(8.8, 1.7, 3.38)))
+            self._tuning = AttentionTuning(target_waves=4 * units, tile_costs=costs)
         return self._tuning
 
     @staticmethod
@@ -547,6 +549,10 @@ class HipOps:
         (what an entry of a plan's ``tiles`` must span), or 0 if this type has no such kernel."""
         return int(self._attention_library(dtype, head_dim).lsa_attention_workgroup_tiles())
 
+    def attention_tile_halves(self, dtype, head_dim) -> int:
+        """Halves that a workgroup of the prompt-portion kernel can split its tiles' keys between (1: it cannot)."""
+        return int(self._attention_library(dtype, head_dim).lsa_attention_tile_halves())
+
     @staticmethod
     def decode_fusion_fits(dtype, head_dim) -> bool:
         """Whether the attention kernel can take the q/k norm, the rotation and the new token's way into the cache
@@ -615,6 +621,8 @@ class HipOps:
             raise ValueError("merging in the workgroup takes steps of one token per row whose plan gives every tile four key ranges "
                              "(or two, with tiles in pairs) and no slots, and, with decode fusion, both norm weights and a rotation")
         lib = self._attention_library(qkv.dtype, head_dim)
+        if n_tiles and int(plan.get("tile_halves", 1)) not in (1, lib.lsa_attention_tile_halves()):
+            raise ValueError(f"the plan splits a workgroup's keys into {plan['tile_halves']} halves, this kernel takes 1 or {lib.lsa_attention_tile_halves()}")
         if plan.get("most_splits", 0) > lib.lsa_attention_most_splits():
             raise ValueError(f"the plan splits a tile's keys into {plan['most_splits']} ranges, the merge kernel takes {lib.lsa_attention_most_splits()}")
         _launched(lib.lsa_paged_attention(
@@ -622,7 +630,8 @@ class HipOps:
             _ptr(row_len), _ptr(row_ctx), _ptr(plan["items"]), _ptr(plan["item_slot"]), n_items, _ptr(plan["merges"]),
             n_merges, n_slots, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), n_tiles, float(scale), int(window) if window else 0,
             page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, fusion_mode, _ptr(q_weight), _ptr(k_weight), float(norm_eps),
-            _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), merge_in_workgroup, _stream()), "paged_attention")
+            _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), merge_in_workgroup, int(plan.get("tile_halves", 1)), _stream()),
+            "paged_attention")
 
     def sample(self, logits, temperature, uniform, out):
         n, vocab = logits.shape

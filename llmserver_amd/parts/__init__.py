@@ -1,4 +1,4 @@
-from .attention import AttentionNames, AttentionPlan, AttentionTuning, GQAttention, build_attention_plan, group_tiling
+from .attention import AttentionNames, AttentionPlan, AttentionTuning, GQAttention, TileLaunchCost, build_attention_plan, group_tiling
 from .base import (INT_TABLE, MATRIX, VECTOR, Block, FeedForward, Mixer, Norm, PagedKVSpec, ParamSpec, Part,
                    PositionEncoding, StateSpec)
 from .block import PreNormBlock
@@ -8,7 +8,7 @@ from .mlp import GatedMLP, GatedMLPNames
 from .norm import RMSNorm
 from .rope import NoPosition, RotaryPosition
 
-__all__ = ["AttentionNames", "AttentionTuning", "GatedMLPNames", "AttentionPlan", "GQAttention", "build_attention_plan", "group_tiling", "INT_TABLE", "MATRIX", "VECTOR",
+__all__ = ["AttentionNames", "AttentionTuning", "TileLaunchCost", "GatedMLPNames", "AttentionPlan", "GQAttention", "build_attention_plan", "group_tiling", "INT_TABLE", "MATRIX", "VECTOR",
            "Block", "FeedForward", "Mixer", "Norm", "PagedKVSpec", "ParamSpec", "Part", "PositionEncoding",
            "StateSpec", "PreNormBlock", "TokenEmbedding", "Linear", "GatedMLP", "RMSNorm", "NoPosition",
            "RotaryPosition"]

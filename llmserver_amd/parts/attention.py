@@ -35,20 +35,31 @@ MIN_KEYS_PER_SPLIT = 64     # shorter key ranges than this are not worth a wavef
 
 
 @dataclasses.dataclass(frozen=True)
+class TileLaunchCost:
+    """What one way of launching the prompt-portion kernel costs: microseconds of start and end, microseconds of one
+    trip of a workgroup through its loop (32 keys; a workgroup makes its trips one after the other, so its longest
+    workgroup bounds a launch), and nanoseconds of one 32-key step of one workgroup per KV head when every compute
+    unit is busy (the work of all workgroups together bounds a launch, too)."""
+    start_us: float = 4.0
+    trip_us: float = 1.0
+    step_ns: float = 1.0
+
+
+@dataclasses.dataclass(frozen=True)
 class AttentionTuning:
     """What the plan needs to know of the machine and its kernels; the kernel namespace of a step supplies it
     (``ops.attention_tuning``), these defaults stand where it does not.
 
     ``target_waves``: wavefronts wanted in flight; rows with few tokens and long contexts are cut into key ranges
-    until there are about that many.  The other four describe the prompt-portion kernel, whose workgroups take four
-    tiles or ``most`` tiles: nanoseconds of a 32-key step per tile-row when every compute unit is busy, and
-    microseconds of such a step when a workgroup has the machine to itself (then the longest workgroup bounds the
-    launch)."""
+    until there are about that many.  ``tile_costs``: the prompt-portion kernel's workgroups take four tiles or the
+    most the kernel offers, and walk their keys whole or in two halves side by side; the costs of each of these
+    ways, keyed by (takes the most tiles, halves)."""
     target_waves: int = 1024
-    step_ns_four_tiles: float = 1.0
-    step_ns_most_tiles: float = 1.0
-    lone_step_us_four_tiles: float = 1.0
-    lone_step_us_most_tiles: float = 1.0
+    tile_costs: Tuple[Tuple[Tuple[bool, int], TileLaunchCost], ...] = (
+        ((False, 1), TileLaunchCost()), ((True, 1), TileLaunchCost()), ((False, 2), TileLaunchCost()), ((True, 2), TileLaunchCost()))
+
+    def tile_cost(self, takes_most: bool, halves: int) -> TileLaunchCost:
+        return dict(self.tile_costs).get((bool(takes_most), int(halves)), TileLaunchCost())
 
 
 DEFAULT_TUNING = AttentionTuning()
@@ -81,13 +92,14 @@ class AttentionPlan:
     ``merges [n_merges, 4] int32``: row, first token of the tile, first slot, number of slots.
     ``tiles [n_tiles, 4] int32``: row, first token, first key, one past the last key of
     ``tiles_per_workgroup`` (4 or 8) consecutive tiles that one workgroup handles together, sharing
-    the keys it loads.
+    the keys it loads (in ``tile_halves`` halves of its wavefronts, each on its share of the keys).
     """
 
-    def __init__(self, items, item_slot, merges, n_slots, tiles=None, tiles_per_workgroup=0):
+    def __init__(self, items, item_slot, merges, n_slots, tiles=None, tiles_per_workgroup=0, tile_halves=1):
         self.items, self.item_slot, self.merges, self.n_slots = items, item_slot, merges, n_slots
         self.tiles = tiles if tiles is not None else np.zeros((0, 4), dtype=np.int32)
         self.tiles_per_workgroup = tiles_per_workgroup
+        self.tile_halves = tile_halves       # 2: the workgroups of ``tiles`` walk their keys in two halves side by side
         self.merge_in_workgroup = 0          # 4: items 4 i .. 4 i + 3 are one tile's key ranges, merged by their workgroup;
                                              # 2: they are the two ranges of each of two tiles
 
@@ -105,16 +117,17 @@ MIN_TILES_FOR_WORKGROUPS = 16      # rows with at least this many tiles go to th
 
 
 def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, heads, window, most: int,
-                              tuning: AttentionTuning = DEFAULT_TUNING) -> int:
-    """4 or ``most`` tiles per workgroup of the prompt-portion kernel, whichever the step's rows finish sooner with.
+                              tuning: AttentionTuning = DEFAULT_TUNING, most_halves: int = 1):
+    """``(tiles per workgroup, halves)`` of the prompt-portion kernel that the step's rows finish soonest with: 4 or
+    ``most`` tiles, the keys of a workgroup walked whole or, where the kernel can, in two halves side by side.
 
-    A workgroup walks its keys in steps of 32.  With all compute units busy, more tiles per workgroup get more out of
-    every step (setting up and draining a workgroup costs about 8 steps more), but a step of theirs takes longer, and
-    the workgroup with the most steps bounds the launch from below: one short prompt finishes sooner with four, long
-    rows and many rows with ``most``.  The costs of a step are the tuning's."""
-    if most <= 4:
-        return most
-    def estimate(per_workgroup, ns_per_step, us_per_step_alone):
+    A workgroup walks its keys in steps of 32.  More tiles per workgroup get more out of every step (setting up and
+    draining a workgroup costs about 8 steps more), and two halves halve the trips of the longest workgroup, which
+    bounds a launch of few workgroups from below; but steps of larger workgroups take longer, which is what counts
+    when every compute unit is busy.  Each way is priced with the tuning's costs: start, then the longest
+    workgroup's trips and all workgroups' steps, whichever is more (blended, since both slow each other down)."""
+    def estimate(per_workgroup, halves):
+        cost = tuning.tile_cost(per_workgroup > 4, halves)
         span = per_workgroup * tokens_per_tile
         total = longest = 0
         for row in range(len(row_len)):
@@ -127,9 +140,10 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
             steps = -(-(k_end - k_begin) // 32)
             total += int(steps.sum()) + 8 * len(steps)
             longest = max(longest, int(steps.max()))
-        return max(total * heads * ns_per_step * 1e-3, longest * us_per_step_alone)
-    return most if estimate(most, tuning.step_ns_most_tiles, tuning.lone_step_us_most_tiles) \
-        < estimate(4, tuning.step_ns_four_tiles, tuning.lone_step_us_four_tiles) else 4
+        path, work = -(-longest // halves) * cost.trip_us, total * heads * cost.step_ns * 1e-3
+        return cost.start_us + (path ** 4 + work ** 4) ** 0.25
+    ways = [(per, halves) for halves in sorted({1, max(1, int(most_halves))}) for per in sorted({min(4, most), most})]
+    return min(ways, key=lambda way: (estimate(*way), way[1], way[0]))
 
 
 WORKGROUP_RANGES = 4    # key ranges of a tile that one workgroup (four wavefronts) walks and merges itself
@@ -171,13 +185,14 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, 
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
                          workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: int = 0,
-                         tuning: AttentionTuning = DEFAULT_TUNING) -> AttentionPlan:
+                         tuning: AttentionTuning = DEFAULT_TUNING, tile_halves: int = 1) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
     arrays have the same shape whatever the contexts are.  With ``workgroup_tiles`` (the number of tiles a
     workgroup of that kernel takes, which the kernel library tells) rows with many tiles (portions of prompts) go
-    to the kernel in which the tiles of a workgroup share the keys they load."""
+    to the kernel in which the tiles of a workgroup share the keys they load; ``tile_halves`` says whether that kernel
+    can split a workgroup's keys between two halves of its wavefronts (2) or not (1)."""
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
@@ -193,8 +208,11 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
     items, slots, merges, tiles = [], [], [], []
     n_slots = 0
-    per_workgroup = _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window,
-                                              int(workgroup_tiles), tuning) if workgroup_tiles and fixed_splits is None else 0
+    per_workgroup, halves = 0, 1
+    if workgroup_tiles and fixed_splits is None:
+        chosen = _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window,
+                                           int(workgroup_tiles), tuning, int(tile_halves))
+        per_workgroup, halves = chosen if isinstance(chosen, tuple) else (chosen, 1)
     for row in range(len(row_len)):
         n, ctx = int(row_len[row]), int(row_ctx[row])
         first_pos = ctx - n
@@ -236,7 +254,8 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     merges = np.asarray(merges, dtype=np.int32).reshape(-1, 4)
     tiles.sort(key=lambda tile: tile[2] - tile[3])       # most keys first: the long tiles must not start last
     tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 4)
-    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, tiles, per_workgroup if len(tiles) else 0)
+    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, tiles, per_workgroup if len(tiles) else 0,
+                         halves if len(tiles) else 1)
 
 
 class GQAttention(Mixer):
@@ -316,13 +335,16 @@ class GQAttention(Mixer):
                 in_workgroup = fixed
         per_workgroup = getattr(ctx.ops, "attention_workgroup_tiles", None)
         per_workgroup = per_workgroup(ctx.dtype, self.head_dim) if per_workgroup is not None else 0
+        halves = getattr(ctx.ops, "attention_tile_halves", None)
+        halves = halves(ctx.dtype, self.head_dim) if halves is not None and per_workgroup else 1
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
                                     target_waves=tuning.target_waves, fixed_splits=fixed, workgroup_tiles=per_workgroup,
-                                    merge_in_workgroup=in_workgroup, tuning=tuning)
+                                    merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves)
         ctx.set_plan(key, {
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
             "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),
-            "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup, "merge_in_workgroup": int(plan.merge_in_workgroup),
+            "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup, "tile_halves": int(plan.tile_halves),
+            "merge_in_workgroup": int(plan.merge_in_workgroup),
             "most_splits": int(plan.merges[:, 3].max()) if len(plan.merges) else 0,
         })
 

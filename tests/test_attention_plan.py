@@ -134,16 +134,24 @@ def test_plan_whose_key_ranges_are_merged_in_the_workgroup(seed):
         assert [(b, e) for _, _, b, e in ranges][len(filled):] == [(context, context)] * (per_tile - len(filled))
 
 
-def test_four_or_eight_tiles_per_workgroup():
-    """One short prompt is bounded by its longest workgroup and takes four tiles per workgroup; long rows and many rows
-    keep every compute unit busy and take eight; a kernel that offers only four gets four."""
-    def chosen(lens, ctxs, most=8):
-        return build_attention_plan(lens, ctxs, 4, 8, None, workgroup_tiles=most).tiles_per_workgroup
-    assert chosen([2048], [2048]) == 4
-    assert chosen([1024], [1024]) == 4
-    assert chosen([4096], [4096]) == 8
-    assert chosen([2048], [32768]) == 8
-    assert chosen([512] * 16, [512] * 16) == 8
-    assert chosen([4096], [4096], most=4) == 4
-    assert chosen([1] * 8, [4096] * 8) == 0                                  # no row has enough tiles
+def test_four_or_eight_tiles_per_workgroup_whole_or_in_halves():
+    """With the costs measured on an MI355X: one prompt is bounded by its longest workgroup, whose walk two halves
+    shorten (eight tiles at 2,048 tokens, four below); long rows and many rows keep every compute unit busy and take eight
+    tiles and no halves; a kernel that offers only four tiles, or no halves, gets what it offers."""
+    from llmserver_amd.parts import AttentionTuning, TileLaunchCost
+    tuning = AttentionTuning(1024, (((False, 1), TileLaunchCost(3.2, 1.16, 2.0)), ((True, 1), TileLaunchCost(8.7, 1.16, 2.75)),
+                                    ((False, 2), TileLaunchCost(3.3, 1.7, 2.42)), ((True, 2), TileLaunchCost(8.8, 1.7, 3.38))))
+
+    def chosen(lens, ctxs, most=8, halves=2):
+        plan = build_attention_plan(lens, ctxs, 4, 8, None, workgroup_tiles=most, tuning=tuning, tile_halves=halves)
+        return plan.tiles_per_workgroup, plan.tile_halves
+    assert chosen([2048], [2048]) == (8, 2)
+    assert chosen([1024], [1024]) == (4, 2)
+    assert chosen([512], [2560]) == (4, 2)                                   # a portion behind a prefix
+    assert chosen([4096], [4096]) == (8, 1)
+    assert chosen([2048], [32768]) == (8, 1)
+    assert chosen([512] * 16, [512] * 16) == (8, 1)
+    assert chosen([1024], [1024], halves=1) == (4, 1)                        # a kernel without halves
+    assert chosen([4096], [4096], most=4) == (4, 1)
+    assert chosen([1] * 8, [4096] * 8) == (0, 1)                             # no row has enough tiles
     assert build_attention_plan([4096], [4096], 4, 8, None).tiles_per_workgroup == 0

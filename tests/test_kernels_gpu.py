@@ -138,7 +138,7 @@ def test_qk_norm_rope_kv_write(ops, dtype, n_q, n_kv, d, page):
 
 
 def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, needle=True, seed=0, target_waves=None, workgroup_tiles=None,
-                   merge_in_workgroup=False):
+                   merge_in_workgroup=False, tile_halves=1):
     """Random q/k/v through both implementations.  Pages are handed out in scrambled order from a
     pool that first held other data (as if used before).  With ``needle``, one far key per request
     is made to dominate its first query's softmax."""
@@ -176,19 +176,20 @@ def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, need
     from llmserver_amd.parts import attention as attention_module
     most = ops.attention_workgroup_tiles(dtype, d) if workgroup_tiles is None or workgroup_tiles else 0
     chooser = attention_module._workgroup_tiles_that_pay
+    most_halves = ops.attention_tile_halves(dtype, d) if most else 1
     if workgroup_tiles:
-        assert workgroup_tiles <= most
-        attention_module._workgroup_tiles_that_pay = lambda *args, **kwargs: workgroup_tiles
+        assert workgroup_tiles <= most and tile_halves <= most_halves
+        attention_module._workgroup_tiles_that_pay = lambda *args, **kwargs: (workgroup_tiles, tile_halves)
     try:
         plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, workgroup_tiles=0 if merge_in_workgroup else most,
-                                    merge_in_workgroup=merge_in_workgroup,
+                                    merge_in_workgroup=merge_in_workgroup, tile_halves=most_halves, tuning=ops.attention_tuning,
                                     **({} if target_waves is None else {"target_waves": target_waves}))
     finally:
         attention_module._workgroup_tiles_that_pay = chooser
     staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
               "merges": torch.from_numpy(plan.merges).to(DEV), "tiles": torch.from_numpy(plan.tiles).to(DEV), "n_tiles": len(plan.tiles),
               "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup,
-              "merge_in_workgroup": int(plan.merge_in_workgroup)}
+              "tile_halves": plan.tile_halves, "merge_in_workgroup": int(plan.merge_in_workgroup)}
     t = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
     got = torch.zeros(tokens, n_q * d, device=DEV, dtype=dtype)
     ref = torch.zeros_like(got)
@@ -353,10 +354,11 @@ def test_attention_prompt_portions_in_workgroup_tiles(ops, n_q, n_kv, d, page, w
     assert len(plan.tiles) > 0 and len(plan.items) > 0
     attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d, workgroup_tiles=0)
     for per_workgroup in (4, 8):                                   # one and two tiles per wavefront
-        if per_workgroup <= ops.attention_workgroup_tiles(torch.bfloat16, d):
-            plan, _ = attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d,
-                                     workgroup_tiles=per_workgroup)
-            assert plan.tiles_per_workgroup == per_workgroup and len(plan.tiles) > 0
+        for halves in (1, 2):                                      # the keys of a workgroup whole, or in two halves of its wavefronts
+            if per_workgroup <= ops.attention_workgroup_tiles(torch.bfloat16, d) and halves <= ops.attention_tile_halves(torch.bfloat16, d):
+                plan, _ = attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d,
+                                         workgroup_tiles=per_workgroup, tile_halves=halves)
+                assert (plan.tiles_per_workgroup, plan.tile_halves) == (per_workgroup, halves) and len(plan.tiles) > 0
 
 
 def test_attention_refuses_sizes_it_cannot_take(ops):
