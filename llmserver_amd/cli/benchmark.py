@@ -96,6 +96,67 @@ def mixed_workload(engine, vocab, requests, low, high, shared_prefix_tokens, sha
             "preemptions": engine.step_profile["preemptions"]}
 
 
+def profile_engine(engine, vocab, prompt_lengths, batches, seed, out_path) -> None:
+    """Kernel tables of a few decode steps (one row and the largest batch, replayed from graphs and launched one by
+    one) and of prefills (the shortest prompts at the largest batch, the longest at up to eight), with the steps'
+    wall-clock times beside them, written to ``out_path``: what the reference's ``--profile`` writes
+    (benchmark_cuda.py:255-330 there)."""
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+
+    def kernel_table(run):
+        with profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA]) as trace:
+            run()
+            torch.cuda.synchronize()
+        return trace.key_averages().table(sort_by="cuda_time_total", row_limit=25, max_name_column_width=70)
+
+    def steps(count):
+        for _ in range(count):
+            engine.step()
+        torch.cuda.synchronize()
+
+    lines = []
+    graphs_possible = engine.runner.use_graphs
+    for batch in sorted({1, max(batches)}):
+        for graphs in ((False, True) if graphs_possible else (False,)):
+            engine.runner.use_graphs = graphs
+            engine.runner.drop_graphs()
+            prompts = build_prompts(vocab, min(prompt_lengths), batch, f"profile-{batch}-{graphs}", seed)
+            requests = [engine.add_request(None, prompt_token_ids=prompt, max_new_tokens=64) for prompt in prompts]
+            steps(4)                                        # the prompts, then a few decoding steps (graphs are captured here)
+            start = time.perf_counter()
+            steps(5)
+            step_ms = (time.perf_counter() - start) / 5 * 1000
+            lines.append(f"===== decode batch={batch} graphs={graphs}: {step_ms:.3f} ms a step =====")
+            lines.append(kernel_table(lambda: steps(5)))
+            for request in requests:
+                engine.cancel_request(request.request_id)
+    engine.runner.use_graphs = graphs_possible
+    engine.runner.drop_graphs()
+    for prompt_length, batch in {(min(prompt_lengths), max(batches)), (max(prompt_lengths), min(8, max(batches)))}:
+        def prefill(tag):
+            prompts = build_prompts(vocab, prompt_length, batch, f"{tag}-{prompt_length}-{batch}", seed)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for prompt in prompts:
+                engine.add_request(None, prompt_token_ids=prompt, max_new_tokens=1)
+            t1 = time.perf_counter()
+            count = 1
+            while engine.step():
+                count += 1
+            torch.cuda.synchronize()
+            return t1 - t0, time.perf_counter() - t1, count
+        prefill("profile-warm")
+        added, stepped, count = prefill("profile-timed")
+        lines.append(f"===== prefill prompt={prompt_length} batch={batch}: add_request x{batch} {added * 1000:.1f} ms + {count} engine steps {stepped * 1000:.1f} ms =====")
+        lines.append(kernel_table(lambda: prefill("profile-traced")))
+    lines.append("===== step profile =====")
+    lines.append(json.dumps(engine.step_profile))
+    with open(out_path, "w") as handle:
+        handle.write("\n".join(lines) + "\n")
+    print(f"kernel tables written to {out_path}", flush=True)
+
+
 def one_prompt(args, model, load_seconds) -> int:
     """One prompt, ``--repeats`` fresh requests: the reference's single-prompt statistics
     (benchmark.py:68-88)."""
@@ -181,7 +242,9 @@ def main(argv=None) -> int:
     parser.add_argument("--shared-prefix-tokens", type=int, default=512, help="length of the prefix that some mixed requests share")
     parser.add_argument("--shared-fraction", type=float, default=0.5, help="fraction of mixed requests that start with the shared prefix")
     parser.add_argument("--max-batch-size", type=int, default=None, help="requests running at a time (default: the largest batch)")
-    parser.add_argument("--profile", action="store_true", help="print the engine's per-phase step counters")
+    parser.add_argument("--profile", action="store_true",
+                        help="print the engine's per-phase step counters and write kernel tables of decode steps and prefills to --profile-out")
+    parser.add_argument("--profile-out", default="profile_kernels.txt", help="where --profile writes its kernel tables")
     parser.add_argument("--json", default=None, help="write the results to this file")
     args = parser.parse_args(argv)
     if (args.model is None) == (args.random_config is None):
@@ -266,6 +329,8 @@ def main(argv=None) -> int:
             results.append(entry)
     if args.profile:
         print("step profile:", json.dumps(engine.step_profile), flush=True)
+        engine.max_new_tokens = 64
+        profile_engine(engine, vocab, prompt_lengths or [high], batches, args.seed, args.profile_out)
     report = {"model": model.name, "dtype": args.dtype, "block_size": args.block_size, "kv_blocks": wanted, "gpu": torch.cuda.get_device_name(0),
               "torch": torch.__version__, "results": results, "step_profile": engine.step_profile}
     if args.json:

@@ -35,6 +35,10 @@ def test_matrix_one_prompt_and_mixed_workload(tmp_path, capsys):
     assert "Prompt tokens: 7 | Generated tokens: 5" in printed and "Time to first token:" in printed and "median decode throughput:" in printed
     assert benchmark.main(["--model", folder, "--prompt", "text without a tokenizer"]) == 2
     assert benchmark.main(["--random-config", "tiny-b", "--mixed-requests", "6", "--mixed-prompt-range", "4,40", "--shared-prefix-tokens", "16",
-                           "--output-tokens", "5", "--block-size", "8", "--max-num-batched-tokens", "64", "--profile"]) == 0
+                           "--output-tokens", "5", "--block-size", "8", "--max-num-batched-tokens", "64", "--profile",
+                           "--profile-out", str(tmp_path / "kernels.txt")]) == 0
     printed = capsys.readouterr().out
-    assert "mixed: 6 requests" in printed and "step profile:" in printed
+    assert "mixed: 6 requests" in printed and "step profile:" in printed and "decode_by_rows" in printed
+    tables = (tmp_path / "kernels.txt").read_text()
+    assert "decode batch=1 graphs=True" in tables and "decode batch=6 graphs=False" in tables and "prefill prompt=40" in tables
+    assert "paged_attention" in tables and "gemm_skinny" in tables           # this repository's kernels, by name, with their times
