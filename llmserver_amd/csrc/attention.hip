@@ -970,6 +970,186 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
         }
     }
 }
+#else  // float32
+// ------------------------------------------------------------------------------------------------
+// Portions of prompts in float32: the same arrangement as the bfloat16 kernel above in its plainest form.  The four
+// wavefronts of a workgroup take four consecutive tiles of 16 pairs of one request; each step's 16 keys and values
+// are fetched from the pages once per workgroup (a step ahead, through registers into the other of two LDS buffers)
+// and every wavefront reads its operands from there, so a key travels from the caches once for 64 pairs instead
+// of once for 16.  Every step is masked; products are true 32-bit (16x16x4 MFMAs).
+constexpr int TK_ROW = D * 4 + 16;                 // bytes of a key row in LDS (padded: the 16 rows of an operand read spread over the banks)
+constexpr int TV_ROW = 16 * 4 + 16;                // bytes of a value row (one head dimension, 16 keys)
+constexpr int TK_BYTES = 16 * TK_ROW, TV_BYTES = D * TV_ROW;
+constexpr int TK_PIECES = 16 * (D / 4), TV_PIECES = D * 4;        // 16-byte pieces of a step: four dimensions of a key; four keys of a dimension
+constexpr int TKP = (TK_PIECES + 255) / 256, TVP = (TV_PIECES + 255) / 256;
+
+__global__ __launch_bounds__(256) void paged_attention_tile_kernel_f32(
+    const float* __restrict__ q, long q_token_stride, float* __restrict__ out,
+    const float* __restrict__ keys, const float* __restrict__ values,
+    const int* __restrict__ table, int table_stride,
+    const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
+    const Item* __restrict__ tiles, Geometry g) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * (TK_BYTES + TV_BYTES)];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int heads = g.n_kv * g.gtiles;
+    const Item tile = tiles[blockIdx.x / heads];
+    const int head_index = blockIdx.x % heads;
+    const int kv_head = head_index / g.gtiles, gtile = head_index % g.gtiles;
+    const int col = lane & 15, quad = lane >> 4;
+    const int row = tile.row;
+    const int n = row_len[row], first_pos = row_ctx[row] - n;
+    const int q0 = tile.q0 + wave * g.tokens_per_tile;             // first token of this wavefront's tile
+    const int pair_token = col / g.gheads, pair_head_in_group = gtile * g.gheads + col % g.gheads;
+    const int head = kv_head * g.group + pair_head_in_group;
+    const bool pair_valid = pair_token < g.tokens_per_tile && q0 + pair_token < n && pair_head_in_group < g.group;
+    const int q_pos = pair_valid ? first_pos + q0 + pair_token : -1;
+    const int* row_table = table + (size_t)row * table_stride;
+    const int ps = g.page_size;
+    const size_t kv_head_keys = (size_t)kv_head * ps * D, kv_head_values = (size_t)kv_head * D * ps;
+    const size_t page_elems = (size_t)g.n_kv * ps * D;
+    const int wave_tokens = max(0, min(g.tokens_per_tile, n - q0));
+    const int wave_hi = wave_tokens > 0 ? first_pos + q0 + wave_tokens : 0;                  // keys this wavefront's pairs can see: [wave_lo, wave_hi)
+    const int wave_lo = g.window > 0 ? max(0, first_pos + q0 - g.window + 1) : 0;
+
+    f32x4 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        f32x4 x = {0.f, 0.f, 0.f, 0.f};
+        if (pair_valid) x = *reinterpret_cast<const f32x4*>(q + (size_t)(row_start[row] + q0 + pair_token) * q_token_stride + (size_t)head * D + 16 * s + 4 * quad);
+        qf[s] = x;
+    }
+    f32x4 acc[ND];
+#pragma unroll
+    for (int c = 0; c < ND; ++c) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float run_max = NEG_INF, run_sum = 0.f;
+
+    const int k_begin = tile.k_begin, k_end = tile.k_end;
+    int chunk = -1, pages_cur = 0, pages_next = 0;
+    auto table_chunk = [&](int c) __attribute__((always_inline)) { return row_table[min(64 * c + lane, table_stride - 1)]; };
+    auto enter_chunk = [&](int kt) __attribute__((always_inline)) {
+        const int c = (int)__umulhi((unsigned)kt, g.page_magic) >> 6;
+        if (c != chunk) {
+            pages_cur = (chunk >= 0 && c == chunk + 1) ? pages_next : table_chunk(c);
+            chunk = c;
+            pages_next = table_chunk(c + 1);
+        }
+    };
+    auto locate = [&](int key, int& slot) __attribute__((always_inline)) {
+        const int block = (int)__umulhi((unsigned)key, g.page_magic);
+        slot = key - block * ps;
+        return (size_t)__shfl(pages_cur, block - 64 * chunk, 64) * page_elems;
+    };
+    struct Staged { f32x4 k[TKP], v[TVP]; };
+    // Loads are unconditional: a piece whose keys lie outside the tile's range reads keys of the step that lie inside.
+    auto issue_loads = [&](Staged& r, int kt) __attribute__((always_inline)) {
+        enter_chunk(kt);
+        const int lo = max(k_begin, kt), hi = min(k_end, kt + 16) - 1;
+#pragma unroll
+        for (int j = 0; j < TKP; ++j) {
+            const int piece = min(tid + 256 * j, TK_PIECES - 1);
+            int slot;
+            const int key = min(max(kt + piece / (D / 4), lo), hi);
+            const size_t page = locate(key, slot);
+            r.k[j] = *reinterpret_cast<const f32x4*>(keys + page + kv_head_keys + (size_t)slot * D + 4 * (piece % (D / 4)));
+        }
+#pragma unroll
+        for (int j = 0; j < TVP; ++j) {
+            const int piece = min(tid + 256 * j, TV_PIECES - 1);
+            int slot;
+            const int key0 = min(max(kt + 4 * (piece & 3), lo & ~3), hi & ~3);
+            const size_t page = locate(key0, slot);
+            r.v[j] = *reinterpret_cast<const f32x4*>(values + page + kv_head_values + (size_t)(piece >> 2) * ps + slot);
+        }
+    };
+    auto store_lds = [&](int buf, Staged& r, int kt) __attribute__((always_inline)) {
+        unsigned char* kl = lds + buf * (TK_BYTES + TV_BYTES);
+        unsigned char* vl = kl + TK_BYTES;
+#pragma unroll
+        for (int j = 0; j < TKP; ++j) {
+            const int piece = tid + 256 * j;
+            if (piece < TK_PIECES) *reinterpret_cast<f32x4*>(kl + (piece / (D / 4)) * TK_ROW + 16 * (piece % (D / 4))) = r.k[j];
+        }
+#pragma unroll
+        for (int j = 0; j < TVP; ++j) {
+            const int piece = tid + 256 * j;
+            f32x4 four = r.v[j];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {               // keys outside the range may hold anything: keep them out of the sums
+                const int kpos = kt + 4 * (piece & 3) + e;
+                if (kpos < k_begin || kpos >= k_end) four[e] = 0.f;
+            }
+            if (piece < TV_PIECES) *reinterpret_cast<f32x4*>(vl + (piece >> 2) * TV_ROW + 16 * (piece & 3)) = four;
+        }
+    };
+    auto compute = [&](int buf, int kt) __attribute__((always_inline)) {
+        if (kt >= wave_hi || kt + 16 <= wave_lo) return;           // nothing for this wavefront's pairs in this step
+        const unsigned char* kl = lds + buf * (TK_BYTES + TV_BYTES);
+        const unsigned char* vl = kl + TK_BYTES;
+        f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const f32x4 kf = *reinterpret_cast<const f32x4*>(kl + col * TK_ROW + 64 * s + 16 * quad);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[r], qf[s][r], s4, 0, 0, 0);
+        }
+        float sv[4];
+        float step_max = NEG_INF;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int kpos = kt + 4 * quad + r;
+            const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos && (g.window <= 0 || kpos > q_pos - g.window);
+            sv[r] = seen ? s4[r] * g.scale : NEG_INF;
+            step_max = fmaxf(step_max, sv[r]);
+        }
+        step_max = fmaxf(step_max, __shfl_xor(step_max, 16, 64));
+        step_max = fmaxf(step_max, __shfl_xor(step_max, 32, 64));
+        const float new_max = fmaxf(run_max, step_max);
+        const float use_max = new_max == NEG_INF ? 0.f : new_max;
+        const float alpha = expf(run_max - use_max);                 // exp(-inf) = 0 for the first keys
+        run_max = new_max;
+        run_sum *= alpha;
+        float pv[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            pv[r] = expf(sv[r] - use_max);
+            run_sum += pv[r];
+        }
+#pragma unroll
+        for (int c = 0; c < ND; ++c) {
+            acc[c] *= alpha;
+            const f32x4 vf = *reinterpret_cast<const f32x4*>(vl + (16 * c + col) * TV_ROW + 16 * quad);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[r], pv[r], acc[c], 0, 0, 0);
+        }
+    };
+
+    if (k_begin < k_end) {
+        Staged ahead;
+        int kt = (k_begin / 16) * 16;
+        const int last = ((k_end - 1) / 16) * 16;
+        issue_loads(ahead, kt);
+        store_lds(0, ahead, kt);
+        __syncthreads();
+        int buf = 0;
+        while (true) {
+            const bool more = kt + 16 <= last;
+            if (more) issue_loads(ahead, kt + 16);                // under way while this step is multiplied
+            compute(buf, kt);
+            if (!more) break;
+            store_lds(buf ^ 1, ahead, kt + 16);                   // the other buffer: everybody left it at the last barrier
+            __syncthreads();
+            buf ^= 1;
+            kt += 16;
+        }
+    }
+    run_sum += __shfl_xor(run_sum, 16, 64);
+    run_sum += __shfl_xor(run_sum, 32, 64);
+    if (!pair_valid) return;
+    const float inv = run_sum > 0.f ? 1.f / run_sum : 0.f;
+    float* o = out + ((size_t)(row_start[row] + q0 + pair_token) * g.n_q + head) * D + 4 * quad;
+#pragma unroll
+    for (int c = 0; c < ND; ++c) *reinterpret_cast<f32x4*>(o + 16 * c) = acc[c] * inv;
+}
 #endif  // LSA_BF16
 
 // Merge the partial slots of a tile: out = sum_s w_s acc_s / sum_s w_s l_s, w_s = exp(m_s - max m).
@@ -1118,7 +1298,12 @@ LSA_EXPORT int lsa_paged_attention(
         const int terr = (int)hipGetLastError();
         if (terr) return terr;
 #else
-        return -1;                    // the workgroup-tile kernel exists for bfloat16 only
+        if (tiles_per_workgroup != 4 || tile_halves != 1) return -1;      // the float32 kernel: four tiles, keys whole
+        paged_attention_tile_kernel_f32<<<dim3(n_tiles * n_kv * gtiles), 256, 0, stream>>>(
+            (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
+            row_start, row_len, row_ctx, (const Item*)tiles, g);
+        const int terr = (int)hipGetLastError();
+        if (terr) return terr;
 #endif
     }
     if (n_items <= 0) return 0;
@@ -1162,13 +1347,13 @@ LSA_EXPORT int lsa_paged_attention(
     LSA_LAUNCH_CHECK();
 }
 
-// Most tiles of 16 pairs that one workgroup of the prompt-portion kernel takes (it also takes 4; 0: no such
-// kernel for this type).
+// Most tiles of 16 pairs that one workgroup of the prompt-portion kernel takes (it also takes 4; the float32 kernel
+// takes 4 only).
 LSA_EXPORT int lsa_attention_workgroup_tiles() {
 #if LSA_BF16
     return 4 * MAX_SUB;
 #else
-    return 0;
+    return 4;
 #endif
 }
 // Halves that a workgroup of the prompt-portion kernel can split a tile's keys between (1: it cannot).

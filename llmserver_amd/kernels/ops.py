@@ -545,8 +545,8 @@ class HipOps:
         return self._attention[key]
 
     def attention_workgroup_tiles(self, dtype, head_dim) -> int:
-        """Tiles of 16 (token, head) pairs that a workgroup of the prompt-portion attention kernel takes together
-        (what an entry of a plan's ``tiles`` must span), or 0 if this type has no such kernel."""
+        """Most tiles of 16 (token, head) pairs that a workgroup of the prompt-portion attention kernel takes together
+        (an entry of a plan's ``tiles`` spans four, or this many)."""
         return int(self._attention_library(dtype, head_dim).lsa_attention_workgroup_tiles())
 
     def attention_tile_halves(self, dtype, head_dim) -> int:
@@ -595,8 +595,9 @@ class HipOps:
         tiles = plan.get("tiles") if n_tiles else None
         if n_tiles:
             _check(tiles, "plan tiles", torch.int32, (n_tiles, 4))
-            if qkv.dtype != torch.bfloat16:
-                raise TypeError("the workgroup-tile attention kernel exists for bfloat16 only")
+            most = self.attention_workgroup_tiles(qkv.dtype, head_dim)
+            if int(plan.get("tiles_per_workgroup", 0)) not in (4, most):
+                raise ValueError(f"the plan gives a workgroup {plan.get('tiles_per_workgroup')} tiles, this kernel takes 4 or {most}")
         gheads, tokens_per_tile, gtiles = group_tiling(n_q // n_kv)
         part_acc = part_ml = None
         if n_slots:

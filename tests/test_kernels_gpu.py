@@ -361,6 +361,19 @@ def test_attention_prompt_portions_in_workgroup_tiles(ops, n_q, n_kv, d, page, w
                 assert (plan.tiles_per_workgroup, plan.tile_halves) == (per_workgroup, halves) and len(plan.tiles) > 0
 
 
+@pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 2, 48, 12), (32, 8, 128, 16), (5, 1, 80, 20), (2, 1, 256, 500)])
+@pytest.mark.parametrize("window", [None, 40])
+def test_attention_prompt_portions_in_workgroup_tiles_float32(ops, n_q, n_kv, d, page, window):
+    """The float32 form of the prompt-portion kernel (four tiles to a workgroup, true 32-bit products) against the twin
+    at float32 tolerances, with a needle among the far keys, beside decoded tokens and short portions."""
+    print(f"attention workgroup tiles float32 {n_q}/{n_kv} d{d} page{page} window {window}", flush=True)
+    assert ops.attention_workgroup_tiles(torch.float32, d) == 4 and ops.attention_tile_halves(torch.float32, d) == 1
+    lens = [333, 1, 200, 97, 1]
+    ctxs = [333, 90, 777, 130, 400]
+    plan, _ = attention_case(ops, torch.float32, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d)
+    assert len(plan.tiles) > 0 and len(plan.items) > 0 and plan.tiles_per_workgroup == 4
+
+
 def test_attention_refuses_sizes_it_cannot_take(ops):
     from llmserver_amd.kernels import build
     with pytest.raises(ValueError, match="head sizes"):
