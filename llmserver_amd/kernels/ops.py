@@ -549,6 +549,15 @@ class HipOps:
         (an entry of a plan's ``tiles`` spans four, or this many)."""
         return int(self._attention_library(dtype, head_dim).lsa_attention_workgroup_tiles())
 
+    def attention_tile_min_workgroups(self, dtype) -> int:
+        """Workgroups below which a launch of the prompt-portion kernel does not pay.  The float32 kernel's steps are
+        slow (true 32-bit products, 16 keys a step), so with few workgroups its longest one decides: measured at head
+        size 128, 1,024 workgroups finish 1.4 times sooner than wavefronts of their own, 256 (one for every compute
+        unit) take a third longer.  Wanted: a quarter more workgroups than compute units."""
+        if dtype == torch.bfloat16:
+            return 0
+        return 5 * torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count // 4
+
     def attention_tile_halves(self, dtype, head_dim) -> int:
         """Halves that a workgroup of the prompt-portion kernel can split its tiles' keys between (1: it cannot)."""
         return int(self._attention_library(dtype, head_dim).lsa_attention_tile_halves())

@@ -185,14 +185,16 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, 
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
                          workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: int = 0,
-                         tuning: AttentionTuning = DEFAULT_TUNING, tile_halves: int = 1) -> AttentionPlan:
+                         tuning: AttentionTuning = DEFAULT_TUNING, tile_halves: int = 1, tile_min_workgroups: int = 0) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
     arrays have the same shape whatever the contexts are.  With ``workgroup_tiles`` (the number of tiles a
     workgroup of that kernel takes, which the kernel library tells) rows with many tiles (portions of prompts) go
     to the kernel in which the tiles of a workgroup share the keys they load; ``tile_halves`` says whether that kernel
-    can split a workgroup's keys between two halves of its wavefronts (2) or not (1)."""
+    can split a workgroup's keys between two halves of its wavefronts (2) or not (1), ``tile_min_workgroups`` how many
+    workgroups a launch of it needs to be worth while (a kernel whose steps are slow is bounded by its longest
+    workgroup unless there are many)."""
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
@@ -213,6 +215,11 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
         chosen = _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window,
                                            int(workgroup_tiles), tuning, int(tile_halves))
         per_workgroup, halves = chosen if isinstance(chosen, tuple) else (chosen, 1)
+        if per_workgroup and tile_min_workgroups:
+            groups = sum(-(-int(n) // (per_workgroup * tokens_per_tile)) for n, tiles_of_row in zip(row_len, tiles_per_row)
+                         if tiles_of_row >= MIN_TILES_FOR_WORKGROUPS)
+            if groups * n_kv_heads * group_tiles < tile_min_workgroups:
+                per_workgroup, halves = 0, 1
     for row in range(len(row_len)):
         n, ctx = int(row_len[row]), int(row_ctx[row])
         first_pos = ctx - n
@@ -337,9 +344,11 @@ class GQAttention(Mixer):
         per_workgroup = per_workgroup(ctx.dtype, self.head_dim) if per_workgroup is not None else 0
         halves = getattr(ctx.ops, "attention_tile_halves", None)
         halves = halves(ctx.dtype, self.head_dim) if halves is not None and per_workgroup else 1
+        fewest = getattr(ctx.ops, "attention_tile_min_workgroups", None)
+        fewest = fewest(ctx.dtype) if fewest is not None and per_workgroup else 0
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
                                     target_waves=tuning.target_waves, fixed_splits=fixed, workgroup_tiles=per_workgroup,
-                                    merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves)
+                                    merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves, tile_min_workgroups=fewest)
         ctx.set_plan(key, {
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
             "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),

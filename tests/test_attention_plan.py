@@ -155,3 +155,8 @@ def test_four_or_eight_tiles_per_workgroup_whole_or_in_halves():
     assert chosen([4096], [4096], most=4) == (4, 1)
     assert chosen([1] * 8, [4096] * 8) == (0, 1)                             # no row has enough tiles
     assert build_attention_plan([4096], [4096], 4, 8, None).tiles_per_workgroup == 0
+    # a kernel that needs many workgroups to pay gets them or nothing
+    few = build_attention_plan([512], [2560], 4, 8, None, workgroup_tiles=4, tile_min_workgroups=512)
+    many = build_attention_plan([2048], [2048], 4, 8, None, workgroup_tiles=4, tile_min_workgroups=512)
+    assert (few.tiles_per_workgroup, len(few.tiles)) == (0, 0) and len(few.items) == 128
+    assert (many.tiles_per_workgroup, len(many.tiles)) == (4, 128)

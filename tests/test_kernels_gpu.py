@@ -370,7 +370,7 @@ def test_attention_prompt_portions_in_workgroup_tiles_float32(ops, n_q, n_kv, d,
     assert ops.attention_workgroup_tiles(torch.float32, d) == 4 and ops.attention_tile_halves(torch.float32, d) == 1
     lens = [333, 1, 200, 97, 1]
     ctxs = [333, 90, 777, 130, 400]
-    plan, _ = attention_case(ops, torch.float32, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d)
+    plan, _ = attention_case(ops, torch.float32, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d, workgroup_tiles=4)
     assert len(plan.tiles) > 0 and len(plan.items) > 0 and plan.tiles_per_workgroup == 4
 
 
