@@ -284,3 +284,32 @@ LSA_EXPORT int lsa_add_bias(int dtype, void* y, const float* bias, int n_tokens,
     return dtype ? launch_add_bias<bf16_t>(y, bias, n_tokens, n, stream)
                  : launch_add_bias<float>(y, bias, n_tokens, n, stream);
 }
+
+// ------------------------------------------------------------------------------------------
+// A plain read of memory, for scale: what the memory system delivers to a kernel that does nothing but read, from a
+// given number of workgroups.  Every workgroup streams a contiguous share of `bytes` with 16-byte loads, eight of
+// them in flight per lane, and adds what it reads up (the sum is written only if it has a value it cannot have, so
+// that the loads stay).  The rooflines of the step's kernels are read against this, not only against the data sheet.
+typedef float read_f32x4 __attribute__((ext_vector_type(4)));
+__global__ void plain_read_kernel(const read_f32x4* __restrict__ data, float* __restrict__ sink, size_t pieces_per_workgroup) {
+    const read_f32x4* base = data + (size_t)blockIdx.x * pieces_per_workgroup;
+    read_f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    const size_t stride = blockDim.x;
+    for (size_t first = threadIdx.x; first < pieces_per_workgroup; first += stride * 8) {
+        read_f32x4 piece[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const size_t at = first + u * stride;
+            piece[u] = base[at < pieces_per_workgroup ? at : first];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += piece[u];
+    }
+    if (sum.x + sum.y + sum.z + sum.w == 12345.678f) sink[0] = 1.f;
+}
+// `bytes` of `data` (a multiple of 16 * workgroups is read; the rest is left out), `threads` per workgroup (64 to 1024).
+LSA_EXPORT int lsa_plain_read(const void* data, float* sink, long bytes, int workgroups, int threads, hipStream_t stream) {
+    if (!data || !sink || workgroups <= 0 || threads < 64 || threads > 1024 || threads % 64 || bytes < 16L * workgroups) return -1;
+    plain_read_kernel<<<workgroups, threads, 0, stream>>>((const read_f32x4*)data, sink, (size_t)(bytes / 16 / workgroups));
+    LSA_LAUNCH_CHECK();
+}

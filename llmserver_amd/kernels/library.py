@@ -14,6 +14,7 @@ _SIGNATURES = {
     "lsa_add_rmsnorm_partial_sums": [c_int, _P, _P, c_int, c_long, _P, c_float, _P, _P, c_int, c_int, _P],
     "lsa_swiglu": [c_int, _P, _P, c_int, c_int, _P],
     "lsa_add_bias": [c_int, _P, _P, c_int, c_int, _P],
+    "lsa_plain_read": [_P, _P, c_long, c_int, c_int, _P],
     "lsa_qk_norm_rope_kv_write": [c_int, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_float, _P, c_int, c_int, c_int, c_int,
                                   c_int, c_int, _P],
     "lsa_rotary_table": [_P, _P, _P, c_int, c_int, _P],

@@ -683,3 +683,18 @@ def test_few_row_kernel_or_library_by_table(ops, tmp_path):
     finally:
         ops.choices = saved_table
         ops.consult_choices = False
+
+
+def test_plain_read_runs_and_refuses_what_it_cannot_split():
+    """The bandwidth tool's kernel: any number of workgroups and threads it is documented for, nothing read past the end."""
+    from llmserver_amd.kernels import bandwidth, library
+    lib = library.load("elementwise")
+    data = torch.ones(1 << 16, device=DEV)
+    sink = torch.zeros(1, device=DEV)
+    for workgroups, threads in ((1, 64), (7, 256), (256, 1024)):
+        assert lib.lsa_plain_read(data.data_ptr(), sink.data_ptr(), data.numel() * 4, workgroups, threads, None) == 0
+    assert lib.lsa_plain_read(data.data_ptr(), sink.data_ptr(), data.numel() * 4, 4, 100, None) == -1
+    assert lib.lsa_plain_read(data.data_ptr(), sink.data_ptr(), 16, 4, 256, None) == -1
+    torch.cuda.synchronize()
+    assert float(sink) == 0.0
+    assert 0 < bandwidth.measure(8, 64, 256, repeats=1) < 1.0
