@@ -584,32 +584,74 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
 // ------------------------------------------------------------------------------------------------
 // Portions of prompts: the four wavefronts of a workgroup take 4 * SUB consecutive tiles of 16 pairs
 // of one request (SUB tiles each).  They see (almost) the same keys, so each step's 32 keys and values are fetched
-// from the pages once per workgroup into LDS (double-buffered: the global loads of step i+1 are
-// issued before the products of step i and stored to the other buffer afterwards, one barrier a
-// step) and every wavefront reads its MFMA operands from there, 16 bytes per lane and read (8-byte
-// reads reach three quarters of the LDS rate at best).  Rows in LDS are padded so that the operand
+// from the pages once per workgroup, straight into LDS (global_load_lds, 16 bytes a lane: no registers and no LDS
+// stores on the way), into a ring of STAGES buffers: the loads of step i + STAGES - 1 are issued before the products
+// of step i, one barrier a step, and every wavefront reads its MFMA operands from LDS, 16 bytes per lane and read
+// (8-byte reads reach three quarters of the LDS rate at best).  Rows in LDS are padded so that the operand
 // reads of a wavefront spread over the banks.  No key ranges are split here: such
 // rows have many tiles.  `tiles[i]` = {row, first token of the workgroup's tiles, k_begin, k_end}.
-constexpr int K_ROW = D * 2 + 16;                 // bytes of a key row in LDS
-constexpr int V_ROW = 32 * 2 + 16;                // bytes of a value row (one head dimension, 32 keys; see store_lds for their order)
-constexpr int K_TILE_BYTES = 32 * K_ROW, V_TILE_BYTES = D * V_ROW;
-// A step is fetched as two halves of 16 keys (with pages of 16 or more keys each half lies in one page):
-// per half, 16-byte pieces of keys (16 keys x D, contiguous in the page) and 8-byte pieces of values (D rows of 4 keys).
-constexpr int K_HALF_PIECES = 16 * (D / 8), V_HALF_PIECES = D * 4;
-constexpr int KPH = (K_HALF_PIECES + 255) / 256, VPH = (V_HALF_PIECES + 255) / 256;      // pieces per thread and half
+//
+// A load writes 64 lanes x 16 bytes to 1 KB of LDS in lane order, from wherever each lane points: a step's buffer is
+// a row of such 1 KB chunks, and a lane's place in its chunk says which 16 bytes of the step it fetches (the padding
+// of the rows, and the places behind the last row of a chunk, fetch a neighbour's bytes again).  Each of the four
+// wavefronts fetches one quarter of a step: the keys of its first 16 keys, the keys of its last 16, the values of the
+// first 16, the values of the last 16.  With pages of 16 keys or a multiple, such a quarter lies in one page: the
+// wavefront looks one page up (a scalar), and every load is that page's address plus the lane's constant offset.
+//   keys:   two blocks of 16 rows of D * 2 + 16 bytes.  The rows of a block are the 16 keys in page order, except that
+//           in the second block rows i and i ^ 4 change places.  The score product t (of two) takes keys
+//           8 a + b + 4 t (a, b = 0 .. 3) for its 16 rows: lane quad q is then left with keys 8 q + 4 t .. 8 q + 4 t + 3,
+//           after both products a lane's eight scores are the step's keys 8 q .. 8 q + 7 in order; and the 16 rows of
+//           a product lie at 16 different row numbers modulo 16 (that is what the exchange is for), so that their
+//           reads spread over all banks.
+//   values: two blocks (the first and the last 16 keys) of D rows (one head dimension) of 32 + 16 bytes: lane quad q
+//           of the output product reads keys 8 q .. 8 q + 7 of its dimension as one 16-byte piece, the same 16 bytes
+//           as in the page.
+constexpr int K_ROW_SLOTS = D / 8 + 1, V_ROW_SLOTS = 3;            // 16-byte places of a row in LDS, the last one padding
+constexpr int K_ROW = 16 * K_ROW_SLOTS, V_ROW = 16 * V_ROW_SLOTS;  // bytes of a key row, of a value row of one block
+constexpr int K_BLOCK_CHUNKS = (16 * K_ROW_SLOTS + 63) / 64, V_BLOCK_CHUNKS = (D * V_ROW_SLOTS + 63) / 64;   // 1 KB each
+constexpr int K_BLOCK_BYTES = 1024 * K_BLOCK_CHUNKS, V_BLOCK_BYTES = 1024 * V_BLOCK_CHUNKS;
+constexpr int K_TILE_BYTES = 2 * K_BLOCK_BYTES, STEP_BYTES = K_TILE_BYTES + 2 * V_BLOCK_BYTES;
+constexpr int STEP_LOADS = K_BLOCK_CHUNKS > V_BLOCK_CHUNKS ? K_BLOCK_CHUNKS : V_BLOCK_CHUNKS;     // of a wavefront per step
+// Buffers in the ring: three where two workgroups of them still fit a compute unit's 160 KB (loads then run two steps
+// ahead of the products), else two.
+#ifndef LSA_TILE_STAGES
+#define LSA_TILE_STAGES (2 * 3 * STEP_BYTES <= 160 * 1024 ? 3 : 2)
+#endif
+constexpr int STAGES = LSA_TILE_STAGES;
 // Tiles of 16 pairs per wavefront (SUB): with two, every key and value operand read from LDS feeds two products, which
-// halves the LDS traffic per flop (the kernel's limit); the accumulators of two tiles fit the registers up to a head size of 128.
+// halves the LDS traffic per flop; the accumulators of two tiles fit the registers up to a head size of 128.
 // The host picks one or two per launch: two pay when the rows are long (the longest workgroup then does not
 // decide the time), one when they are short and there are few workgroups.
 constexpr int MAX_SUB = LSA_ND <= 8 ? 2 : 1;
-// Halves of a workgroup that split the keys between them (see the kernel): two where their buffers leave room in LDS for
-// more than one workgroup.
+// Halves of a workgroup that split the keys between them (see the kernel): two where their buffers fit into LDS.
 constexpr int MAX_HALVES = LSA_ND <= 8 ? 2 : 1;
 // Wavefronts per SIMD wanted (they hide the latency of a step's dependent chain: LDS read, MFMA, softmax, MFMA),
 // as far as the registers of SUB tiles allow.
 #define LSA_TILE_MIN_WAVES(SUB) ((SUB) == 1 ? (LSA_ND <= 8 ? 3 : 1) : (LSA_ND <= 4 ? 3 : 2))
 struct FullStep { static constexpr bool value = true; };        // every key of the step is seen by every pair
 struct MaskedStep { static constexpr bool value = false; };
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
+
+// One load of a wavefront straight into LDS: lane i's 16 bytes go to `lds_address` + 16 i (a byte address in LDS, the
+// same for all lanes).  Written out rather than called as a builtin: the compiler makes every later LDS read wait for
+// all loads it knows to write LDS, and these are meant to stay in flight while the steps before them are read.
+__device__ __forceinline__ void load_16_bytes_a_lane_to_lds(const void* source, unsigned lds_address) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(source), "s"(lds_address) : "memory", "m0");
+}
+// The same with one base for all lanes and a byte offset per lane.
+__device__ __forceinline__ void load_16_bytes_a_lane_to_lds(const void* base, unsigned offset, unsigned lds_address) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(base), "s"(lds_address) : "memory", "m0");
+}
+
+// Waits until at most PENDING of this wavefront's loads are still under way (they land in the order they were
+// issued), then for the workgroup.  Written out because __syncthreads() would wait for every load, also for those
+// of the steps ahead, which are meant to stay in flight across the barrier.
+template <int PENDING>
+__device__ __forceinline__ void loads_landed_then_barrier() {
+    static_assert(PENDING >= 0 && PENDING < 64, "the counter of loads in flight has six bits");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(PENDING) : "memory");
+}
 
 // HALVES = 2: the workgroup has eight wavefronts; wavefronts 4 .. 7 take the same tiles as wavefronts 0 .. 3 and the
 // second half of the keys' steps, through LDS buffers of their own, and leave their running maximum, sum and
@@ -624,10 +666,10 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
     const int* __restrict__ table, int table_stride,
     const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
     const Item* __restrict__ tiles, Geometry g) {
-    constexpr int STEP_BYTES = K_TILE_BYTES + V_TILE_BYTES;
-    __shared__ __attribute__((aligned(16))) unsigned char lds_all[HALVES * 2 * STEP_BYTES];
-    const int half = HALVES > 1 ? (int)(threadIdx.x >> 8) : 0;
-    const int lds_base = half * 2 * STEP_BYTES;                       // this half's two buffers
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_all[HALVES * STAGES * STEP_BYTES];
+    const int half = HALVES > 1 ? __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) : 0;     // (the same in all lanes, and known to be)
+    const int lds_base = half * STAGES * STEP_BYTES;                  // this half's ring of buffers
+    const unsigned lds_begin = (unsigned)__builtin_amdgcn_readfirstlane((int)((unsigned)(size_t)(lds_ptr_t)lds_all + (unsigned)lds_base));      // its byte address in LDS
     const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
     // Workgroups are handed to the eight XCDs in turn, and each XCD has its own L2: with the KV head
     // running fastest over the workgroup index, an XCD keeps meeting the same few KV heads, whose
@@ -688,112 +730,100 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
     const int cut = min(tile.k_end, first_step + 32 * trips);         // where the second half's keys begin
     const int k_begin = half ? cut : tile.k_begin, k_end = half ? tile.k_end : cut;
     const int my_steps = half ? all_steps - trips : trips;
-    int chunk = -1, pages_cur = 0, pages_next = 0;
-    auto table_chunk = [&](int c) __attribute__((always_inline)) { return row_table[min(64 * c + lane, table_stride - 1)]; };
+    // The row's table, 64 entries at a time, one in each lane: a step's pages are read from there (64 pages hold a
+    // whole number of steps).  After the load of the next 64 entries the wavefront waits for every load it has in
+    // flight, this one included, and says so to the compiler: a wait that the compiler places itself would stand in
+    // every trip (it cannot tell the trips that bring new entries from those that do not).
+    // Each of the four wavefronts fetches one quarter of a step: keys or values (`of_values`), of the step's first or
+    // last 16 keys (`late`); beside the page's number a lane keeps where the wavefront's kind of data begins in it.
+    const int wave_uniform = __builtin_amdgcn_readfirstlane(wave);
+    const bool of_values = wave_uniform >= 2;
+    const int late = wave_uniform & 1;
+    const char* const quarter_data = of_values ? reinterpret_cast<const char*>(values + kv_head_values) : reinterpret_cast<const char*>(keys + kv_head_keys);
+    int chunk = -1, chunk_pages = 0;
+    unsigned long long chunk_begins = 0;
     auto enter_chunk = [&](int kt) __attribute__((always_inline)) {
         const int c = (int)__umulhi((unsigned)kt, g.page_magic) >> 6;
         if (c != chunk) {
-            pages_cur = (chunk >= 0 && c == chunk + 1) ? pages_next : table_chunk(c);
             chunk = c;
-            pages_next = table_chunk(c + 1);
+            chunk_pages = row_table[min(64 * c + lane, table_stride - 1)];
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            chunk_begins = (unsigned long long)(quarter_data + 2 * (size_t)chunk_pages * page_elems);
         }
-    };
-    auto locate = [&](int key, int& slot) __attribute__((always_inline)) {
-        const int block = (int)__umulhi((unsigned)key, g.page_magic);
-        slot = key - block * ps;
-        return (size_t)__shfl(pages_cur, block - 64 * chunk, 64) * page_elems;
     };
 
-    struct Staged {
-        bf16x8 k[2][KPH];
-        bf16x4 v[2][VPH];
-    };
-    // Where each of this thread's pieces lies inside a half step: constant over the steps.  Piece q of the keys is
-    // bytes [16 q, 16 q + 16) of the half's 16 x D block; piece q of the values is keys 4 (q & 3) .. + 4 of dimension q >> 2.
-    unsigned k_off[KPH], v_off[VPH];                // byte offsets from the half's first key in the page
+    // What this lane fetches in each of its wavefront's loads of a step: constant over the steps.  `piece_key` is the
+    // piece's (first) key among those 16, `piece_at` the 16-byte piece of the key's row (keys) or the head dimension
+    // (values), `piece_offset` its byte offset from where the first of the 16 keys lies in its page.
+    const int quarter_chunks = of_values ? V_BLOCK_CHUNKS : K_BLOCK_CHUNKS;
+    const unsigned quarter_lds = lds_begin + (unsigned)(of_values ? K_TILE_BYTES + late * V_BLOCK_BYTES : late * K_BLOCK_BYTES);
+    int piece_key[STEP_LOADS], piece_at[STEP_LOADS];
+    unsigned piece_offset[STEP_LOADS];
 #pragma unroll
-    for (int j = 0; j < KPH; ++j) k_off[j] = 16u * (unsigned)min(tid + 256 * j, K_HALF_PIECES - 1);
-#pragma unroll
-    for (int j = 0; j < VPH; ++j) {
-        const int q = min(tid + 256 * j, V_HALF_PIECES - 1);
-        v_off[j] = 2u * (unsigned)((q >> 2) * ps + 4 * (q & 3));
+    for (int m = 0; m < STEP_LOADS; ++m) {
+        const int place = 64 * min(m, quarter_chunks - 1) + lane;
+        if (!of_values) {
+            const int r = min(place / K_ROW_SLOTS, 15);
+            piece_at[m] = min(place % K_ROW_SLOTS, D / 8 - 1);
+            piece_key[m] = late ? (r ^ 4) : r;
+            piece_offset[m] = (unsigned)(piece_key[m] * (2 * D) + 16 * piece_at[m]);
+        } else {
+            piece_at[m] = min(place / V_ROW_SLOTS, D - 1);
+            piece_key[m] = 8 * min(place % V_ROW_SLOTS, 1);
+            piece_offset[m] = (unsigned)(2 * (piece_at[m] * ps + piece_key[m]));
+        }
     }
     const bool pages_of_16 = (ps & 15) == 0;        // then each half of a step (16 keys) lies inside one page
-    auto issue_loads = [&](Staged& r, int kt) __attribute__((always_inline)) {
+    auto issue_loads = [&](int stage, int kt) __attribute__((always_inline)) {
         enter_chunk(kt);
+        const unsigned buffer = quarter_lds + (unsigned)(stage * STEP_BYTES);
+        const int first_key = kt + 16 * late;
         if (pages_of_16 && kt >= k_begin && kt + 32 <= k_end) {
-            // Interior step: one page lookup per half for the whole wavefront (scalar); every piece is then the
-            // half's base, the same for all lanes, plus the thread's constant offset.
+            // Interior step: one page lookup for the whole wavefront (scalar).
+            const int block = (int)__umulhi((unsigned)first_key, g.page_magic), slot = first_key - block * ps;
+            const unsigned low = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)chunk_begins, block - 64 * chunk);
+            const unsigned high = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(chunk_begins >> 32), block - 64 * chunk);
+            const char* base = reinterpret_cast<const char*>(((unsigned long long)high << 32) | low) + (of_values ? 2 * slot : 2 * D * slot);
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int key = kt + 16 * h;
-                const int block = (int)__umulhi((unsigned)key, g.page_magic), slot = key - block * ps;
-                const size_t page = (size_t)__builtin_amdgcn_readlane(pages_cur, block - 64 * chunk) * page_elems;
-                const char* kbase = reinterpret_cast<const char*>(keys + page + kv_head_keys + (size_t)slot * D);
-                const char* vbase = reinterpret_cast<const char*>(values + page + kv_head_values + slot);
-#pragma unroll
-                for (int j = 0; j < KPH; ++j) r.k[h][j] = *reinterpret_cast<const bf16x8*>(kbase + k_off[j]);
-#pragma unroll
-                for (int j = 0; j < VPH; ++j) r.v[h][j] = *reinterpret_cast<const bf16x4*>(vbase + v_off[j]);
-            }
+            for (int m = 0; m < STEP_LOADS; ++m)
+                load_16_bytes_a_lane_to_lds(base, piece_offset[m], buffer + 1024u * (unsigned)min(m, quarter_chunks - 1));
             return;
         }
+        // A step at an end of the key range, or pages that are no multiple of 16 keys: every lane looks its key's
+        // page up.  Keys outside the range are never fetched (their pages may not be the request's): the nearest
+        // key inside stands in, and the scores and values of such places are masked where they are used.
         const int lo = max(k_begin, kt), hi = min(k_end, kt + 32) - 1;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-#pragma unroll
-            for (int j = 0; j < KPH; ++j) {
-                const int q = min(tid + 256 * j, K_HALF_PIECES - 1);
-                int slot;
-                const int key = min(max(kt + 16 * h + q / (D / 8), lo), hi);
-                const size_t page = locate(key, slot);
-                r.k[h][j] = *reinterpret_cast<const bf16x8*>(keys + page + kv_head_keys + (size_t)slot * D + 8 * (q % (D / 8)));
-            }
-#pragma unroll
-            for (int j = 0; j < VPH; ++j) {
-                const int q = min(tid + 256 * j, V_HALF_PIECES - 1);
-                int slot;
-                const int key0 = min(max(kt + 16 * h + 4 * (q & 3), lo & ~3), hi & ~3);
-                const size_t page = locate(key0, slot);
-                r.v[h][j] = *reinterpret_cast<const bf16x4*>(values + page + kv_head_values + (size_t)(q >> 2) * ps + slot);
-            }
+        for (int m = 0; m < STEP_LOADS; ++m) {
+            const int key = of_values ? min(max(first_key + piece_key[m], lo & ~7), hi & ~7) : min(max(first_key + piece_key[m], lo), hi);
+            const int block = (int)__umulhi((unsigned)key, g.page_magic), slot = key - block * ps;
+            const size_t page = (size_t)__shfl(chunk_pages, block - 64 * chunk, 64) * page_elems;
+            const char* source = of_values
+                ? reinterpret_cast<const char*>(values + page + kv_head_values + (size_t)piece_at[m] * ps + slot)
+                : reinterpret_cast<const char*>(keys + page + kv_head_keys + (size_t)slot * D + 8 * piece_at[m]);
+            load_16_bytes_a_lane_to_lds(source, buffer + 1024u * (unsigned)min(m, quarter_chunks - 1));
         }
     };
-    auto store_lds = [&](int buf, Staged& r, int kt) __attribute__((always_inline)) {
-        unsigned char* kl = lds_all + lds_base + buf * STEP_BYTES;
-        unsigned char* vl = kl + K_TILE_BYTES;
-        const bool edge = kt < k_begin || kt + 32 > k_end;
+    // Where this lane reads its operands in a step's buffer: the key row of each of the two score products (key
+    // 8 a + b + 4 t for lane column 4 a + b), and its 16 bytes of a value row.
+    int key_row_at[2];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-#pragma unroll
-            for (int j = 0; j < KPH; ++j) {
-                const int q = tid + 256 * j;
-                if (q < K_HALF_PIECES) *reinterpret_cast<bf16x8*>(kl + (16 * h + q / (D / 8)) * K_ROW + 16 * (q % (D / 8))) = r.k[h][j];
-            }
-#pragma unroll
-            for (int j = 0; j < VPH; ++j) {
-                const int q = tid + 256 * j;
-                bf16x4 piece = r.v[h][j];
-                if (edge) {                       // keys outside the range may hold anything: keep them out of the sums
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int kpos = kt + 16 * h + 4 * (q & 3) + e;
-                        if (kpos < k_begin || kpos >= k_end) piece[e] = (bf16_t)0.f;
-                    }
-                }
-                // Keys 4 s .. 4 s + 3 of half h go to bytes 16 s + 8 h: the eight keys that lane quad s of the output
-                // product multiplies (four of each half, as the score product left them) are then 16 contiguous bytes.
-                if (q < V_HALF_PIECES) *reinterpret_cast<bf16x4*>(vl + (q >> 2) * V_ROW + 16 * (q & 3) + 8 * h) = piece;
-            }
-        }
-    };
+    for (int t2 = 0; t2 < 2; ++t2) {
+        const int key = 8 * (col >> 2) + (col & 3) + 4 * t2;
+        key_row_at[t2] = (key >> 4) * K_BLOCK_BYTES + (key < 16 ? key : ((key - 16) ^ 4)) * K_ROW + 16 * quad;
+    }
+    const int value_at = K_TILE_BYTES + (quad >> 1) * V_BLOCK_BYTES + col * V_ROW + 16 * (quad & 1);
+    // The steps that every pair of the wavefront sees completely (they need no mask) lie in [full_from, full_to]; the
+    // steps that have anything for its pairs in (active_from, active_to).
+    const bool whole_tiles = wave_tokens == SUB * g.tokens_per_tile && g.gheads * g.tokens_per_tile == 16 && (gtile + 1) * g.gheads <= g.group;
+    const int full_from = !whole_tiles ? 0x7fffffff : g.window > 0 ? max(k_begin, first_pos + q0 + wave_tokens - g.window) : k_begin;
+    const int full_to = min(k_end - 32, q_pos_min - 31);
     // Scores stay as the products left them; the scale (in units of ln 2, so that the exponential is one
     // instruction) goes into the multiply-add that also subtracts the running maximum.  FULL: every key of
     // the step is seen by every pair of the wavefront, nothing is masked.
-    auto compute_step = [&](auto full_tag, int buf, int kt) __attribute__((always_inline)) {
+    auto compute_step = [&](auto full_tag, int stage, int kt) __attribute__((always_inline)) {
         constexpr bool FULL = decltype(full_tag)::value;
-        const unsigned char* kl = lds_all + lds_base + buf * STEP_BYTES;
-        const unsigned char* vl = kl + K_TILE_BYTES;
+        const unsigned char* buffer = lds_all + lds_base + stage * STEP_BYTES;
         float sv[SUB][8];
         float tile_max[SUB];
 #pragma unroll
@@ -806,7 +836,7 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 bf16x8 kf = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (32 * s + 32 <= D || quad < 2) kf = *reinterpret_cast<const bf16x8*>(kl + (16 * t2 + col) * K_ROW + 64 * s + 16 * quad);
+                if (32 * s + 32 <= D || quad < 2) kf = *reinterpret_cast<const bf16x8*>(buffer + key_row_at[t2] + 64 * s);
 #pragma unroll
                 for (int u = 0; u < SUB; ++u) s4[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u][s], s4[u], 0, 0, 0);
             }
@@ -816,7 +846,7 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
                 for (int r = 0; r < 4; ++r) {
                     float v = s4[u][r];
                     if (!FULL) {
-                        const int kpos = kt + 16 * t2 + 4 * quad + r;
+                        const int kpos = kt + 8 * quad + 4 * t2 + r;
                         const bool seen = kpos >= k_begin && kpos < k_end && kpos <= q_pos[u] && (g.window <= 0 || kpos > q_pos[u] - g.window);
                         v = seen ? v : NEG_INF;
                     }
@@ -824,13 +854,27 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
                     tile_max[u] = fmaxf(tile_max[u], v);
                 }
         }
+        // Values of keys outside the range may be anything (a page's places behind the context were never written):
+        // their weights are zero, and so that zero times anything stays zero they are cleared where they are read.
+        u32x4 keep = {~0u, ~0u, ~0u, ~0u};
+        if (!FULL) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int kpos = kt + 8 * quad + 2 * i;
+                keep[i] = ((kpos >= k_begin && kpos < k_end) ? 0x0000ffffu : 0u) | ((kpos + 1 >= k_begin && kpos + 1 < k_end) ? 0xffff0000u : 0u);
+            }
+        }
+        auto value_operand = [&](int c) __attribute__((always_inline)) {
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(buffer + value_at + 16 * c * V_ROW);
+            return __builtin_bit_cast(bf16x8, FULL ? raw : (raw & keep));
+        };
         // The value operands are asked for now, so that they arrive while the softmax runs, and the output products
         // of the first tile are issued before the softmax of the second: the MFMA pipe works on them meanwhile.
         // (With one tile per wavefront there is nothing to overlap them with; they are read where they are used.)
         bf16x8 vf[SUB > 1 ? ND : 1];
         if (SUB > 1) {
 #pragma unroll
-            for (int c = 0; c < ND; ++c) vf[c] = *reinterpret_cast<const bf16x8*>(vl + (16 * c + col) * V_ROW + 16 * quad);
+            for (int c = 0; c < ND; ++c) vf[c] = value_operand(c);
         }
         // The running maximum of a pair only moves when some key of this step beats it, which
         // soon becomes rare: then the exchange between the lanes of a pair and the rescaling of
@@ -857,55 +901,44 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
             }
 #pragma unroll
             for (int c = 0; c < ND; ++c) {
-                const bf16x8 value = SUB > 1 ? vf[SUB > 1 ? c : 0] : *reinterpret_cast<const bf16x8*>(vl + (16 * c + col) * V_ROW + 16 * quad);
+                const bf16x8 value = SUB > 1 ? vf[SUB > 1 ? c : 0] : value_operand(c);
                 acc[u][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(value, pf, acc[u][c], 0, 0, 0);
             }
         }
     };
-    auto compute = [&](int buf, int kt) __attribute__((always_inline)) {
+    auto compute = [&](int stage, int kt) __attribute__((always_inline)) {
         if (kt >= wave_hi || kt + 32 <= wave_lo) return;          // nothing for this wavefront's pairs in this step
-        // Steps every pair of the wavefront sees completely need no mask.
-        const bool full = kt >= k_begin && kt + 32 <= k_end && kt + 31 <= q_pos_min && wave_tokens == SUB * g.tokens_per_tile &&
-                          g.gheads * g.tokens_per_tile == 16 && (gtile + 1) * g.gheads <= g.group &&
-                          (g.window <= 0 || kt > first_pos + q0 + wave_tokens - 1 - g.window);
-        if (full) compute_step(FullStep{}, buf, kt);
-        else compute_step(MaskedStep{}, buf, kt);
+        if (kt >= full_from && kt <= full_to) compute_step(FullStep{}, stage, kt);
+        else compute_step(MaskedStep{}, stage, kt);
     };
 
     if (all_steps > 0) {
-        // Loads run two steps ahead of the products: while step i is multiplied out of one LDS
-        // buffer, step i+1 sits in registers on its way to the other buffer and step i+2 is being
-        // fetched.  Loads are issued unconditionally (past the end they fetch the last step again; a half
-        // without keys fetches the step before its own), so that nothing between a load and its use makes the wait
-        // stricter than it has to be.  The trips through the loop are the same for every wavefront of the workgroup.
-        Staged r0, r1;
+        // Loads run STAGES - 1 steps ahead of the products.  They are issued unconditionally (past the end they fetch
+        // the last step again; a half without keys fetches the step before its own), the same number by every
+        // wavefront in every trip, so that counting them tells which have landed.  A trip: wait for this step's loads
+        // (all but those of the steps ahead), meet the others (now everybody's pieces of this step are in LDS, and
+        // everybody is through with the buffer of the step before, which the next loads overwrite), issue, compute.
         int kt = half ? first_step + 32 * trips : first_step;
         const int last = my_steps > 0 ? kt + 32 * (my_steps - 1) : max(first_step, kt - 32);
         if (my_steps == 0) kt = last;
-        issue_loads(r0, kt);
-        issue_loads(r1, min(kt + 32, last));
-        store_lds(0, r0, kt);
-        __syncthreads();
-        int trip = 0;
-        while (true) {
-            issue_loads(r0, min(kt + 64, last));
-            if (trip < my_steps) compute(0, kt);
-            if (trip + 1 >= trips) break;
-            store_lds(1, r1, kt + 32);
-            __syncthreads();
-            issue_loads(r1, min(kt + 96, last));
-            if (trip + 1 < my_steps) compute(1, kt + 32);
-            if (trip + 2 >= trips) break;
-            store_lds(0, r0, kt + 64);
-            __syncthreads();
-            kt += 64;
-            trip += 2;
+        // (every load so far has landed before the first one into LDS is issued: the compiler, which does not see
+        // those, then never waits for "all loads" inside the loop on behalf of the queries)
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+        for (int ahead = 0; ahead < STAGES - 1; ++ahead) issue_loads(ahead, min(kt + 32 * ahead, last));
+        int stage = 0;
+        for (int trip = 0; trip < trips; ++trip) {
+            loads_landed_then_barrier<(STAGES - 2) * STEP_LOADS>();
+            issue_loads(stage == 0 ? STAGES - 1 : stage - 1, min(kt + 32 * (STAGES - 1), last));
+            if (trip < my_steps) compute(stage, kt);
+            stage = stage + 1 == STAGES ? 0 : stage + 1;
+            kt += 32;
         }
     }
     if constexpr (HALVES > 1) {
         // The second half's wavefronts hand over what they have; the first half's add it to theirs.  The buffers
-        // of keys and values are free once everybody has passed the barrier.
-        __syncthreads();
+        // of keys and values are free once every load has landed and everybody has passed the barrier.
+        loads_landed_then_barrier<0>();
         float* handed = reinterpret_cast<float*>(lds_all);
         constexpr int PER_WAVE = SUB * (ND * 256 + 32);               // floats: accumulators (ND x 64 lanes x 4), then max and sum of 16 pairs
         static_assert(4 * PER_WAVE * sizeof(float) <= sizeof(lds_all), "the buffers of keys and values hold what the second half hands over");
@@ -953,6 +986,8 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
         }
         return;
     }
+    // (the loads issued past the end still write LDS: a wavefront ends only when they have landed)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
     for (int u = 0; u < SUB; ++u) {
         float total = run_sum[u];
@@ -1283,8 +1318,9 @@ LSA_EXPORT int lsa_paged_attention(
     g.page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     if (n_tiles > 0) {
 #if LSA_BF16
-        // The plan's entries of `tiles` span what a workgroup takes: 4 or 8 tiles.
+        // The plan's entries of `tiles` span what a workgroup takes: 4 or 8 tiles.  A load brings 8 keys of a value row.
         if (tiles_per_workgroup != 4 && tiles_per_workgroup != 4 * MAX_SUB) return -1;
+        if (page_size % 8 != 0) return -1;
         dim3 tgrid(n_tiles * n_kv * gtiles);
         if (tile_halves != 1 && tile_halves != MAX_HALVES) return -1;
 #define LSA_LAUNCH_TILES(SUB, HALVES) paged_attention_tile_kernel<SUB, HALVES><<<tgrid, 256 * HALVES, 0, stream>>>( \
@@ -1348,7 +1384,8 @@ LSA_EXPORT int lsa_paged_attention(
 }
 
 // Most tiles of 16 pairs that one workgroup of the prompt-portion kernel takes (it also takes 4; the float32 kernel
-// takes 4 only).
+// takes 4 only).  The bfloat16 kernel takes pages of a multiple of 8 keys only (lsa_attention_tile_page_multiple).
+LSA_EXPORT int lsa_attention_tile_page_multiple() { return LSA_BF16 ? 8 : 4; }
 LSA_EXPORT int lsa_attention_workgroup_tiles() {
 #if LSA_BF16
     return 4 * MAX_SUB;

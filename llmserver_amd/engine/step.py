@@ -139,6 +139,7 @@ class ModelRunner:
             self._flip ^= 1
             staging = self._staging[self._flip]
         ctx = StepContext(self.ops, self.device, self.dtype, staging)
+        ctx.page_size = self.cache.page_size
         ctx.fill(token_ids, positions, token_row, row_start, row_len, row_ctx, logit_idx, tables, slots, request_ids)
         return ctx
 

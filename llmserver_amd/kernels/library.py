@@ -25,6 +25,7 @@ _SIGNATURES = {
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, c_int,
                             c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_attention_workgroup_tiles": [],
+    "lsa_attention_tile_page_multiple": [],
     "lsa_attention_tile_halves": [],
     "lsa_attention_most_splits": [],
     "lsa_attention_head_dim": [],

@@ -544,10 +544,14 @@ class HipOps:
             self._attention[key] = library.load(build.attention_module(dtype == torch.bfloat16, head_dim))
         return self._attention[key]
 
-    def attention_workgroup_tiles(self, dtype, head_dim) -> int:
+    def attention_workgroup_tiles(self, dtype, head_dim, page_size=None) -> int:
         """Most tiles of 16 (token, head) pairs that a workgroup of the prompt-portion attention kernel takes together
-        (an entry of a plan's ``tiles`` spans four, or this many)."""
-        return int(self._attention_library(dtype, head_dim).lsa_attention_workgroup_tiles())
+        (an entry of a plan's ``tiles`` spans four, or this many); 0 if that kernel does not take pages of
+        ``page_size`` keys (its loads bring 8 keys of a value row at a time in bfloat16)."""
+        lib = self._attention_library(dtype, head_dim)
+        if page_size is not None and int(page_size) % int(lib.lsa_attention_tile_page_multiple()):
+            return 0
+        return int(lib.lsa_attention_workgroup_tiles())
 
     def attention_tile_min_workgroups(self, dtype) -> int:
         """Workgroups below which a launch of the prompt-portion kernel does not pay.  The float32 kernel's steps are
@@ -604,7 +608,10 @@ class HipOps:
         tiles = plan.get("tiles") if n_tiles else None
         if n_tiles:
             _check(tiles, "plan tiles", torch.int32, (n_tiles, 4))
-            most = self.attention_workgroup_tiles(qkv.dtype, head_dim)
+            most = self.attention_workgroup_tiles(qkv.dtype, head_dim, page_size)
+            if not most:
+                raise ValueError(f"the kernel for prompt portions in workgroups does not take pages of {page_size} keys: "
+                                 "plan this step with attention_workgroup_tiles(dtype, head_dim, page_size), which says so")
             if int(plan.get("tiles_per_workgroup", 0)) not in (4, most):
                 raise ValueError(f"the plan gives a workgroup {plan.get('tiles_per_workgroup')} tiles, this kernel takes 4 or {most}")
         gheads, tokens_per_tile, gtiles = group_tiling(n_q // n_kv)

@@ -341,7 +341,7 @@ class GQAttention(Mixer):
             elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
                 in_workgroup = fixed
         per_workgroup = getattr(ctx.ops, "attention_workgroup_tiles", None)
-        per_workgroup = per_workgroup(ctx.dtype, self.head_dim) if per_workgroup is not None else 0
+        per_workgroup = per_workgroup(ctx.dtype, self.head_dim, getattr(ctx, "page_size", None)) if per_workgroup is not None else 0
         halves = getattr(ctx.ops, "attention_tile_halves", None)
         halves = halves(ctx.dtype, self.head_dim) if halves is not None and per_workgroup else 1
         fewest = getattr(ctx.ops, "attention_tile_min_workgroups", None)

@@ -174,7 +174,7 @@ def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, need
     # workgroup_tiles: None lets the plan choose between the tile counts the kernel offers, 0 keeps every row out of the
     # prompt-portion kernel, 4 or 8 fixes the count.
     from llmserver_amd.parts import attention as attention_module
-    most = ops.attention_workgroup_tiles(dtype, d) if workgroup_tiles is None or workgroup_tiles else 0
+    most = ops.attention_workgroup_tiles(dtype, d, page) if workgroup_tiles is None or workgroup_tiles else 0
     chooser = attention_module._workgroup_tiles_that_pay
     most_halves = ops.attention_tile_halves(dtype, d) if most else 1
     if workgroup_tiles:
@@ -340,13 +340,14 @@ def test_attention_window_edge(ops, dtype, window):
     attention_case(ops, dtype, 4, 2, 32, 8, [1, 9], [700, 400], window=window, seed=window, target_waves=10 ** 6)
 
 
-@pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 2, 48, 12), (32, 8, 128, 16), (5, 1, 80, 20), (20, 1, 16, 4),
-                                                (2, 1, 256, 500), (16, 16, 64, 64)])
+@pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 2, 48, 24), (32, 8, 128, 16), (5, 1, 80, 40), (20, 1, 16, 8),
+                                                (2, 1, 256, 504), (16, 16, 64, 64), (12, 4, 96, 32), (3, 1, 112, 48)])
 @pytest.mark.parametrize("window", [None, 40])
 def test_attention_prompt_portions_in_workgroup_tiles(ops, n_q, n_kv, d, page, window):
     """Long portions of prompts, with and without a prefix, beside decoded tokens: the portions go
     through the kernel whose four wavefronts share the keys they load (bfloat16), with one tile of 16 pairs per
-    wavefront and with two."""
+    wavefront and with two.  Pages of 16 keys or a multiple (a wavefront's quarter of a step lies in one page) and
+    other multiples of 8 (every lane looks its page up)."""
     print(f"attention workgroup tiles {n_q}/{n_kv} d{d} page{page} window {window}", flush=True)
     lens = [333, 1, 200, 97, 1]
     ctxs = [333, 90, 777, 130, 400]
@@ -359,6 +360,29 @@ def test_attention_prompt_portions_in_workgroup_tiles(ops, n_q, n_kv, d, page, w
                 plan, _ = attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d,
                                          workgroup_tiles=per_workgroup, tile_halves=halves)
                 assert (plan.tiles_per_workgroup, plan.tile_halves) == (per_workgroup, halves) and len(plan.tiles) > 0
+
+
+def test_pages_the_workgroup_kernel_does_not_take_go_to_wavefronts_of_their_own(ops):
+    """The bfloat16 prompt-portion kernel fetches 8 keys of a value row at a time: with pages of 4, 12 or 20 keys the
+    plan keeps every row out of it (the kernel library says so), and a plan that does not is refused."""
+    for page in (4, 12, 20):
+        assert ops.attention_workgroup_tiles(torch.bfloat16, 32, page) == 0
+        plan, _ = attention_case(ops, torch.bfloat16, 8, 2, 32, page, [333, 1, 97], [333, 90, 130], seed=page)
+        assert len(plan.tiles) == 0 and len(plan.items) > 0
+    assert ops.attention_workgroup_tiles(torch.bfloat16, 32, 8) > 0 and ops.attention_workgroup_tiles(torch.float32, 32, 12) == 4
+    from llmserver_amd.parts.attention import build_attention_plan
+    plan = build_attention_plan([333], [333], 4, 2, None, workgroup_tiles=4)
+    staged = {"items": torch.zeros((0, 4), dtype=torch.int32, device=DEV), "item_slot": torch.zeros((0,), dtype=torch.int32, device=DEV),
+              "merges": torch.zeros((0, 4), dtype=torch.int32, device=DEV), "tiles": torch.from_numpy(plan.tiles).to(DEV), "n_tiles": len(plan.tiles),
+              "n_items": 0, "n_merges": 0, "n_slots": 0, "tiles_per_workgroup": 4, "tile_halves": 1}
+    qkv = torch.zeros(333, (8 + 2 * 2) * 32, device=DEV, dtype=torch.bfloat16)
+    out = torch.zeros(333, 8 * 32, device=DEV, dtype=torch.bfloat16)
+    keys = torch.zeros(30, 2, 12, 32, device=DEV, dtype=torch.bfloat16)
+    values = torch.zeros(30, 2, 32, 12, device=DEV, dtype=torch.bfloat16)
+    t = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match="does not take pages of 12 keys"):
+        ops.paged_attention(qkv, out, keys, values, torch.zeros((1, 28), dtype=torch.int32, device=DEV), t([0]), t([333]), t([333]), staged,
+                            32 ** -0.5, None, 12, 8, 2, 32, Ctx())
 
 
 @pytest.mark.parametrize("n_q, n_kv, d, page", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 2, 48, 12), (32, 8, 128, 16), (5, 1, 80, 20), (2, 1, 256, 500)])
