@@ -370,7 +370,7 @@ class Engine:
             return 0
         return self.runner.graph_count()
 
-    def calibrate(self, save_to: Optional[str] = None, portions=(24, 32, 48, 64, 96, 128)) -> int:
+    def calibrate(self, save_to: Optional[str] = None, portions=(24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 640, 768, 896, 1024)) -> int:
         """Measure, for this model's shapes, which products go through a hand-written kernel and which through the
         library, for every number of decoding rows up to ``max_batch_size`` and for prompt portions of the given sizes;
         an idle engine only, never part of serving.  The findings join the kernel namespace's table of choices (and the

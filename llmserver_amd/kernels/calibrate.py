@@ -5,8 +5,8 @@
     python -m llmserver_amd.kernels.calibrate --random-config qwen3-8b [...]  (a size the benchmark command knows by name)
 
 Every product shape of the models is timed both ways (a hand-written kernel with what it folds in; the library's
-product and the kernels it would have absorbed) at 1 to ``--max-batch-size`` decoding rows and at prompt portions of
-17 to 128 tokens, and the faster way is written to ``--out`` (default: the table that ships with the package) under
+product and the kernels it would have absorbed; the library's product whole or in ranges of its inner dimension) at 1
+to ``--max-batch-size`` decoding rows and at prompt portions of 17 to 1,024 tokens, and the faster way is written to ``--out`` (default: the table that ships with the package) under
 the GPU's name.  Serving never measures; it reads this table.
 """
 from __future__ import annotations
@@ -50,7 +50,7 @@ def main(argv=None) -> int:
                     raw = json.load(handle)
             raw["num_hidden_layers"] = min(int(raw.get("num_hidden_layers", args.layers)), args.layers)
             model = random_model_on_device(config_from_dict(raw), "cuda", parse_dtype(args.dtype))
-        engine = Engine(model, None, max_new_tokens=1, max_batch_size=args.max_batch_size, max_num_batched_tokens=max(256, args.max_batch_size),
+        engine = Engine(model, None, max_new_tokens=1, max_batch_size=args.max_batch_size, max_num_batched_tokens=max(1024, args.max_batch_size),
                         kv_cache_num_blocks=args.max_batch_size * 8 + 64, kv_cache_block_size=16, enable_prefix_caching=False)
         measured = engine.calibrate(save_to=args.out)
         total += measured

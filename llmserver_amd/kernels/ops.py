@@ -366,12 +366,77 @@ class HipOps:
         return out
 
     SPLIT_ROWS = 128        # most rows the product that leaves partial sums takes (it starts above the few-row kernels')
+    PARTS_ROWS = 1024       # most rows for which the library's product is tried in ranges of the inner dimension
+
+    @staticmethod
+    def _parts_bucket(rows: int) -> int:
+        """One table entry stands for 64 neighbouring numbers of rows up to 256, for 128 beyond."""
+        step = 64 if rows <= 256 else 128
+        return -(-rows // step) * step
+
+    @staticmethod
+    def _in_parts(x, weight, parts: int):
+        """``x @ weight^T`` as ``parts`` products over ranges of the inner dimension, one batched call of the library
+        with float32 results ``[parts, T, out]`` (views only: nothing is copied)."""
+        rows, width = x.shape
+        return torch.bmm(x.view(rows, parts, width // parts).transpose(0, 1),
+                         weight.view(weight.shape[0], parts, width // parts).permute(1, 2, 0), out_dtype=torch.float32)
+
+    def library_parts(self, x, weight) -> int:
+        """In how many ranges of the inner dimension the library's product of these sizes goes, when its result joins
+        the residual stream anyway (the kernel of the sum and the norm adds float32 partial sums up as it goes): 0
+        (whole), 2 or 4.  With a few hundred rows and an inner dimension of many thousands the library's whole product
+        leaves compute units idle (a tile to each, walking all of the inner dimension); as a batched product of
+        ranges it has several times the tiles.  Looked up in the table of choices; measured only inside
+        ``measuring()``."""
+        rows, width = x.shape
+        if not self.consult_choices or not self.split_products or not self.fuse_stream_updates or x.dtype != torch.bfloat16 \
+                or weight.dtype != torch.bfloat16 or not self.SPLIT_ROWS < rows <= self.PARTS_ROWS or not x.is_contiguous() \
+                or not weight.is_contiguous():
+            return 0
+        ways = [parts for parts in (2, 4) if width % (8 * parts) == 0]
+        if not ways:
+            return 0
+        bucket = self._parts_bucket(rows)
+        keys = {parts: choice_key(f"parts{parts}", bucket, weight.shape[0], width, False, False) for parts in ways}
+        known = {parts: self.choices.get(key) for parts, key in keys.items()}
+        if all(value is not None for value in known.values()):
+            return max((parts for parts, best in known.items() if best), default=0)
+        if not self._measuring or torch.cuda.is_current_stream_capturing():
+            return 0
+        stream = torch.zeros((rows, weight.shape[0]), device=x.device, dtype=x.dtype)
+        norm_weight = torch.ones(weight.shape[0], device=x.device, dtype=torch.float32)
+        normed = torch.empty_like(stream)
+        saved, self.consult_choices = self.consult_choices, False
+        try:
+            overhead = self._replay_cost()
+            times = {0: self._median_time(lambda: self.add_rmsnorm(stream, torch.mm(x, weight.t()), norm_weight, 1e-6, normed)) - overhead}
+            for parts in ways:
+                times[parts] = self._median_time(
+                    lambda: self.add_rmsnorm(stream, self._in_parts(x, weight, parts), norm_weight, 1e-6, normed)) - overhead
+            best = min(ways, key=lambda parts: times[parts])
+            if times[best] >= self.LIBRARY_MARGIN * times[0]:
+                best = 0
+        except RuntimeError as error:
+            import warnings
+            warnings.warn(f"timing the library's product in parts failed ({error!r}); keeping it whole")
+            best = 0
+        finally:
+            self.consult_choices = saved
+        for parts, key in keys.items():
+            self.choices.record(key, parts == best)
+        return best
 
     def linear_partial_sums(self, x, weight, few_rows_too=False):
         """``x @ weight^T`` for 17 to 128 rows (fewer if ``few_rows_too``) as float32 partial sums ``[parts, T, out]``
         over ranges of the inner dimension (their sum is the product), or None if this is no case for it.  Whoever
-        adds the result to the residual stream adds the parts up (:meth:`add_rmsnorm` takes them)."""
+        adds the result to the residual stream adds the parts up (:meth:`add_rmsnorm` takes them).  Beyond 128 rows
+        the library multiplies, in ranges where the table of choices says that this is faster (see
+        :meth:`library_parts`)."""
         rows, width = x.shape
+        if rows > self.SPLIT_ROWS and x.shape[1] == weight.shape[1]:
+            parts = self.library_parts(x, weight)      # beyond this repository's product: the library's, whole or in ranges
+            return self._in_parts(x, weight, parts) if parts else None
         if not ((0 if few_rows_too else self.skinny_rows) < rows <= self.SPLIT_ROWS) or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
                 or x.shape[1] != weight.shape[1] or not self.split_products:
             return None

@@ -657,6 +657,53 @@ def test_gated_product_beyond_few_rows(ops, rows, inter, k):
     assert ops._gemm.lsa_gemm_split_gated(x.data_ptr(), w.data_ptr(), x.data_ptr(), 16, inter, k, None) == -1
 
 
+def test_library_product_in_ranges_of_the_inner_dimension_by_table(ops):
+    """A product of a few hundred rows whose result joins the residual stream goes through the library whole, or as a
+    batched product of two or four ranges of the inner dimension with float32 results, as the table of choices says;
+    unknown shapes go whole and nothing is timed unless the caller is inside ``measuring()``.  Either way the sums that
+    reach the stream are right."""
+    from llmserver_amd.kernels.choices import ChoiceTable, choice_key
+    print("library product in ranges by table", flush=True)
+    torch.manual_seed(9)
+    rows, out, width = 200, 320, 1536
+    x = torch.randn(rows, width, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(out, width, device=DEV) / width ** 0.5).to(torch.bfloat16)
+    expected = (x.double() @ w.double().t()).float()
+    keys = {parts: choice_key(f"parts{parts}", 256, out, width, False, False) for parts in (2, 4)}
+    bucket = type(ops)._parts_bucket
+    assert bucket(129) == 192 and bucket(256) == 256 and bucket(257) == 384 and bucket(1024) == 1024
+    saved_table, ops.choices = ops.choices, ChoiceTable(ops.choices.device_name)
+    ops.consult_choices = True
+    try:
+        assert ops.library_parts(x, w) == 0 and ops.linear_partial_sums(x, w) is None and not ops.choices.entries
+        for best in (2, 4, 0):
+            for parts, key in keys.items():
+                ops.choices.entries[key] = parts == best
+            assert ops.library_parts(x, w) == best
+            sums = ops.linear_partial_sums(x, w)
+            if not best:
+                assert sums is None
+                continue
+            assert sums.shape == (best, rows, out) and sums.dtype == torch.float32
+            torch.testing.assert_close(sums.sum(0), expected, atol=2e-3, rtol=2e-3)
+            stream = torch.randn(rows, out, device=DEV).to(torch.bfloat16)
+            before = stream.float()
+            normed = torch.empty_like(stream)
+            ops.add_rmsnorm(stream, sums, torch.ones(out, device=DEV), 1e-6, normed)
+            torch.testing.assert_close(stream.float(), (before + expected).to(torch.bfloat16).float(), atol=2e-2, rtol=1e-2)
+        assert ops.library_parts(x[:, :1532].contiguous(), w[:, :1532].contiguous()) == 0       # ranges must be multiples of 8
+        assert ops.library_parts(x[:100], w) == 0 and ops.library_parts(torch.zeros(1100, width, device=DEV, dtype=torch.bfloat16), w) == 0
+        ops.choices = ChoiceTable(ops.choices.device_name)
+        with ops.measuring():
+            chosen = ops.library_parts(x, w)
+        assert chosen in (0, 2, 4) and set(ops.choices.measured) == set(keys.values())
+        assert [ops.choices.entries[keys[parts]] for parts in (2, 4)] == [chosen == 2, chosen == 4]
+        assert ops.library_parts(x, w) == chosen and ops._flush is None
+    finally:
+        ops.choices = saved_table
+        ops.consult_choices = False
+
+
 def test_few_row_kernel_or_library_by_table(ops, tmp_path):
     """A shape goes the way the table of choices says; a shape the table does not know goes the few-row kernel's way
     and nothing is timed, unless the caller is inside ``measuring()``: then it is timed once, entered into the table
