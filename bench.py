@@ -11,7 +11,7 @@ is decoded tokens per second; ``prefill`` times one engine step that takes a 2,0
 its arrival to its first token; ``roofline`` relates the bytes a decode step has to read (every
 weight once, plus the cache of the live requests) to the published HBM bandwidth; ``points`` holds
 batch 1 and 64 of the same model (tokens per second, with the step's milliseconds and its share of
-the HBM peak beside them) and, unless ``--no-extra-points``, the two other workloads the baseline
+the HBM peak beside them), prompts of 512 and 8,192 tokens and four requests at a context of 16,384, and, unless ``--no-extra-points``, the two other workloads the baseline
 names: 64 mixed requests with a shared prefix on Qwen3-1.7B sizes, and batch 16 behind 8,192 tokens
 on Qwen3-32B sizes.  Token ids are seeded uniform random numbers (synthetic data), weights seeded normal.
 """
@@ -212,6 +212,17 @@ def main() -> int:
             points[f"decode_b{batch}"] = round(rate, 2)
             points[f"decode_b{batch}_ms_per_step"] = round(ms, 4)
             points[f"decode_b{batch}_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
+        # further sizes of the same model: a short and a long prompt, and a few requests far into their contexts
+        for tokens in (512, 8192):
+            log(f"[bench] prefill of {tokens} tokens")
+            seconds = prefill_through_engine(model, args.page_size, tokens)
+            points[f"prefill_{tokens}_ms"] = round(1000.0 * seconds, 3)
+            points[f"prefill_{tokens}_mfma_frac"] = round(prefill_flops(config, tokens) / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)
+        log("[bench] decode batch 4 at a context of 16,384")
+        rate, ms, gbs = decode_point(model, config, elem, args.page_size, 4, 16384, 32, 4)
+        points["decode_b4_ctx16384"] = round(rate, 2)
+        points["decode_b4_ctx16384_ms_per_step"] = round(ms, 4)
+        points["decode_b4_ctx16384_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
     del model
     torch.cuda.empty_cache()
     if not args.no_points and not args.no_extra_points and dtype == torch.bfloat16 and not args.layers:
