@@ -42,3 +42,29 @@ def test_matrix_one_prompt_and_mixed_workload(tmp_path, capsys):
     tables = (tmp_path / "kernels.txt").read_text()
     assert "decode batch=1 graphs=True" in tables and "decode batch=6 graphs=False" in tables and "prefill prompt=40" in tables
     assert "paged_attention" in tables and "gemm_skinny" in tables           # this repository's kernels, by name, with their times
+
+
+def test_bench_prints_one_line_with_every_part_and_refuses_more_gpus():
+    """``bench.py`` as the driver runs it, on two layers of the benchmark's sizes so that it takes seconds: one JSON line
+    whose parts are all there (value, roofline, prefill, points at further sizes); more than one GPU: one line, exit 2."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    print("bench.py on two layers", flush=True)
+    done = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--layers", "2", "--steps", "4", "--warmup", "1", "--context", "256"],
+                          capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    lines = [line for line in done.stdout.splitlines() if line.strip()]
+    assert len(lines) == 1
+    record = json.loads(lines[0])
+    assert record["n_gpus"] == 1 and record["steps"] == 4 and record["warmup"] == 1 and record["value"] > 0 and record["unit"] == "tokens/s"
+    assert record["config"]["layers"] == 2 and record["config"]["layers_full"] == 36 and len(record["config"]) <= 20
+    assert all(not isinstance(value, (dict, list)) for value in record["config"].values())
+    assert record["roofline"]["bound"] == "hbm" and 0 < record["roofline"]["frac"] < 1
+    assert record["prefill"]["tokens"] == 2048 and record["prefill"]["ms"] > 0 and 0 < record["prefill"]["frac"] < 1
+    for key in ("decode_b1", "decode_b64", "decode_b64_ms_per_step", "prefill_512_ms", "prefill_8192_ms", "decode_b4_ctx16384"):
+        assert record["points"][key] > 0, key
+    assert not any(key.startswith("mixed_") for key in record["points"])       # fewer layers: the other models' points are left out
+    more = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert more.returncode == 2 and len(more.stdout.strip().splitlines()) == 1
