@@ -612,10 +612,11 @@ constexpr int K_BLOCK_CHUNKS = (16 * K_ROW_SLOTS + 63) / 64, V_BLOCK_CHUNKS = (D
 constexpr int K_BLOCK_BYTES = 1024 * K_BLOCK_CHUNKS, V_BLOCK_BYTES = 1024 * V_BLOCK_CHUNKS;
 constexpr int K_TILE_BYTES = 2 * K_BLOCK_BYTES, STEP_BYTES = K_TILE_BYTES + 2 * V_BLOCK_BYTES;
 constexpr int STEP_LOADS = K_BLOCK_CHUNKS > V_BLOCK_CHUNKS ? K_BLOCK_CHUNKS : V_BLOCK_CHUNKS;     // of a wavefront per step
-// Buffers in the ring: three where two workgroups of them still fit a compute unit's 160 KB (loads then run two steps
-// ahead of the products), else two.
+// Buffers in the ring: two (the loads of step i + 1 are under way while step i is multiplied).  A third, with the loads
+// two steps ahead, was measured and gains nothing where the registers bound the wavefronts per SIMD, and costs the
+// third workgroup per compute unit that the form with four tiles otherwise has room for (2,048 x 2,048: 95 against 78 us).
 #ifndef LSA_TILE_STAGES
-#define LSA_TILE_STAGES (2 * 3 * STEP_BYTES <= 160 * 1024 ? 3 : 2)
+#define LSA_TILE_STAGES 2
 #endif
 constexpr int STAGES = LSA_TILE_STAGES;
 // Tiles of 16 pairs per wavefront (SUB): with two, every key and value operand read from LDS feeds two products, which

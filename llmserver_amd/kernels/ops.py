@@ -103,7 +103,7 @@ class HipOps:
         halves shorten the longest workgroup's walk but make every step dearer)."""
         if self._tuning is None:
             units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-            costs = (((False, 1), TileLaunchCost(3.2, 0.89, 1.85)), ((True, 1), TileLaunchCost(8.7, 0.94, 2.45)),
+            costs = (((False, 1), TileLaunchCost(3.2, 0.89, 1.55)), ((True, 1), TileLaunchCost(8.7, 0.94, 2.45)),
                      ((False, 2), TileLaunchCost(3.3, 1.11, 2.08)), ((True, 2), TileLaunchCost(8.8, 1.44, 2.84)))
             self._tuning = AttentionTuning(target_waves=4 * units, tile_costs=costs)
         return self._tuning
