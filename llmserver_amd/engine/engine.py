@@ -120,9 +120,8 @@ class Engine:
                              "yield_s": 0.0, "tokens": 0, "prefix_hit_tokens": 0, "preemptions": 0,
                              "decode_by_rows": {}}       # decoding rows of a step -> [steps, seconds] (utils/engine.py:69, 468-471)
         ops = ops if ops is not None else self._default_ops()
-        check = getattr(ops, "check_cache_geometry", None)
-        if check is not None:                        # what the kernels cannot take is refused here, not at the first step
-            check(model.cache_specs(), config.kv_cache_block_size)
+        # what the kernels cannot take is refused here, not at the first step
+        ops.check_cache_geometry(model.cache_specs(), config.kv_cache_block_size)
         self.kv_cache = CacheManager(model.cache_specs(), config.kv_cache_block_size, config.kv_cache_num_blocks,
                                      num_state_slots=config.max_batch_size, device=self.device, dtype=self.dtype,
                                      model_identity=str(getattr(model, "name", "model")))
@@ -376,15 +375,17 @@ class Engine:
         an idle engine only, never part of serving.  The findings join the kernel namespace's table of choices (and the
         file ``save_to``, if given, which ``LLMSERVER_AMD_CHOICES`` can name in later runs).  Returns how many shapes
         were measured.  Graphs captured before are dropped: they may hold the other choice."""
-        measuring = getattr(self.runner.ops, "measuring", None)
-        if measuring is None or self.active_requests:
+        if self.active_requests:
             return 0
+        measuring = self.runner.ops.measuring
         most = self.scheduler.max_batch_size
         sizes = [(rows, 1) for rows in range(1, most + 1)]
         sizes += [(1, tokens) for tokens in portions if tokens <= self.max_num_batched_tokens]
         graphs, self.runner.use_graphs = self.runner.use_graphs, False
         try:
             with measuring() as choices:
+                if choices is None:                  # a kernel namespace that keeps no table of choices
+                    return 0
                 before = len(choices.measured)
                 for rows, tokens in sizes:
                     if rows * -(-tokens // self.block_size) > min(self.kv_cache.available_pages() or [1 << 30]):

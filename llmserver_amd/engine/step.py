@@ -63,7 +63,7 @@ class ModelRunner:
         self.vocab = model.head.out_features
         graph_safe = all(block.mixer.graph_safe for block in model.blocks) and not cache.state_specs
         if use_graphs is None:
-            use_graphs = self.device.type == "cuda" and getattr(ops, "name", "") == "hip"
+            use_graphs = self.device.type == "cuda" and ops.name == "hip"
         self.use_graphs = bool(use_graphs and graph_safe)
         self._graphs: "OrderedDict[tuple, _CapturedStep]" = OrderedDict()
         self.graph_replays = 0

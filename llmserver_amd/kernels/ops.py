@@ -12,6 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..parts.attention import AttentionTuning, TileLaunchCost, group_tiling
+from ..parts.kernel_namespace import KernelNamespace
 from . import build, library
 from .choices import ChoiceTable, choice_key
 
@@ -57,7 +58,7 @@ def _launched(code: int, what: str):
         raise RuntimeError(f"launch of {what} failed with HIP error {code}")
 
 
-class HipOps:
+class HipOps(KernelNamespace):
     """Kernel namespace handed to the parts through the step context."""
 
     name = "hip"

@@ -26,6 +26,7 @@ from typing import Optional, Tuple
 import numpy as np
 
 from .base import VECTOR, Mixer, PagedKVSpec, ParamSpec, PositionEncoding
+from .kernel_namespace import tuning_of
 from .linear import Linear
 
 TILE_ROWS = 16          # rows of (token, group head) pairs one wavefront handles (MFMA N dimension)
@@ -326,7 +327,7 @@ class GQAttention(Mixer):
         if ctx.has_plan(key):
             return
         fixed = None
-        tuning = getattr(ctx.ops, "attention_tuning", None) or DEFAULT_TUNING
+        tuning = tuning_of(ctx.ops, DEFAULT_TUNING)
         if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
             fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves)
         # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:
@@ -340,12 +341,9 @@ class GQAttention(Mixer):
                 in_workgroup = fixed = WORKGROUP_RANGES
             elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
                 in_workgroup = fixed
-        per_workgroup = getattr(ctx.ops, "attention_workgroup_tiles", None)
-        per_workgroup = per_workgroup(ctx.dtype, self.head_dim, getattr(ctx, "page_size", None)) if per_workgroup is not None else 0
-        halves = getattr(ctx.ops, "attention_tile_halves", None)
-        halves = halves(ctx.dtype, self.head_dim) if halves is not None and per_workgroup else 1
-        fewest = getattr(ctx.ops, "attention_tile_min_workgroups", None)
-        fewest = fewest(ctx.dtype) if fewest is not None and per_workgroup else 0
+        per_workgroup = ctx.ops.attention_workgroup_tiles(ctx.dtype, self.head_dim, getattr(ctx, "page_size", None))
+        halves = ctx.ops.attention_tile_halves(ctx.dtype, self.head_dim) if per_workgroup else 1
+        fewest = ctx.ops.attention_tile_min_workgroups(ctx.dtype) if per_workgroup else 0
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
                                     target_waves=tuning.target_waves, fixed_splits=fixed, workgroup_tiles=per_workgroup,
                                     merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves, tile_min_workgroups=fewest)
@@ -363,11 +361,10 @@ class GQAttention(Mixer):
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
         cos_sin = self.position.cos_sin(ctx)
         # A step of single tokens: the attention kernel does the norm, the rotation and the cache write itself.
-        fits = getattr(ctx.ops, "decode_fusion_fits", None)
         fusion = None
         # (the kernel that merges a tile's key ranges in its workgroup fuses only the whole of norm and rotation)
         whole = self.q_norm_weight is not None and cos_sin is not None
-        if fits is not None and ctx.n_tokens == ctx.n_rows and fits(qkv.dtype, self.head_dim) \
+        if ctx.n_tokens == ctx.n_rows and ctx.ops.decode_fusion_fits(qkv.dtype, self.head_dim) \
                 and (whole or not ctx.get_plan(self.plan_key()).get("merge_in_workgroup")):
             fusion = (self.q_norm_weight, self.k_norm_weight, eps, cos_sin, cache.writable)
         else:

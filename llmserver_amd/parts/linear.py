@@ -70,13 +70,12 @@ class Linear(Part):
         come back as a :class:`StreamUpdate`: already added to the residual stream, the following norm prepared
         or carried out."""
         ops = ctx.ops
-        fused = getattr(ops, "fuse_stream_updates", False)
+        fused = ops.fuse_stream_updates
         row_scale = None
         if isinstance(x, PendingNorm):
             scaled = x.row_scale() if fused else None
-            library_is_faster = getattr(ops, "library_is_faster", None)
-            if scaled is not None and ops.row_scale_fits(scaled[0], self.weight, scaled[1]) and not (
-                    library_is_faster is not None and library_is_faster("plain", scaled[0], self.weight, True, self.out_float32)):
+            if scaled is not None and ops.row_scale_fits(scaled[0], self.weight, scaled[1]) \
+                    and not ops.library_is_faster("plain", scaled[0], self.weight, True, self.out_float32):
                 x, row_scale = scaled            # the norm becomes a scale of the product's rows
             else:
                 x = x.tensor()
@@ -84,20 +83,18 @@ class Linear(Part):
         if following is not None:
             # The product may leave its result as partial sums, which the kernel of the sum and the norm adds up on
             # its way: that is the way of 17 rows and more, and of fewer where it has been measured to be faster.
-            partial_sums = getattr(ops, "linear_partial_sums", None)
-            split_few_rows = partial_sums is not None and row_scale is None and getattr(ops, "partial_sums_are_faster", None) is not None \
-                and ops.partial_sums_are_faster(x, self.weight)
+            split_few_rows = row_scale is None and ops.partial_sums_are_faster(x, self.weight)
             if not split_few_rows:
                 done = ops.linear_into_stream(x, self.weight, sink.stream(), following[0], row_scale=row_scale)
                 if done is not None:
                     return StreamUpdate(sink.norm, *done)
             sums = None
-            if partial_sums is not None and row_scale is None:
-                sums = partial_sums(x, self.weight, few_rows_too=True) if split_few_rows else partial_sums(x, self.weight)
+            if row_scale is None:
+                sums = ops.linear_partial_sums(x, self.weight, few_rows_too=split_few_rows)
             if sums is not None:
                 stream = sink.stream()
                 return StreamUpdate(sink.norm, stream, normed=sink.norm.add_norm(stream, sums, ctx))
-        if self.bias is not None and getattr(ops, "fuses_bias", False):
+        if self.bias is not None and ops.fuses_bias:
             # The bias joins the product's float32 sums, which are then rounded once.
             if row_scale is not None:
                 return ops.linear_few_rows(x, self.weight, out=out, out_float32=self.out_float32, row_scale=row_scale, bias=self.bias)

@@ -55,18 +55,17 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, ctx, sink=None):
         ops = ctx.ops
-        gated = getattr(ops, "linear_gated", None)
-        if gated is not None and self.gate_up.bias is None:
+        if self.gate_up.bias is None:
             # Few rows: one launch for both products with the activation in its epilogue.
             row_scale = None
             tensor = x
             if isinstance(x, PendingNorm):
-                scaled = x.row_scale() if getattr(ops, "fuse_stream_updates", False) else None
+                scaled = x.row_scale() if ops.fuse_stream_updates else None
                 if scaled is not None and ops.row_scale_fits(scaled[0], self.gate_up.weight, scaled[1]):
                     tensor, row_scale = scaled
                 else:
                     tensor = x.tensor()
-            hidden = gated(tensor, self.gate_up.weight, row_scale=row_scale)
+            hidden = ops.linear_gated(tensor, self.gate_up.weight, row_scale=row_scale)
             if hidden is not None:
                 return self.down.forward(hidden, ctx, sink=sink)
             if row_scale is not None:

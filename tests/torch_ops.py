@@ -10,9 +10,10 @@ from __future__ import annotations
 import torch
 
 from llmserver_amd.parts.attention import group_tiling  # noqa: F401  (kept for symmetry of imports)
+from llmserver_amd.parts.kernel_namespace import KernelNamespace
 
 
-class TorchOps:
+class TorchOps(KernelNamespace):
     """``fused=True`` also offers the twins of the fused kernels (sum and norm folded into the few-row products, q/k
     norm, rotation and cache write inside the attention of single-token steps), for any type and size, so that the
     parts' fused dataflow runs on the CPU as it does on the GPU."""
