@@ -1,0 +1,73 @@
+"""The calls that the parts, the step function and the engine make on ``ctx.ops`` are the methods of
+``parts.KernelNamespace``: the shipped HIP namespace and the tests' torch twins both answer the required ones, and a
+namespace that offers nothing beyond them (the base class's neutral answers) still runs a model."""
+import inspect
+import re
+import os
+
+import torch
+
+from llmserver_amd.parts import KernelNamespace
+from torch_ops import TorchOps
+
+REQUIRED = ("linear", "embedding", "add_rmsnorm", "swiglu", "add_bias_", "rotary_table", "qk_norm_rope_kv_write", "paged_attention", "sample")
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_both_namespaces_answer_what_must_be_answered():
+    from llmserver_amd.kernels.ops import HipOps
+    for cls in (HipOps, TorchOps):
+        assert issubclass(cls, KernelNamespace)
+        for name in REQUIRED:
+            assert getattr(cls, name) is not getattr(KernelNamespace, name), (cls.__name__, name)
+    for name in REQUIRED:                       # the base class refuses them
+        method = getattr(KernelNamespace(), name)
+        arguments = [None] * len([p for p in inspect.signature(method).parameters.values() if p.default is p.empty])
+        try:
+            method(*arguments)
+        except NotImplementedError:
+            continue
+        raise AssertionError(f"KernelNamespace.{name} should be abstract")
+
+
+def test_every_call_on_ops_in_the_package_is_named_by_the_interface():
+    """No caller outside the kernels' own folder uses a method that the interface does not name, and none asks
+    whether a method exists."""
+    used = set()
+    for folder in ("parts", "models", "engine", "sampling", "cache"):
+        for base, _, files in os.walk(os.path.join(ROOT, "llmserver_amd", folder)):
+            for file in files:
+                if file.endswith(".py"):
+                    text = open(os.path.join(base, file)).read()
+                    assert not re.search(r"(getattr|hasattr)\([^)]*\bops\b", text), (file, "asks whether the namespace has something")
+                    used.update(re.findall(r"\bops\.([A-Za-z_]\w*)", text))
+    used -= {"py"}                                # (a file name in a comment)
+    missing = sorted(name for name in used if not hasattr(KernelNamespace, name))
+    assert not missing, missing
+
+
+def test_a_namespace_that_offers_nothing_runs_a_model():
+    """The torch twins with every offer withdrawn (the base class's answers) give the same logits as with them."""
+    import numpy as np
+    from helpers import model_folder
+    from llmserver_amd.engine.replay import make_runner
+    from llmserver_amd.engine.step import StepEntry
+
+    class Bare(TorchOps):
+        row_scale_fits = KernelNamespace.row_scale_fits
+        linear_few_rows = KernelNamespace.linear_few_rows
+        linear_into_stream = KernelNamespace.linear_into_stream
+        linear_partial_sums = KernelNamespace.linear_partial_sums
+        linear_gated = KernelNamespace.linear_gated
+        decode_fusion_fits = KernelNamespace.decode_fusion_fits
+
+    outs = []
+    for ops in (TorchOps(fused=True), Bare(fused=False)):
+        runner = make_runner(model_folder("A"), "float32", 128, 16, device="cpu", ops=ops)
+        runner.cache.open("r")
+        runner.cache.ensure("r", 9)
+        first = runner.step([StepEntry("r", [3, 1, 4, 1, 5, 9, 2, 6], [7])])
+        runner.cache.advance("r", 8)
+        second = runner.step([StepEntry("r", [5], [0])])
+        outs.append(np.concatenate([first.float().cpu().numpy(), second.float().cpu().numpy()]))
+    np.testing.assert_allclose(outs[0], outs[1], atol=2e-5, rtol=1e-5)
