@@ -337,11 +337,11 @@ class GQAttention(Mixer):
         #    of one tile leave wavefronts idle through the others' walk: a tenth slower at 64 rows behind 4,096 tokens.)
         in_workgroup = 0
         if ctx.n_tokens == ctx.n_rows:
-            if getattr(ctx, "short_contexts", False):
+            if ctx.short_contexts:
                 in_workgroup = fixed = WORKGROUP_RANGES
             elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
                 in_workgroup = fixed
-        per_workgroup = ctx.ops.attention_workgroup_tiles(ctx.dtype, self.head_dim, getattr(ctx, "page_size", None))
+        per_workgroup = ctx.ops.attention_workgroup_tiles(ctx.dtype, self.head_dim, ctx.page_size)
         halves = ctx.ops.attention_tile_halves(ctx.dtype, self.head_dim) if per_workgroup else 1
         fewest = ctx.ops.attention_tile_min_workgroups(ctx.dtype) if per_workgroup else 0
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
