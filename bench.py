@@ -11,7 +11,8 @@ is decoded tokens per second; ``prefill`` times one engine step that takes a 2,0
 its arrival to its first token; ``roofline`` relates the bytes a decode step has to read (every
 weight once, plus the cache of the live requests) to the published HBM bandwidth; ``points`` holds
 batch 1 and 64 of the same model (tokens per second, with the step's milliseconds and its share of
-the HBM peak beside them), prompts of 512 and 8,192 tokens and four requests at a context of 16,384, and, unless ``--no-extra-points``, the two other workloads the baseline
+the HBM peak beside them), prompts of 512 and 8,192 tokens, a prompt of which all but the last 128 tokens lie in the cache already (8,064 of them: the next turn
+of a conversation) and four requests at a context of 16,384, and, unless ``--no-extra-points``, the two other workloads the baseline
 names: 64 mixed requests with a shared prefix on Qwen3-1.7B sizes, and batch 16 behind 8,192 tokens
 on Qwen3-32B sizes.  Token ids are seeded uniform random numbers (synthetic data), weights seeded normal.
 """
@@ -145,6 +146,38 @@ def prefill_through_engine(model, page_size, tokens, repeats=3, seed=1):
     return best
 
 
+def turn_through_engine(model, page_size, cached, fresh, repeats=3, seed=2):
+    """Seconds of the one engine step that takes a prompt whose first ``cached`` tokens lie in the cache already (an
+    earlier request left them there) and whose last ``fresh`` tokens are new to its first token: the next turn of a
+    conversation.  Best of ``repeats``."""
+    import torch
+
+    from llmserver_amd.engine import Engine
+    engine = Engine(model, None, max_new_tokens=1, max_batch_size=1, max_num_batched_tokens=max(cached, fresh),
+                    kv_cache_num_blocks=2 * (-(-(cached + fresh) // page_size)) + 8, kv_cache_block_size=page_size, stream_text=False,
+                    max_completed_requests=0, ignore_eos=True, enable_prefix_caching=True)
+    generator = torch.Generator().manual_seed(seed)
+    vocab = model.config.vocab_size
+    earlier = torch.randint(0, vocab, (cached,), generator=generator).tolist()
+    engine.add_request(None, prompt_token_ids=earlier)
+    while engine.step():
+        pass
+    best = float("inf")
+    for attempt in range(repeats + 1):
+        request = engine.add_request(None, prompt_token_ids=earlier + torch.randint(0, vocab, (fresh,), generator=generator).tolist())
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        more = engine.step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+        assert not more and len(request.generated_token_ids) == 1, "the earlier turn's pages were not found in the cache"
+        if attempt:
+            best = min(best, elapsed)
+    del engine
+    torch.cuda.empty_cache()
+    return best
+
+
 def decode_point(model, config, elem, page_size, batch, context, steps, warmup):
     seconds, _ = decode_through_engine(model, page_size, batch, context, steps, warmup)
     ms = 1000.0 * seconds / steps
@@ -218,6 +251,8 @@ def main() -> int:
             seconds = prefill_through_engine(model, args.page_size, tokens)
             points[f"prefill_{tokens}_ms"] = round(1000.0 * seconds, 3)
             points[f"prefill_{tokens}_mfma_frac"] = round(prefill_flops(config, tokens) / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)
+        log("[bench] 128 new tokens behind 8,064 cached ones")
+        points["turn_128_after_8064_ms"] = round(1000.0 * turn_through_engine(model, args.page_size, 8064, 128), 3)
         log("[bench] decode batch 4 at a context of 16,384")
         rate, ms, gbs = decode_point(model, config, elem, args.page_size, 4, 16384, 32, 4)
         points["decode_b4_ctx16384"] = round(rate, 2)

@@ -102,6 +102,7 @@ class CacheManager:
         self.page_size = page_size
         self.device, self.dtype = device, dtype
         self.model_identity = model_identity
+        self._identity_bytes = str(model_identity).encode("utf-8")
         self.groups: List[CacheGroup] = []
         self.group_of_cache: Dict[int, int] = {}
         self.layer_in_group: Dict[int, int] = {}
@@ -280,15 +281,22 @@ class CacheManager:
     def digest(self, parent: str, tokens: Sequence[int]) -> str:
         """Chained sha256 over (parent digest, page tokens, model, adapter), root parent "root"
         (utils/engine.py:193-195)."""
-        payload = json.dumps([parent, list(tokens), self.model_identity, "none"], separators=(",", ":")).encode("utf-8")
-        return hashlib.sha256(payload).hexdigest()
+        return self._digest(parent, np.asarray(tokens, dtype=np.int64).tobytes())
+
+    def _digest(self, parent: str, page_tokens: bytes) -> str:
+        # (the tokens as 64-bit integers, the rest as text; the lengths of the parts are fixed or delimited, so no two
+        # different inputs give the same bytes)
+        return hashlib.sha256(b"%s|%d|%s|%s|none" % (parent.encode("ascii"), len(page_tokens), page_tokens, self._identity_bytes)).hexdigest()
 
     def prefix_digests(self, prompt: Sequence[int]) -> List[str]:
         """The chained digests of the prompt's complete pages that may be shared (at least one
         prompt token always remains to be computed)."""
         digests, parent = [], "root"
-        for block in range((len(prompt) - 1) // self.page_size):
-            parent = self.digest(parent, prompt[block * self.page_size:(block + 1) * self.page_size])
+        blocks = (len(prompt) - 1) // self.page_size
+        data = np.asarray(prompt[:blocks * self.page_size], dtype=np.int64).tobytes()       # converted once, not page by page
+        page_bytes = 8 * self.page_size
+        for block in range(blocks):
+            parent = self._digest(parent, data[block * page_bytes:(block + 1) * page_bytes])
             digests.append(parent)
         return digests
 
@@ -306,11 +314,12 @@ class CacheManager:
         if digests is None:
             digests = self.prefix_digests(prompt)
         covered = 0
+        listed = [set(record.tables[group.index]) for group in self.groups]      # (a table never lists a page twice)
         for digest in digests[have:]:
             if any(group.pool.lookup(digest) is None for group in self.groups):
                 break
             for group in self.groups:
-                group.pool.adopt(digest, record.tables[group.index])
+                group.pool.adopt(digest, record.tables[group.index], listed[group.index])
             covered += self.page_size
         record.num_computed += covered
         return covered

@@ -183,15 +183,19 @@ class PagePool:
             return None
         return page
 
-    def adopt(self, digest: str, table: List[int]) -> Optional[int]:
-        """Append the page published under ``digest`` to ``table``; None if there is none."""
+    def adopt(self, digest: str, table: List[int], listed: Optional[set] = None) -> Optional[int]:
+        """Append the page published under ``digest`` to ``table``; None if there is none.  ``listed``: the pages of
+        ``table`` as a set, kept up to date here (who adopts many pages in a row passes it, so that the look whether
+        the table has the page already does not walk the table each time)."""
         page = self.lookup(digest)
         if page is None:
             return None
-        if page in table:
+        if page in (table if listed is None else listed):
             raise ValueError(f"page {page} is already in this block table")
         self.hold(page)
         table.append(page)
+        if listed is not None:
+            listed.add(page)
         return page
 
     # -- self-check ----------------------------------------------------------------------------

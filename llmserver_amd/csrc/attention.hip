@@ -660,13 +660,22 @@ __device__ __forceinline__ void loads_landed_then_barrier() {
 // (the tiles that see the most keys) then walks half as many steps: a launch with few workgroups, which that
 // workgroup bounds, ends sooner.  Both halves make the same number of trips through the loop (one of them may
 // have a step less to compute), so that they meet at the same barriers.
+//
+// Key ranges: a plan may give the tiles of a workgroup a part of their keys only and the other parts to other
+// workgroups (rows of few tiles behind long contexts: few workgroups, each with a long walk).  `tile_slots[i]` then
+// names where entry i leaves its partial results, in the form the wavefront kernel leaves them (accumulators, running
+// maximum in natural-logarithm units, sum): tile j of the workgroup writes slot `first + j * stride`, and `merge`
+// combines a tile's slots.  first < 0 (or no `tile_slots` at all): the entry holds all keys and writes the output.
+struct TileSlots { int first, stride; };
+
 template <int SUB, int HALVES>
 __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_attention_tile_kernel(
     const elem_t* __restrict__ q, long q_token_stride, elem_t* __restrict__ out,
     const elem_t* __restrict__ keys, const elem_t* __restrict__ values,
     const int* __restrict__ table, int table_stride,
     const int* __restrict__ row_start, const int* __restrict__ row_len, const int* __restrict__ row_ctx,
-    const Item* __restrict__ tiles, Geometry g) {
+    const Item* __restrict__ tiles, const TileSlots* __restrict__ tile_slots, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    Geometry g) {
     __shared__ __attribute__((aligned(1024))) unsigned char lds_all[HALVES * STAGES * STEP_BYTES];
     const int half = HALVES > 1 ? __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) : 0;     // (the same in all lanes, and known to be)
     const int lds_base = half * STAGES * STEP_BYTES;                  // this half's ring of buffers
@@ -936,6 +945,9 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
             kt += 32;
         }
     }
+    // Where this entry's results go: the output, or a slot per tile (asked for here, at the end, where it is needed).
+    TileSlots slots = {-1, 0};
+    if (tile_slots != nullptr) slots = tile_slots[blockIdx.x / heads];
     if constexpr (HALVES > 1) {
         // The second half's wavefronts hand over what they have; the first half's add it to theirs.  The buffers
         // of keys and values are free once every load has landed and everybody has passed the barrier.
@@ -974,6 +986,20 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
             const float w1 = other_max == NEG_INF ? 0.f : __builtin_amdgcn_exp2f((other_max - top) * scale_log2);
             const float total = w0 * run_sum[u] + w1 * other_sum;
             if (!pair_valid[u]) continue;
+            if (slots.first >= 0) {
+                const size_t base = ((size_t)(slots.first + (wave * SUB + u) * slots.stride) * heads + head_index) * 16 + col;
+                float* pa = part_acc + base * D + 4 * quad;
+#pragma unroll
+                for (int c = 0; c < ND; ++c) {
+                    const f32x4 other = *reinterpret_cast<const f32x4*>(block + (c * 64 + lane) * 4);
+                    *reinterpret_cast<f32x4*>(pa + 16 * c) = acc[u][c] * w0 + other * w1;
+                }
+                if (quad == 0) {
+                    part_ml[base * 2] = top == NEG_INF ? NEG_INF : top * g.scale;
+                    part_ml[base * 2 + 1] = total;
+                }
+                continue;
+            }
             const float inv = total > 0.f ? 1.f / total : 0.f;
             elem_t* o = out + ((size_t)(row_start[row] + q0 + u * g.tokens_per_tile + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
@@ -995,6 +1021,17 @@ __global__ __launch_bounds__(256 * HALVES, LSA_TILE_MIN_WAVES(SUB)) void paged_a
         total += __shfl_xor(total, 16, 64);
         total += __shfl_xor(total, 32, 64);
         if (!pair_valid[u]) continue;
+        if (slots.first >= 0) {
+            const size_t base = ((size_t)(slots.first + (wave * SUB + u) * slots.stride) * heads + head_index) * 16 + col;
+            float* pa = part_acc + base * D + 4 * quad;
+#pragma unroll
+            for (int c = 0; c < ND; ++c) *reinterpret_cast<f32x4*>(pa + 16 * c) = acc[u][c];
+            if (quad == 0) {
+                part_ml[base * 2] = run_max[u] == NEG_INF ? NEG_INF : run_max[u] * g.scale;
+                part_ml[base * 2 + 1] = total;
+            }
+            continue;
+        }
         const float inv = total > 0.f ? 1.f / total : 0.f;
         elem_t* o = out + ((size_t)(row_start[row] + q0 + u * g.tokens_per_tile + pair_token) * g.n_q + head) * D + 4 * quad;
 #pragma unroll
@@ -1304,7 +1341,8 @@ __global__ __launch_bounds__(MERGE_WAVES * 64) void merge_kernel(
 LSA_EXPORT int lsa_paged_attention(
     const void* q, long q_token_stride, void* out, const void* keys, const void* values, const int* table, int table_stride,
     const int* row_start, const int* row_len, const int* row_ctx, const void* items, const int* item_slot, int n_items,
-    const void* merges, int n_merges, int n_slots, float* part_acc, float* part_ml, const void* tiles, int n_tiles, float scale,
+    const void* merges, int n_merges, int n_slots, float* part_acc, float* part_ml, const void* tiles, const void* tile_slots, int n_tiles,
+    float scale,
     int window, int page_size, int n_q, int n_kv, int gheads, int tokens_per_tile, int gtiles,
     int decode_fusion, const float* q_weight, const float* k_weight, float norm_eps, const float* cos_sin, int tiles_per_workgroup,
     int merge_in_workgroup, int tile_halves, hipStream_t stream) {
@@ -1326,7 +1364,8 @@ LSA_EXPORT int lsa_paged_attention(
         if (tile_halves != 1 && tile_halves != MAX_HALVES) return -1;
 #define LSA_LAUNCH_TILES(SUB, HALVES) paged_attention_tile_kernel<SUB, HALVES><<<tgrid, 256 * HALVES, 0, stream>>>( \
                 (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride, \
-                row_start, row_len, row_ctx, (const Item*)tiles, g)
+                row_start, row_len, row_ctx, (const Item*)tiles, (const TileSlots*)tile_slots, part_acc, part_ml, g)
+        if (tile_slots != nullptr && (part_acc == nullptr || part_ml == nullptr || n_merges <= 0)) return -1;
         if (tiles_per_workgroup == 4 && tile_halves == 1) LSA_LAUNCH_TILES(1, 1);
         else if (tiles_per_workgroup == 4) LSA_LAUNCH_TILES(1, MAX_HALVES);
         else if (tile_halves == 1) LSA_LAUNCH_TILES(MAX_SUB, 1);
@@ -1335,7 +1374,7 @@ LSA_EXPORT int lsa_paged_attention(
         const int terr = (int)hipGetLastError();
         if (terr) return terr;
 #else
-        if (tiles_per_workgroup != 4 || tile_halves != 1) return -1;      // the float32 kernel: four tiles, keys whole
+        if (tiles_per_workgroup != 4 || tile_halves != 1 || tile_slots != nullptr) return -1;      // the float32 kernel: four tiles, keys whole
         paged_attention_tile_kernel_f32<<<dim3(n_tiles * n_kv * gtiles), 256, 0, stream>>>(
             (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride,
             row_start, row_len, row_ctx, (const Item*)tiles, g);
@@ -1343,38 +1382,40 @@ LSA_EXPORT int lsa_paged_attention(
         if (terr) return terr;
 #endif
     }
-    if (n_items <= 0) return 0;
-    // merge_in_workgroup (0, 2 or 4 ranges a tile): items 4 i .. 4 i + 3 are the four key ranges of one tile, or the two
-    // ranges of each of two tiles (some may be empty), no item has a slot, nothing is left to merge.
-    if (merge_in_workgroup && ((merge_in_workgroup != 2 && merge_in_workgroup != 4) || n_items % 4 != 0 || n_merges != 0)) return -1;
-    dim3 grid((n_items + 3) / 4, n_kv * gtiles);
+    int err = 0;
+    if (n_items > 0) {
+        // merge_in_workgroup (0, 2 or 4 ranges a tile): items 4 i .. 4 i + 3 are the four key ranges of one tile, or the two
+        // ranges of each of two tiles (some may be empty), no item has a slot, nothing is left to merge.
+        if (merge_in_workgroup && ((merge_in_workgroup != 2 && merge_in_workgroup != 4) || n_items % 4 != 0 || n_merges != 0)) return -1;
+        dim3 grid((n_items + 3) / 4, n_kv * gtiles);
 #define LSA_LAUNCH_ITEMS(MODE, PLAIN) LSA_LAUNCH_ITEMS_MERGE(MODE, PLAIN, 0)
 #define LSA_LAUNCH_ITEMS_MERGE(MODE, PLAIN, RANGES) paged_attention_kernel<MODE, PLAIN, RANGES><<<grid, 256, 0, stream>>>( \
-        (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride, \
-        row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g, fusion)
+            (const elem_t*)q, q_token_stride, (elem_t*)out, (const elem_t*)keys, (const elem_t*)values, table, table_stride, \
+            row_start, row_len, row_ctx, (const Item*)items, item_slot, n_items, part_acc, part_ml, g, fusion)
 #if LSA_BF16
-    const bool plain = q_weight != nullptr && cos_sin != nullptr;
-    if (merge_in_workgroup && decode_fusion && !plain) return -1;      // the caller asks lsa_attention_merges_in_workgroup first
-    if (merge_in_workgroup == 4 && decode_fusion == 3) LSA_LAUNCH_ITEMS_MERGE(3, true, 4);
-    else if (merge_in_workgroup == 4 && decode_fusion == 1) LSA_LAUNCH_ITEMS_MERGE(1, true, 4);
-    else if (merge_in_workgroup == 4) LSA_LAUNCH_ITEMS_MERGE(0, false, 4);
-    else if (merge_in_workgroup == 2 && decode_fusion == 3) LSA_LAUNCH_ITEMS_MERGE(3, true, 2);
-    else if (merge_in_workgroup == 2 && decode_fusion == 1) LSA_LAUNCH_ITEMS_MERGE(1, true, 2);
-    else if (merge_in_workgroup == 2) LSA_LAUNCH_ITEMS_MERGE(0, false, 2);
-    else if (decode_fusion == 3 && plain) LSA_LAUNCH_ITEMS(3, true);
-    else if (decode_fusion == 3) LSA_LAUNCH_ITEMS(3, false);
-    else if (decode_fusion == 1 && plain) LSA_LAUNCH_ITEMS(1, true);
-    else if (decode_fusion == 1) LSA_LAUNCH_ITEMS(1, false);
-    else
+        const bool plain = q_weight != nullptr && cos_sin != nullptr;
+        if (merge_in_workgroup && decode_fusion && !plain) return -1;      // the caller asks lsa_attention_merges_in_workgroup first
+        if (merge_in_workgroup == 4 && decode_fusion == 3) LSA_LAUNCH_ITEMS_MERGE(3, true, 4);
+        else if (merge_in_workgroup == 4 && decode_fusion == 1) LSA_LAUNCH_ITEMS_MERGE(1, true, 4);
+        else if (merge_in_workgroup == 4) LSA_LAUNCH_ITEMS_MERGE(0, false, 4);
+        else if (merge_in_workgroup == 2 && decode_fusion == 3) LSA_LAUNCH_ITEMS_MERGE(3, true, 2);
+        else if (merge_in_workgroup == 2 && decode_fusion == 1) LSA_LAUNCH_ITEMS_MERGE(1, true, 2);
+        else if (merge_in_workgroup == 2) LSA_LAUNCH_ITEMS_MERGE(0, false, 2);
+        else if (decode_fusion == 3 && plain) LSA_LAUNCH_ITEMS(3, true);
+        else if (decode_fusion == 3) LSA_LAUNCH_ITEMS(3, false);
+        else if (decode_fusion == 1 && plain) LSA_LAUNCH_ITEMS(1, true);
+        else if (decode_fusion == 1) LSA_LAUNCH_ITEMS(1, false);
+        else
 #else
-    if (merge_in_workgroup == 4) LSA_LAUNCH_ITEMS_MERGE(0, false, 4);
-    else if (merge_in_workgroup == 2) LSA_LAUNCH_ITEMS_MERGE(0, false, 2);
-    else
+        if (merge_in_workgroup == 4) LSA_LAUNCH_ITEMS_MERGE(0, false, 4);
+        else if (merge_in_workgroup == 2) LSA_LAUNCH_ITEMS_MERGE(0, false, 2);
+        else
 #endif
-    LSA_LAUNCH_ITEMS(0, false);
+        LSA_LAUNCH_ITEMS(0, false);
 #undef LSA_LAUNCH_ITEMS_MERGE
 #undef LSA_LAUNCH_ITEMS
-    int err = (int)hipGetLastError();
+        err = (int)hipGetLastError();
+    }
     if (err || n_merges <= 0) return err;
     dim3 mgrid(n_merges, n_kv * gtiles, 16);
     // A wavefront for every four slots of an average merge (the slots of a step's merges differ little).
@@ -1404,5 +1445,7 @@ LSA_EXPORT int lsa_attention_tile_halves() {
 }
 // Most key ranges a tile's keys may be split into (the merge takes no more slots per tile).
 LSA_EXPORT int lsa_attention_most_splits() { return MERGE_MOST_SLOTS; }
+// Most key ranges that the tiles of a workgroup of the prompt-portion kernel may share with other workgroups (1: none).
+LSA_EXPORT int lsa_attention_tile_key_ranges() { return LSA_BF16 ? MERGE_MOST_SLOTS : 1; }
 LSA_EXPORT int lsa_attention_head_dim() { return D; }
 LSA_EXPORT int lsa_attention_is_bf16() { return LSA_BF16; }

@@ -22,12 +22,13 @@ _SIGNATURES = {
     "lsa_sample_chunks": [c_int],
     "lsa_sample_static": [_P, _P, _P, _P, c_int, c_int, _P],
     "lsa_sample_static_max_rows": [],
-    "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, c_int,
+    "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, _P, c_int,
                             c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_attention_workgroup_tiles": [],
     "lsa_attention_tile_page_multiple": [],
     "lsa_attention_tile_halves": [],
     "lsa_attention_most_splits": [],
+    "lsa_attention_tile_key_ranges": [],
     "lsa_attention_head_dim": [],
     "lsa_attention_is_bf16": [],
     "lsa_gemm_skinny": [c_int, _P, _P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P, _P],

@@ -44,12 +44,14 @@ def _ptr(tensor):
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
 def _stream():
-    """Handle of torch's current stream on the current device (asked for at every launch: the fast way if torch has it)."""
-    if _raw_stream is not None:
-        return _raw_stream(torch.cuda.current_device())
+    """Handle of torch's current stream on the current device (asked for at every launch, a few hundred times a step:
+    the short way if torch has it; whoever launches a kernel holds a tensor on the GPU, so torch's runtime is up)."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -632,6 +634,11 @@ class HipOps(KernelNamespace):
         """Halves that a workgroup of the prompt-portion kernel can split its tiles' keys between (1: it cannot)."""
         return int(self._attention_library(dtype, head_dim).lsa_attention_tile_halves())
 
+    def attention_tile_key_ranges(self, dtype, head_dim) -> int:
+        """Most ranges that the keys of a workgroup's tiles may be cut into, each range another workgroup's (their
+        partial results are merged afterwards); 1: the kernel does not offer that."""
+        return int(self._attention_library(dtype, head_dim).lsa_attention_tile_key_ranges())
+
     @staticmethod
     def decode_fusion_fits(dtype, head_dim) -> bool:
         """Whether the attention kernel can take the q/k norm, the rotation and the new token's way into the cache
@@ -680,6 +687,12 @@ class HipOps(KernelNamespace):
                                  "plan this step with attention_workgroup_tiles(dtype, head_dim, page_size), which says so")
             if int(plan.get("tiles_per_workgroup", 0)) not in (4, most):
                 raise ValueError(f"the plan gives a workgroup {plan.get('tiles_per_workgroup')} tiles, this kernel takes 4 or {most}")
+        tile_slots = plan.get("tile_slots") if n_tiles else None
+        if tile_slots is not None:
+            _check(tile_slots, "plan tile_slots", torch.int32, (n_tiles, 2))
+            if self.attention_tile_key_ranges(qkv.dtype, head_dim) <= 1 or not n_slots or not n_merges:
+                raise ValueError("the plan shares the keys of a workgroup's tiles between workgroups: that takes a kernel that "
+                                 "offers it (attention_tile_key_ranges), slots for the partial results and their merges")
         gheads, tokens_per_tile, gtiles = group_tiling(n_q // n_kv)
         part_acc = part_ml = None
         if n_slots:
@@ -711,7 +724,7 @@ class HipOps(KernelNamespace):
         _launched(lib.lsa_paged_attention(
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(keys), _ptr(values), _ptr(table), table.shape[1], _ptr(row_start),
             _ptr(row_len), _ptr(row_ctx), _ptr(plan["items"]), _ptr(plan["item_slot"]), n_items, _ptr(plan["merges"]),
-            n_merges, n_slots, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), n_tiles, float(scale), int(window) if window else 0,
+            n_merges, n_slots, _ptr(part_acc), _ptr(part_ml), _ptr(tiles), _ptr(tile_slots), n_tiles, float(scale), int(window) if window else 0,
             page_size, n_q, n_kv, gheads, tokens_per_tile, gtiles, fusion_mode, _ptr(q_weight), _ptr(k_weight), float(norm_eps),
             _ptr(cos_sin), int(plan.get("tiles_per_workgroup", 0)), merge_in_workgroup, int(plan.get("tile_halves", 1)), _stream()),
             "paged_attention")

@@ -54,10 +54,16 @@ class AttentionTuning:
     ``target_waves``: wavefronts wanted in flight; rows with few tokens and long contexts are cut into key ranges
     until there are about that many.  ``tile_costs``: the prompt-portion kernel's workgroups take four tiles or the
     most the kernel offers, and walk their keys whole or in two halves side by side; the costs of each of these
-    ways, keyed by (takes the most tiles, halves)."""
+    ways, keyed by (takes the most tiles, halves).  Where the kernel can give ranges of a workgroup's keys to
+    workgroups of their own, the partial results cost ``merge_us`` and ``slot_ns``, and rows need only
+    ``min_tiles_with_ranges`` tiles to go there (without ranges, a short row behind a long context would be a few
+    workgroups' long walk)."""
     target_waves: int = 1024
     tile_costs: Tuple[Tuple[Tuple[bool, int], TileLaunchCost], ...] = (
         ((False, 1), TileLaunchCost()), ((True, 1), TileLaunchCost()), ((False, 2), TileLaunchCost()), ((True, 2), TileLaunchCost()))
+    merge_us: float = 4.0               # a launch that merges partial results, and ...
+    slot_ns: float = 8.0                # ... writing and reading one tile's partial result of one key range, per KV head
+    min_tiles_with_ranges: int = 2      # rows with this many tiles go to the prompt-portion kernel if it can cut their keys
 
     def tile_cost(self, takes_most: bool, halves: int) -> TileLaunchCost:
         return dict(self.tile_costs).get((bool(takes_most), int(halves)), TileLaunchCost())
@@ -94,11 +100,16 @@ class AttentionPlan:
     ``tiles [n_tiles, 4] int32``: row, first token, first key, one past the last key of
     ``tiles_per_workgroup`` (4 or 8) consecutive tiles that one workgroup handles together, sharing
     the keys it loads (in ``tile_halves`` halves of its wavefronts, each on its share of the keys).
+    ``tile_slots [n_tiles, 2] int32`` or None: where the keys of some workgroups' tiles are cut into ranges, each range
+    an entry of ``tiles`` of its own, the first slot of the entry's partial results and the slots between one of its
+    tiles and the next (tile j writes slot first + j * stride); first = -1: the entry has all keys and writes the
+    output.  ``merges`` holds the merges of such tiles, too.
     """
 
-    def __init__(self, items, item_slot, merges, n_slots, tiles=None, tiles_per_workgroup=0, tile_halves=1):
+    def __init__(self, items, item_slot, merges, n_slots, tiles=None, tiles_per_workgroup=0, tile_halves=1, tile_slots=None):
         self.items, self.item_slot, self.merges, self.n_slots = items, item_slot, merges, n_slots
         self.tiles = tiles if tiles is not None else np.zeros((0, 4), dtype=np.int32)
+        self.tile_slots = tile_slots
         self.tiles_per_workgroup = tiles_per_workgroup
         self.tile_halves = tile_halves       # 2: the workgroups of ``tiles`` walk their keys in two halves side by side
         self.merge_in_workgroup = 0          # 4: items 4 i .. 4 i + 3 are one tile's key ranges, merged by their workgroup;
@@ -117,34 +128,78 @@ def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: i
 MIN_TILES_FOR_WORKGROUPS = 16      # rows with at least this many tiles go to the prompt-portion kernel
 
 
+TILE_WALKS = (512, 256, 128, 64, 32, 16, 8)      # most steps of 32 keys a workgroup may be left with, if its keys are cut
+
+
+def _ranges_of_steps(steps, walk, most_ranges):
+    """Into how many ranges ``steps`` steps of keys are cut when no workgroup is to walk more than ``walk``."""
+    if walk is None or most_ranges <= 1:
+        return np.ones_like(steps)
+    return np.minimum(most_ranges, np.maximum(1, -(-steps // walk)))
+
+
+def _workgroups_of_rows(rows, row_len, row_ctx, tokens_per_tile, window, per_workgroup):
+    """The workgroups that ``rows`` make with ``per_workgroup`` tiles each, all rows at once: arrays of their row, first
+    token, first key, one past the last key, and tiles (the last workgroup of a row may have fewer)."""
+    lens = row_len[rows]
+    first_positions = row_ctx[rows] - lens
+    span = per_workgroup * tokens_per_tile
+    groups_of_row = -(-lens // span)
+    of_row = np.repeat(np.arange(len(rows)), groups_of_row)
+    starts = (np.arange(int(groups_of_row.sum())) - np.repeat(np.cumsum(groups_of_row) - groups_of_row, groups_of_row)) * span
+    k_end = first_positions[of_row] + np.minimum(starts + span, lens[of_row])
+    k_begin = np.zeros_like(starts) if window is None else np.maximum(0, first_positions[of_row] + starts - window + 1)
+    tiles = -(-np.minimum(span, lens[of_row] - starts) // tokens_per_tile)
+    return rows[of_row], starts, k_begin, k_end, tiles
+
+
 def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, heads, window, most: int,
-                              tuning: AttentionTuning = DEFAULT_TUNING, most_halves: int = 1):
-    """``(tiles per workgroup, halves)`` of the prompt-portion kernel that the step's rows finish soonest with: 4 or
-    ``most`` tiles, the keys of a workgroup walked whole or, where the kernel can, in two halves side by side.
+                              tuning: AttentionTuning = DEFAULT_TUNING, most_halves: int = 1, most_ranges: int = 1,
+                              min_tiles: int = MIN_TILES_FOR_WORKGROUPS, workgroups: Optional[dict] = None):
+    """``(tiles per workgroup, halves, walk)`` of the prompt-portion kernel that the step's rows finish soonest with:
+    4 or ``most`` tiles, the keys of a workgroup walked whole or, where the kernel can, in two halves side by side,
+    and, where the kernel can (``most_ranges`` > 1), cut into ranges of at most ``walk`` steps for workgroups of
+    their own (None: never cut).
 
     A workgroup walks its keys in steps of 32.  More tiles per workgroup get more out of every step (setting up and
     draining a workgroup costs about 8 steps more), and two halves halve the trips of the longest workgroup, which
     bounds a launch of few workgroups from below; but steps of larger workgroups take longer, which is what counts
-    when every compute unit is busy.  Each way is priced with the tuning's costs: start, then the longest
-    workgroup's trips and all workgroups' steps, whichever is more (blended, since both slow each other down)."""
-    def estimate(per_workgroup, halves):
-        cost = tuning.tile_cost(per_workgroup > 4, halves)
-        span = per_workgroup * tokens_per_tile
-        total = longest = 0
-        for row in range(len(row_len)):
-            if tiles_per_row[row] < MIN_TILES_FOR_WORKGROUPS:
-                continue
-            n, first_pos = int(row_len[row]), int(row_ctx[row]) - int(row_len[row])
-            starts = np.arange(0, n, span)
-            k_end = first_pos + np.minimum(starts + span, n)
-            k_begin = np.zeros_like(starts) if window is None else np.maximum(0, first_pos + starts - window + 1)
-            steps = -(-(k_end - k_begin) // 32)
-            total += int(steps.sum()) + 8 * len(steps)
-            longest = max(longest, int(steps.max()))
-        path, work = -(-longest // halves) * cost.trip_us, total * heads * cost.step_ns * 1e-3
-        return cost.start_us + (path ** 4 + work ** 4) ** 0.25
-    ways = [(per, halves) for halves in sorted({1, max(1, int(most_halves))}) for per in sorted({min(4, most), most})]
-    return min(ways, key=lambda way: (estimate(*way), way[1], way[0]))
+    when every compute unit is busy.  Ranges shorten the longest walk as far as one likes, for the price of a
+    second launch and the partial results' way through memory.  Each way is priced with the tuning's costs: start,
+    then the longest workgroup's trips and all workgroups' steps, whichever is more (blended, since both slow each
+    other down), then the merge.  Shorter and shorter walks are priced until one costs more than the one before."""
+    rows = np.flatnonzero(np.asarray(tiles_per_row) >= min_tiles)
+    row_len, row_ctx = np.asarray(row_len, dtype=np.int64), np.asarray(row_ctx, dtype=np.int64)
+    best, best_key = None, None
+    for per_workgroup in sorted({min(4, most), most}):
+        of_rows = _workgroups_of_rows(rows, row_len, row_ctx, tokens_per_tile, window, per_workgroup)
+        if workgroups is not None:
+            workgroups[per_workgroup] = of_rows                  # (the caller goes on with those of the way chosen)
+        _, _, k_begin, k_end, tiles_of_group = of_rows
+        steps = -(-(k_end - k_begin) // 32)
+        unsplit = int(steps.max(initial=0))
+        for halves in sorted({1, max(1, int(most_halves))}):
+            cost = tuning.tile_cost(per_workgroup > 4, halves)
+            before = None
+            for walk in (None,) + (tuple(w for w in TILE_WALKS if w < unsplit) if most_ranges > 1 else ()):
+                if walk is None:
+                    total, longest, slots = int(steps.sum()) + 8 * len(steps), unsplit, 0
+                else:
+                    ranges = _ranges_of_steps(steps, walk, most_ranges)
+                    per_range = -(-steps // ranges)
+                    total = int((per_range * ranges).sum()) + 8 * int(ranges.sum())
+                    longest = int(per_range.max(initial=0))
+                    slots = int((ranges * tiles_of_group)[ranges > 1].sum())
+                path, work = -(-longest // halves) * cost.trip_us, total * heads * cost.step_ns * 1e-3
+                merge = tuning.merge_us + slots * heads * tuning.slot_ns * 1e-3 if slots else 0.0
+                estimate = cost.start_us + (path ** 4 + work ** 4) ** 0.25 + merge
+                key = (estimate, walk is not None, halves, per_workgroup)
+                if best_key is None or key < best_key:
+                    best, best_key = (per_workgroup, halves, walk), key
+                if walk is not None and before is not None and estimate > before:
+                    break
+                before = estimate if walk is not None else before
+    return best
 
 
 WORKGROUP_RANGES = 4    # key ranges of a tile that one workgroup (four wavefronts) walks and merges itself
@@ -186,7 +241,8 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, 
 def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, window: Optional[int] = None,
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
                          workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: int = 0,
-                         tuning: AttentionTuning = DEFAULT_TUNING, tile_halves: int = 1, tile_min_workgroups: int = 0) -> AttentionPlan:
+                         tuning: AttentionTuning = DEFAULT_TUNING, tile_halves: int = 1, tile_min_workgroups: int = 0,
+                         tile_key_ranges: int = 1) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
@@ -195,7 +251,9 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     to the kernel in which the tiles of a workgroup share the keys they load; ``tile_halves`` says whether that kernel
     can split a workgroup's keys between two halves of its wavefronts (2) or not (1), ``tile_min_workgroups`` how many
     workgroups a launch of it needs to be worth while (a kernel whose steps are slow is bounded by its longest
-    workgroup unless there are many)."""
+    workgroup unless there are many), ``tile_key_ranges`` into how many ranges it lets the keys of a workgroup's tiles
+    be cut, each for a workgroup of its own (1: it does not; more: rows of few tiles go to it as well, and their
+    partial results are merged like those of split items)."""
     _, tokens_per_tile, group_tiles = group_tiling(group_size)
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
@@ -211,24 +269,48 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
     items, slots, merges, tiles = [], [], [], []
     n_slots = 0
-    per_workgroup, halves = 0, 1
-    if workgroup_tiles and fixed_splits is None:
+    per_workgroup, halves, walk = 0, 1, None
+    workgroups = {}
+    most_ranges = max(1, min(int(tile_key_ranges), MAX_SPLITS))
+    min_tiles = tuning.min_tiles_with_ranges if most_ranges > 1 else MIN_TILES_FOR_WORKGROUPS
+    if workgroup_tiles and fixed_splits is None and int(tiles_per_row.max(initial=0)) >= min_tiles:
         chosen = _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window,
-                                           int(workgroup_tiles), tuning, int(tile_halves))
-        per_workgroup, halves = chosen if isinstance(chosen, tuple) else (chosen, 1)
+                                           int(workgroup_tiles), tuning, int(tile_halves), most_ranges, min_tiles, workgroups=workgroups)
+        per_workgroup, halves, walk = (tuple(chosen) + (None,))[:3] if isinstance(chosen, tuple) else (chosen, 1, None)
         if per_workgroup and tile_min_workgroups:
             groups = sum(-(-int(n) // (per_workgroup * tokens_per_tile)) for n, tiles_of_row in zip(row_len, tiles_per_row)
-                         if tiles_of_row >= MIN_TILES_FOR_WORKGROUPS)
+                         if tiles_of_row >= min_tiles)
             if groups * n_kv_heads * group_tiles < tile_min_workgroups:
                 per_workgroup, halves = 0, 1
+    if per_workgroup:
+        # The rows of many tiles, all at once: a workgroup for every ``per_workgroup`` tiles, or one for each range of
+        # their keys.  Tile j of a workgroup whose keys are cut leaves the partial result of range s in slot
+        # first + j * ranges + s, where ``first`` is the group's first slot.
+        rows_in_tiles = np.flatnonzero(tiles_per_row >= min_tiles)
+        of_row, starts, k_begin, k_end, tiles_of_group = workgroups.get(per_workgroup) or _workgroups_of_rows(
+            rows_in_tiles, row_len, row_ctx, tokens_per_tile, window, per_workgroup)
+        aligned = (k_begin // KEY_ALIGN) * KEY_ALIGN
+        steps = -(-(k_end - aligned) // 32)
+        per = -(-steps // _ranges_of_steps(steps, walk, most_ranges)) * 32
+        ranges = np.maximum(1, -(-(k_end - aligned) // np.maximum(per, 32)))      # (none of them empty)
+        cut = ranges > 1
+        first = np.cumsum(np.where(cut, ranges * tiles_of_group, 0)) - np.where(cut, ranges * tiles_of_group, 0)
+        n_slots = int(np.where(cut, ranges * tiles_of_group, 0).sum())
+        group = np.repeat(np.arange(len(ranges)), ranges)                        # an entry for every range of every group
+        s = np.arange(len(group)) - np.repeat(np.cumsum(ranges) - ranges, ranges)
+        entry_begin = np.maximum(k_begin[group], aligned[group] + s * per[group])
+        entry_end = np.minimum(k_end[group], aligned[group] + (s + 1) * per[group])
+        tiles = np.stack([of_row[group], starts[group], entry_begin, entry_end,
+                          np.where(cut[group], first[group] + s, -1), np.where(cut[group], ranges[group], 0)], axis=1)
+        if n_slots:
+            cut_groups = np.flatnonzero(cut)
+            group = np.repeat(cut_groups, tiles_of_group[cut_groups])            # a merge for every tile of every cut group
+            j = np.arange(len(group)) - np.repeat(np.cumsum(tiles_of_group[cut_groups]) - tiles_of_group[cut_groups], tiles_of_group[cut_groups])
+            merges = np.stack([of_row[group], starts[group] + j * tokens_per_tile, first[group] + j * ranges[group], ranges[group]], axis=1).tolist()
     for row in range(len(row_len)):
         n, ctx = int(row_len[row]), int(row_ctx[row])
         first_pos = ctx - n
-        if per_workgroup and tiles_per_row[row] >= MIN_TILES_FOR_WORKGROUPS:
-            span = per_workgroup * tokens_per_tile
-            for q0 in range(0, n, span):
-                k_begin = 0 if window is None else max(0, first_pos + q0 - window + 1)
-                tiles.append((row, q0, k_begin, first_pos + min(q0 + span, n)))
+        if per_workgroup and tiles_per_row[row] >= min_tiles:
             continue
         for tile in range(int(tiles_per_row[row])):
             q0 = tile * tokens_per_tile
@@ -260,10 +342,11 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
             merges.append((row, q0, first_slot, count))
     items = np.asarray(items, dtype=np.int32).reshape(-1, 4)
     merges = np.asarray(merges, dtype=np.int32).reshape(-1, 4)
-    tiles.sort(key=lambda tile: tile[2] - tile[3])       # most keys first: the long tiles must not start last
-    tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 4)
-    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, tiles, per_workgroup if len(tiles) else 0,
-                         halves if len(tiles) else 1)
+    tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 6)
+    tiles = tiles[np.argsort(tiles[:, 2] - tiles[:, 3], kind="stable")]       # most keys first: the long tiles must not start last
+    tile_slots = np.ascontiguousarray(tiles[:, 4:]) if len(tiles) and int(tiles[:, 4].max()) >= 0 else None
+    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, np.ascontiguousarray(tiles[:, :4]),
+                         per_workgroup if len(tiles) else 0, halves if len(tiles) else 1, tile_slots)
 
 
 class GQAttention(Mixer):
@@ -344,10 +427,13 @@ class GQAttention(Mixer):
         per_workgroup = ctx.ops.attention_workgroup_tiles(ctx.dtype, self.head_dim, ctx.page_size)
         halves = ctx.ops.attention_tile_halves(ctx.dtype, self.head_dim) if per_workgroup else 1
         fewest = ctx.ops.attention_tile_min_workgroups(ctx.dtype) if per_workgroup else 0
+        key_ranges = ctx.ops.attention_tile_key_ranges(ctx.dtype, self.head_dim) if per_workgroup else 1
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
                                     target_waves=tuning.target_waves, fixed_splits=fixed, workgroup_tiles=per_workgroup,
-                                    merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves, tile_min_workgroups=fewest)
+                                    merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves, tile_min_workgroups=fewest,
+                                    tile_key_ranges=key_ranges)
         ctx.set_plan(key, {
+            **({"tile_slots": plan.tile_slots} if plan.tile_slots is not None else {}),
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,
             "n_tiles": len(plan.tiles), "n_items": len(plan.items), "n_merges": len(plan.merges),
             "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup, "tile_halves": int(plan.tile_halves),

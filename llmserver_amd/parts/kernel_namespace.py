@@ -87,6 +87,10 @@ class KernelNamespace:
     def attention_tile_halves(self, dtype, head_dim) -> int:
         return 1
 
+    def attention_tile_key_ranges(self, dtype, head_dim) -> int:
+        """Most ranges the keys of a workgroup's tiles may be cut into for workgroups of their own (1: not offered)."""
+        return 1
+
     def attention_tile_min_workgroups(self, dtype) -> int:
         return 0
 

@@ -6,7 +6,7 @@ import random
 import numpy as np
 import pytest
 
-from llmserver_amd.parts.attention import (KEY_ALIGN, MAX_SPLITS, MIN_TILES_FOR_WORKGROUPS, build_attention_plan, fixed_split_count,
+from llmserver_amd.parts.attention import (DEFAULT_TUNING, KEY_ALIGN, MAX_SPLITS, MIN_TILES_FOR_WORKGROUPS, build_attention_plan, fixed_split_count,
                                            group_tiling)
 
 
@@ -25,7 +25,23 @@ def covered_tokens(plan, row_len, row_ctx, group_size, window):
     return seen
 
 
-@pytest.mark.parametrize("seed", range(12))
+def slots_of_tiles(plan, row_len, group_size):
+    """{(row, first token of a tile): slots its key ranges write}, over the entries of ``tiles`` that have slots."""
+    _, tokens_per_tile, _ = group_tiling(group_size)
+    written = {}
+    if plan.tile_slots is None:
+        return written
+    assert plan.tile_slots.shape == (len(plan.tiles), 2) and plan.tile_slots.dtype == np.int32
+    for (row, q0, _, _), (first, stride) in zip(plan.tiles.tolist(), plan.tile_slots.tolist()):
+        if first < 0:
+            continue
+        tiles_here = -(-min(plan.tiles_per_workgroup * tokens_per_tile, row_len[row] - q0) // tokens_per_tile)
+        for j in range(tiles_here):
+            written.setdefault((row, q0 + j * tokens_per_tile), []).append(first + j * stride)
+    return written
+
+
+@pytest.mark.parametrize("seed", range(40))
 def test_every_token_meets_its_keys_exactly_once(seed):
     rng = random.Random(seed)
     group_size = rng.choice([1, 2, 4, 5, 8, 16, 20])
@@ -35,7 +51,9 @@ def test_every_token_meets_its_keys_exactly_once(seed):
     row_len = [rng.choice([1, 1, 1, 2, 7, 33, 200, 900]) for _ in range(rows)]
     row_ctx = [n + rng.choice([0, 0, 5, 64, 1000, 5000]) for n in row_len]
     most = rng.choice([0, 4, 8])
-    plan = build_attention_plan(row_len, row_ctx, group_size, n_kv, window, workgroup_tiles=most)
+    key_ranges = rng.choice([1, 128, 128, 5])
+    plan = build_attention_plan(row_len, row_ctx, group_size, n_kv, window, workgroup_tiles=most, tile_key_ranges=key_ranges,
+                                tile_halves=rng.choice([1, 2]))
     _, tokens_per_tile, _ = group_tiling(group_size)
     seen = covered_tokens(plan, row_len, row_ctx, group_size, window)
     for row in range(rows):
@@ -53,21 +71,42 @@ def test_every_token_meets_its_keys_exactly_once(seed):
             assert lo <= (0 if window is None else max(0, position - window + 1))
             if window is None:
                 assert lo == 0
-    # slots: one per split item, consecutive within a merge, none left over
+    # slots: one per split item and per tile and key range of a workgroup's tiles, consecutive within a merge, none
+    # written twice, none left over
     slots = plan.item_slot.tolist()
-    used = sorted(s for s in slots if s >= 0)
+    of_tiles = slots_of_tiles(plan, row_len, group_size)
+    used = sorted([s for s in slots if s >= 0] + [s for written in of_tiles.values() for s in written])
     assert used == list(range(plan.n_slots))
     for (row, q0, first_slot, count) in plan.merges.tolist():
+        assert 1 < count <= MAX_SPLITS or (row, q0) not in of_tiles
+        if (row, q0) in of_tiles:
+            assert sorted(of_tiles.pop((row, q0))) == list(range(first_slot, first_slot + count)) and count <= key_ranges
+            continue
         members = [i for i, s in enumerate(slots) if first_slot <= s < first_slot + count]
         assert len(members) == count and count <= MAX_SPLITS
         assert all(plan.items[i][0] == row and plan.items[i][1] == q0 for i in members)
         begins = [int(plan.items[i][2]) for i in members]
         assert all(b % KEY_ALIGN == 0 for b in begins[1:])
+    assert not of_tiles                                                       # every tile with slots has its merge
     assert sum(c for *_, c in plan.merges.tolist()) == plan.n_slots
-    # rows with many tiles go to the workgroup kernel when it is offered, and only those
+    # key ranges of a workgroup's tiles begin at multiples of KEY_ALIGN (but the first) and none is empty
+    if plan.tile_slots is not None:
+        for (_, _, k_begin, k_end), (first, stride) in zip(plan.tiles.tolist(), plan.tile_slots.tolist()):
+            assert k_begin < k_end and (first < 0 or stride > 1)
+        groups = {}
+        for (row, q0, k_begin, k_end), (first, stride) in zip(plan.tiles.tolist(), plan.tile_slots.tolist()):
+            groups.setdefault((row, q0), []).append((k_begin, k_end, first, stride))
+        for ranges in groups.values():
+            ranges.sort()
+            assert all(b[0] % KEY_ALIGN == 0 for b in ranges[1:]) and all(a[1] == b[0] for a, b in zip(ranges, ranges[1:]))
+            assert len(ranges) == 1 or ([r[2] for r in ranges] == list(range(ranges[0][2], ranges[0][2] + len(ranges)))
+                                        and all(r[3] == len(ranges) for r in ranges))
+    # rows with many tiles go to the workgroup kernel when it is offered, and only those; rows of few tiles too if the
+    # kernel can cut their keys into ranges
     tiles_per_row = [-(-n // tokens_per_tile) for n in row_len]
     rows_in_tiles = {int(r) for r in plan.tiles[:, 0]} if len(plan.tiles) else set()
-    expected = {r for r in range(rows) if most and tiles_per_row[r] >= MIN_TILES_FOR_WORKGROUPS}
+    enough = MIN_TILES_FOR_WORKGROUPS if key_ranges == 1 else DEFAULT_TUNING.min_tiles_with_ranges
+    expected = {r for r in range(rows) if most and tiles_per_row[r] >= enough}
     assert rows_in_tiles == expected
     keys_of_tiles = [int(k_end - k_begin) for _, _, k_begin, k_end in plan.tiles.tolist()]
     assert keys_of_tiles == sorted(keys_of_tiles, reverse=True)              # the longest start first
@@ -160,3 +199,35 @@ def test_four_or_eight_tiles_per_workgroup_whole_or_in_halves():
     many = build_attention_plan([2048], [2048], 4, 8, None, workgroup_tiles=4, tile_min_workgroups=512)
     assert (few.tiles_per_workgroup, len(few.tiles)) == (0, 0) and len(few.items) == 128
     assert (many.tiles_per_workgroup, len(many.tiles)) == (4, 128)
+
+
+def test_short_rows_behind_long_contexts_share_their_keys_between_workgroups():
+    """With the costs measured on an MI355X and a kernel that offers key ranges: a portion of 64 tokens behind 4,032 is
+    cut into ranges of at most 16 steps for workgroups of their own (four workgroups a KV head would otherwise walk 128
+    steps each), eight rows of 16 tokens likewise, rows of 8 tokens go to that kernel at all; a whole prompt is not cut;
+    beside a whole prompt only the short row is."""
+    from llmserver_amd.parts import AttentionTuning, TileLaunchCost
+    tuning = AttentionTuning(1024, (((False, 1), TileLaunchCost(3.2, 0.89, 1.55)), ((True, 1), TileLaunchCost(8.7, 0.94, 2.45)),
+                                    ((False, 2), TileLaunchCost(3.3, 1.11, 2.08)), ((True, 2), TileLaunchCost(8.8, 1.44, 2.84))))
+
+    def plan_of(lens, ctxs, key_ranges=128):
+        return build_attention_plan(lens, ctxs, 4, 8, None, workgroup_tiles=8, tuning=tuning, tile_halves=2, tile_key_ranges=key_ranges)
+    plan = plan_of([64], [4096])
+    assert len(plan.items) == 0 and plan.tile_slots is not None and len(plan.merges) == 16 and int(plan.merges[:, 3].min()) >= 4
+    steps = -(-(plan.tiles[:, 3] - plan.tiles[:, 2]) // 32)
+    assert int(steps.max()) * (1 if plan.tile_halves == 2 else 2) <= 32
+    plan = plan_of([16] * 8, [4096] * 8)
+    assert len(plan.items) == 0 and plan.tile_slots is not None and len(plan.merges) == 32
+    plan = plan_of([8] * 32, [512] * 32)
+    assert len(plan.items) == 0 and len(plan.tiles) == 32 and plan.tile_slots is None and plan.n_slots == 0
+    plan = plan_of([2048], [2048])
+    assert plan.tile_slots is None and plan.n_slots == 0 and (plan.tiles_per_workgroup, plan.tile_halves) == (8, 2)
+    plan = plan_of([2048, 64], [2048, 4096])
+    with_slots = plan.tiles[plan.tile_slots[:, 0] >= 0]
+    assert len(with_slots) and (with_slots[:, 0] == 1).all()
+    # a kernel that offers no ranges keeps short rows out (they would be a few workgroups' long walk) and cuts nothing
+    plan = plan_of([64, 40], [4096, 4096], key_ranges=1)
+    assert plan.tile_slots is None and {int(r) for r in plan.tiles[:, 0]} == {0} and {int(r) for r in plan.items[:, 0]} == {1}
+    # decoded tokens never go there
+    plan = plan_of([1] * 8 + [40], [4096] * 9)
+    assert {int(r) for r in plan.items[:, 0]} == set(range(8)) and {int(r) for r in plan.tiles[:, 0]} == {8}

@@ -138,7 +138,7 @@ def test_qk_norm_rope_kv_write(ops, dtype, n_q, n_kv, d, page):
 
 
 def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, needle=True, seed=0, target_waves=None, workgroup_tiles=None,
-                   merge_in_workgroup=False, tile_halves=1):
+                   merge_in_workgroup=False, tile_halves=1, tile_walk=None):
     """Random q/k/v through both implementations.  Pages are handed out in scrambled order from a
     pool that first held other data (as if used before).  With ``needle``, one far key per request
     is made to dominate its first query's softmax."""
@@ -172,24 +172,29 @@ def attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=None, need
         values[pages, :, :, (place % page).to(DEV)] = v.to(dtype)
         table[r, :first] = -1                                                     # pages a window has passed are gone
     # workgroup_tiles: None lets the plan choose between the tile counts the kernel offers, 0 keeps every row out of the
-    # prompt-portion kernel, 4 or 8 fixes the count.
+    # prompt-portion kernel, 4 or 8 fixes the count (and ``tile_halves`` and ``tile_walk``, the most steps of 32 keys a
+    # workgroup is left with, the rest going to workgroups of their own).
     from llmserver_amd.parts import attention as attention_module
     most = ops.attention_workgroup_tiles(dtype, d, page) if workgroup_tiles is None or workgroup_tiles else 0
     chooser = attention_module._workgroup_tiles_that_pay
     most_halves = ops.attention_tile_halves(dtype, d) if most else 1
+    key_ranges = ops.attention_tile_key_ranges(dtype, d) if most else 1
     if workgroup_tiles:
-        assert workgroup_tiles <= most and tile_halves <= most_halves
-        attention_module._workgroup_tiles_that_pay = lambda *args, **kwargs: (workgroup_tiles, tile_halves)
+        assert workgroup_tiles <= most and tile_halves <= most_halves and (tile_walk is None or key_ranges > 1)
+        attention_module._workgroup_tiles_that_pay = lambda *args, **kwargs: (workgroup_tiles, tile_halves, tile_walk)
     try:
         plan = build_attention_plan(lens, ctxs, n_q // n_kv, n_kv, window, workgroup_tiles=0 if merge_in_workgroup else most,
                                     merge_in_workgroup=merge_in_workgroup, tile_halves=most_halves, tuning=ops.attention_tuning,
-                                    **({} if target_waves is None else {"target_waves": target_waves}))
+                                    tile_key_ranges=key_ranges, **({} if target_waves is None else {"target_waves": target_waves}))
     finally:
         attention_module._workgroup_tiles_that_pay = chooser
     staged = {"items": torch.from_numpy(plan.items).to(DEV), "item_slot": torch.from_numpy(plan.item_slot).to(DEV),
               "merges": torch.from_numpy(plan.merges).to(DEV), "tiles": torch.from_numpy(plan.tiles).to(DEV), "n_tiles": len(plan.tiles),
               "n_items": len(plan.items), "n_merges": len(plan.merges), "n_slots": plan.n_slots, "tiles_per_workgroup": plan.tiles_per_workgroup,
-              "tile_halves": plan.tile_halves, "merge_in_workgroup": int(plan.merge_in_workgroup)}
+              "tile_halves": plan.tile_halves, "merge_in_workgroup": int(plan.merge_in_workgroup),
+              "most_splits": int(plan.merges[:, 3].max()) if len(plan.merges) else 0}
+    if plan.tile_slots is not None:
+        staged["tile_slots"] = torch.from_numpy(plan.tile_slots).to(DEV)
     t = lambda a: torch.tensor(a, dtype=torch.int32, device=DEV)
     got = torch.zeros(tokens, n_q * d, device=DEV, dtype=dtype)
     ref = torch.zeros_like(got)
@@ -360,6 +365,36 @@ def test_attention_prompt_portions_in_workgroup_tiles(ops, n_q, n_kv, d, page, w
                 plan, _ = attention_case(ops, torch.bfloat16, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d,
                                          workgroup_tiles=per_workgroup, tile_halves=halves)
                 assert (plan.tiles_per_workgroup, plan.tile_halves) == (per_workgroup, halves) and len(plan.tiles) > 0
+
+
+@pytest.mark.parametrize("n_q, n_kv, d, page", [(32, 8, 128, 16), (4, 2, 16, 16), (8, 2, 32, 8), (6, 2, 48, 24), (5, 1, 80, 40), (20, 1, 64, 16),
+                                                (2, 1, 256, 64), (12, 4, 96, 32), (3, 1, 112, 48)])
+@pytest.mark.parametrize("window", [None, 300])
+def test_attention_key_ranges_of_workgroup_tiles(ops, n_q, n_kv, d, page, window):
+    """Rows of few tokens behind long contexts in the prompt-portion kernel, their keys cut into ranges for workgroups
+    of their own and the partial results merged: with four and with eight tiles to a workgroup, keys whole or in halves,
+    ranges of 2, 5 and 16 steps; beside decoded tokens, whole prompts and rows too short for that kernel; a far key
+    decides the first query of every row, so a range that is lost or counted twice shows."""
+    print(f"attention key ranges of workgroup tiles {n_q}/{n_kv} d{d} page{page} window {window}", flush=True)
+    lens = [70, 1, 9, 333, 2, 37, 130]
+    ctxs = [1500, 400, 777, 333, 65, 1061, 2200]
+    dtype = torch.bfloat16
+    assert ops.attention_tile_key_ranges(dtype, d) == 128 and ops.attention_tile_key_ranges(torch.float32, d) == 1
+    plan, _ = attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d)      # as the plan chooses
+    assert len(plan.tiles) > 0 and len(plan.items) > 0
+    for per_workgroup in (4, 8):
+        for halves in (1, 2):
+            if per_workgroup > ops.attention_workgroup_tiles(dtype, d) or halves > ops.attention_tile_halves(dtype, d):
+                continue
+            for walk in (2, 5, 16):
+                plan, _ = attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q + d,
+                                         workgroup_tiles=per_workgroup, tile_halves=halves, tile_walk=walk)
+                if window is not None and walk == 16:                        # a window of 300 keys is 11 steps at most
+                    assert plan.tile_slots is None
+                    continue
+                assert plan.tile_slots is not None and (plan.tile_slots[:, 0] >= 0).any() and plan.n_slots > 0
+                assert window is not None or int(plan.merges[:, 3].max()) >= min(128, 2200 // (32 * walk))
+                assert (plan.tile_slots[:, 0] < 0).any() or walk < 5         # the whole prompt's first tiles have few keys
 
 
 def test_pages_the_workgroup_kernel_does_not_take_go_to_wavefronts_of_their_own(ops):

@@ -62,15 +62,22 @@ def build_steps(main, others):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_sharp_attention_over_a_long_context(sharp_model, dtype, tmp_path):
+def test_sharp_attention_over_a_long_context(sharp_model, dtype, tmp_path, monkeypatch):
     from llmserver_amd.engine.replay import make_runner, replay
     print(f"sharp attention over {LENGTH} tokens, {dtype}", flush=True)
     folder, main, others, expected = sharp_model
     steps, owner = build_steps(main, others)
     runner = make_runner(folder, dtype, traces.peak_tokens(steps), 16)
     out = str(tmp_path / "out")
+    from llmserver_amd.parts import attention as attention_module
+    plans, build = [], attention_module.build_attention_plan
+    monkeypatch.setattr(attention_module, "build_attention_plan", lambda *args, **kwargs: plans.append(build(*args, **kwargs)) or plans[-1])
     assert replay(runner, traces.to_lines(steps).splitlines(), out, report=io.StringIO()) == len(steps)
     runner.cache.check_invariants()
+    # what the steps went through: wavefronts with split key ranges, workgroups of tiles, and (bfloat16) workgroups
+    # that share the keys of short portions behind the long context
+    assert any(plan.n_slots and len(plan.items) for plan in plans) and any(len(plan.tiles) for plan in plans)
+    assert (dtype == "bfloat16") == any(plan.tile_slots is not None for plan in plans)
     results = traces.collect(steps, out, CONFIG["vocab_size"])
     errors = {}
     for (rid, position), logits in results.items():

@@ -102,6 +102,7 @@ def test_attention_part_and_block(dtype, bias):
             n = end - start
             cache.ensure("r", end)
             ctx, pos, token_row, row_start = context(dtype, [n], [start])
+            ctx.page_size = page                          # as the step function says it: the plan asks the kernels with it
             table = torch.tensor([cache.record("r").tables[0]], dtype=torch.int32).numpy()
             ctx.fill([0] * n, pos, token_row, row_start, [n], [end], [], [table], None, ["r"])
             attention.prepare(ctx)
