@@ -274,9 +274,9 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     most_ranges = max(1, min(int(tile_key_ranges), MAX_SPLITS))
     min_tiles = tuning.min_tiles_with_ranges if most_ranges > 1 else MIN_TILES_FOR_WORKGROUPS
     if workgroup_tiles and fixed_splits is None and int(tiles_per_row.max(initial=0)) >= min_tiles:
-        chosen = _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window,
-                                           int(workgroup_tiles), tuning, int(tile_halves), most_ranges, min_tiles, workgroups=workgroups)
-        per_workgroup, halves, walk = (tuple(chosen) + (None,))[:3] if isinstance(chosen, tuple) else (chosen, 1, None)
+        per_workgroup, halves, walk = _workgroup_tiles_that_pay(
+            row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window, int(workgroup_tiles), tuning,
+            int(tile_halves), most_ranges, min_tiles, workgroups=workgroups)
         if per_workgroup and tile_min_workgroups:
             groups = sum(-(-int(n) // (per_workgroup * tokens_per_tile)) for n, tiles_of_row in zip(row_len, tiles_per_row)
                          if tiles_of_row >= min_tiles)
