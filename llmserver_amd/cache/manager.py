@@ -21,7 +21,6 @@ from __future__ import annotations
 
 import dataclasses
 import hashlib
-import json
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np

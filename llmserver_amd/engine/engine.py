@@ -25,8 +25,6 @@ from collections import OrderedDict
 from datetime import datetime, timedelta
 from typing import Dict, List, Optional
 
-import torch
-
 from ..cache import CacheExhaustedError, CacheManager
 from ..sampling import Sampler, request_uniform
 from .batch import StepEntry

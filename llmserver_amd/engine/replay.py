@@ -18,7 +18,6 @@ import os
 import sys
 from typing import Iterable, TextIO
 
-import numpy as np
 import torch
 
 from ..cache import CacheManager

@@ -22,7 +22,7 @@ from __future__ import annotations
 
 import warnings
 from collections import OrderedDict
-from typing import List, Optional, Sequence
+from typing import Optional, Sequence
 
 import numpy as np
 import torch

@@ -9,7 +9,7 @@ final norm and the head (utils/model.py:147-158).
 from __future__ import annotations
 
 import dataclasses
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, Optional, Sequence
 
 import torch
 

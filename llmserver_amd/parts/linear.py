@@ -8,7 +8,7 @@ utils/layers.py:194-203).
 """
 from __future__ import annotations
 
-from typing import Dict, List, Sequence
+from typing import Dict, Sequence
 
 import torch
 

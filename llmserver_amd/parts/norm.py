@@ -7,8 +7,6 @@ residual stream (utils/fused_ops.py:73).
 """
 from __future__ import annotations
 
-import torch
-
 from .base import VECTOR, Norm, ParamSpec
 
 

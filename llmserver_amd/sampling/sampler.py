@@ -10,7 +10,6 @@ from __future__ import annotations
 import random
 from typing import List, Sequence
 
-import numpy as np
 import torch
 
 
