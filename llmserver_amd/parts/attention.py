@@ -64,6 +64,7 @@ class AttentionTuning:
     merge_us: float = 4.0               # a launch that merges partial results, and ...
     slot_ns: float = 8.0                # ... writing and reading one tile's partial result of one key range, per KV head
     min_tiles_with_ranges: int = 2      # rows with this many tiles go to the prompt-portion kernel if it can cut their keys
+                                        # (and if such rows have MIN_TILES_FOR_WORKGROUPS tiles together)
 
     def tile_cost(self, takes_most: bool, halves: int) -> TileLaunchCost:
         return dict(self.tile_costs).get((bool(takes_most), int(halves)), TileLaunchCost())
@@ -125,7 +126,7 @@ def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: i
     return max(1, min(MAX_SPLITS, target_waves // waves, max_keys // MIN_KEYS_PER_SPLIT))
 
 
-MIN_TILES_FOR_WORKGROUPS = 16      # rows with at least this many tiles go to the prompt-portion kernel
+MIN_TILES_FOR_WORKGROUPS = 16      # rows with at least this many tiles go to the prompt-portion kernel (see AttentionTuning for rows with fewer)
 
 
 TILE_WALKS = (512, 256, 128, 64, 32, 16, 8)      # most steps of 32 keys a workgroup may be left with, if its keys are cut
@@ -273,7 +274,9 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     workgroups = {}
     most_ranges = max(1, min(int(tile_key_ranges), MAX_SPLITS))
     min_tiles = tuning.min_tiles_with_ranges if most_ranges > 1 else MIN_TILES_FOR_WORKGROUPS
-    if workgroup_tiles and fixed_splits is None and int(tiles_per_row.max(initial=0)) >= min_tiles:
+    # (rows of few tiles go there only if together they have as many as one row needs without ranges: a launch of its
+    # own, and a merge, for a handful of tiles costs more than the items they would be beside the step's other rows)
+    if workgroup_tiles and fixed_splits is None and int(tiles_per_row[tiles_per_row >= min_tiles].sum()) >= MIN_TILES_FOR_WORKGROUPS:
         per_workgroup, halves, walk = _workgroup_tiles_that_pay(
             row_len, row_ctx, tiles_per_row, tokens_per_tile, n_kv_heads * group_tiles, window, int(workgroup_tiles), tuning,
             int(tile_halves), most_ranges, min_tiles, workgroups=workgroups)
