@@ -158,6 +158,48 @@ def test_temperature_sampling_is_seeded_per_request():
     assert r.generated_token_ids != together[3]
 
 
+def test_temperature_sampling_matches_the_plain_inverse_cdf():
+    """Workload of tiny configuration B (prompts of 1, 40, 64 and 100 tokens under a budget of 32, 12 tokens each at
+    temperature 0.8, a seed per request) in float32 against the plain implementation: every sampled token is the one
+    that the request's own uniform number picks from softmax(logits / 0.8) of the plain logits over the request's
+    sequence so far.  (The reference samples greedily only, utils/engine.py:295-297; stops and streaming as
+    utils/engine.py:299-314.)  A wrong scale of the softmax, an edge off by one token or a number drawn for the wrong
+    request or step moves most tokens.  The one exception has a name: a number within NEAR_AN_EDGE of the edge between
+    two tokens may fall to either side (32-bit logits and running sums differ from the 64-bit ones in the sixth
+    digit), and then the neighbouring token is demanded."""
+    from llmserver_amd import Engine, load_model
+    from llmserver_amd.sampling import request_uniform
+    print("temperature sampling against the plain inverse CDF", flush=True)
+    NEAR_AN_EDGE = 2e-5
+    case, temperature, new_tokens = "B", 0.8, 12
+    vocab = CASES[case][0]["vocab_size"]
+    config, tensors = plain_model(case)
+    prompts = [random_tokens(vocab, n, 80 + i) for i, n in enumerate((1, 40, 64, 100))]
+    model = load_model(model_folder(case), "cuda", "float32")
+    engine = Engine(model, None, max_new_tokens=new_tokens, max_batch_size=4, max_num_batched_tokens=32,
+                    kv_cache_num_blocks=64, kv_cache_block_size=8, ignore_eos=True, temperature=temperature)
+    requests = [engine.add_request(None, prompt, seed=1000 + i) for i, prompt in enumerate(prompts)]
+    while engine.step():
+        pass
+    assert engine.step_profile["prefill_steps"] >= 7          # the budget cut the prompts into portions beside decodes
+    near, greedy_agrees = 0, 0
+    for i, (prompt, request) in enumerate(zip(prompts, requests)):
+        generated = list(request.generated_token_ids)
+        assert len(generated) == new_tokens
+        for draw, token in enumerate(generated):
+            logits = plain.forward(config, tensors, prompt + generated[:draw])[-1]
+            uniform = request_uniform(1000 + i, draw)
+            expected, margin = plain.inverse_cdf_sample(logits, temperature, uniform)
+            greedy_agrees += token == int(torch.argmax(logits))
+            if margin < NEAR_AN_EDGE:
+                near += 1
+                assert abs(token - expected) <= 1, (i, draw, token, expected, margin)
+            else:
+                assert token == expected, (i, draw, token, expected, margin)
+    assert near <= 1, f"{near} of {4 * new_tokens} numbers fell next to an edge between two tokens"
+    assert greedy_agrees < 2 * new_tokens                     # (the temperature did something: these are not the greedy tokens)
+
+
 def test_engine_refuses_to_run_without_its_kernels(monkeypatch):
     """No CPU path: asking for the kernels where no GPU is visible raises instead of falling back."""
     from llmserver_amd.kernels import KernelLibraryMissing, ops

@@ -299,3 +299,44 @@ def test_where_rope_theta_is_looked_up(keys, theta):
     raw = dict(model_type="qwen3", vocab_size=50, hidden_size=24, intermediate_size=40, num_hidden_layers=1,
                num_attention_heads=3, num_key_value_heads=1, head_dim=16, rms_norm_eps=1e-5, **keys)
     assert config_from_dict(raw).rope_theta == theta
+
+
+def test_inverse_cdf_sample_on_a_distribution_worked_out_by_hand():
+    """The inverse CDF on a distribution worked out by hand: probabilities 0.1, 0.2, 0.3, 0.4 at temperature 1,
+    and at temperature 0.5 their squares over 0.30."""
+    logits = torch.log(torch.tensor([0.1, 0.2, 0.3, 0.4], dtype=torch.float64))
+    assert [plain.inverse_cdf_sample(logits, 1.0, u)[0] for u in (0.0, 0.0999, 0.1001, 0.2999, 0.3001, 0.5999, 0.6001, 0.9999)] == [0, 0, 1, 1, 2, 2, 3, 3]
+    edges = [0.01 / 0.30, 0.05 / 0.30, 0.14 / 0.30]
+    assert [plain.inverse_cdf_sample(logits, 0.5, u)[0] for u in (edges[0] - 1e-9, edges[0] + 1e-9, edges[1] + 1e-9, edges[2] - 1e-9, edges[2] + 1e-9)] == [0, 1, 2, 2, 3]
+    assert abs(plain.inverse_cdf_sample(logits, 1.0, 0.31)[1] - 0.01) < 1e-12
+
+
+def test_rounded_oracle_rounds_at_the_reference_kernels_places():
+    """The mode that says what a bfloat16 run may lose: a rounding that keeps everything is the exact oracle bit for bit;
+    rounding to bfloat16 moves the logits by a few parts in a thousand of their size (8 bits at a dozen places a layer),
+    to float32 by a few parts in ten million; and each place named in the docstrings rounds indeed (its output is
+    representable in the rounded type)."""
+    tensors = {name: plain.rounding_to(torch.bfloat16)(tensor) for name, tensor in tiny_tensors(CONFIG, std=0.2).items()}
+    tokens = [3, 9, 1, 44, 17, 5, 30, 2, 2, 11, 49, 0]
+    exact = plain.forward(CONFIG, tensors, tokens)
+    assert torch.equal(plain.forward(CONFIG, tensors, tokens, r=plain.rounding_to(torch.float64)), exact)
+    size = exact.abs().max(dim=-1).values
+    for dtype, low, high in ((torch.bfloat16, 5e-4, 3e-2), (torch.float32, 1e-9, 2e-6)):
+        lost = ((plain.forward(CONFIG, tensors, tokens, r=plain.rounding_to(dtype)) - exact).abs().max(dim=-1).values / size)
+        assert low < float(lost.median()) and float(lost.max()) < high, (dtype, lost)
+    r = plain.rounding_to(torch.bfloat16)
+    x = r(torch.randn(5, 24, dtype=D64))
+
+    def representable(t):
+        return torch.equal(r(t), t)
+    assert representable(plain.rms_norm(x, tensors["model.norm.weight"], 1e-5, r))
+    assert representable(plain.swiglu_mlp(x, tensors, "model.layers.0.mlp", r))
+    assert representable(plain.attention_block(x, tensors, "model.layers.0.self_attn", CONFIG, torch.arange(5), r=r))
+    assert representable(plain.decoder_layer(x, tensors, 1, CONFIG, torch.arange(5), r=r))
+    q = r(torch.randn(6, 5, 8, dtype=D64))
+    cos, sin = plain.rope_cos_sin(torch.arange(5), 8, 100.0)
+    assert representable(plain.apply_rope(q, cos, sin, r)) and not representable(plain.apply_rope(q, cos, sin))
+    # q/k norms round before and after the weight: not the same numbers as one rounding at the end
+    once, twice = plain.rms_norm(q, 1 + 0.3 * torch.randn(8, dtype=D64), 1e-5, r), None
+    twice = plain.rms_norm(q, 1 + 0.3 * torch.randn(8, dtype=D64), 1e-5, r, rounds_before_weight=True)
+    assert representable(once) and representable(twice)

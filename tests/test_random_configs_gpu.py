@@ -13,24 +13,28 @@ import torch
 
 import plain_qwen3 as plain
 import traces
-from helpers import random_tokens
+from helpers import BF16, check_against_rounded_oracle, random_tokens, relative_error
 from llmserver_amd.config import config_from_dict
 from llmserver_amd.weights import RandomInit, write_random_model
 
 pytestmark = pytest.mark.gpu
 
-SEEDS = (1, 2, 3, 5, 8, 13, 21, 34, 55, 62)
+# The first nine are any seeds; the others are the ones at which wider runs of this same generator (some three hundred
+# seeds) found the largest bfloat16 errors, 3 to 4.3 per cent of the logits, on narrow or deep configurations: one head of
+# 160 over a width of 520 in four layers (7002), 35 heads of 16 over a width of 88 (0), a width of 12 (62), ...
+SEEDS = (1, 2, 3, 5, 8, 13, 21, 34, 55, 0, 62, 71, 72, 158, 1001, 2013, 2032, 2036, 2049, 7002, 7003)
 
 
 def random_config(rng):
     kv_heads = rng.choice((1, 1, 2, 2, 3, 4, 5, 8))
     group = rng.choice((1, 1, 2, 3, 4, 5, 7, 8))
-    return dict(model_type="qwen3", num_hidden_layers=rng.choice((1, 2, 3, 4)),
-                hidden_size=rng.choice((24, 40, 56, 72, 88, 104, 136, 200, 264, 520, 100, 36, 1000, 20, 12)),
-                num_attention_heads=kv_heads * group, num_key_value_heads=kv_heads,
-                head_dim=16 * rng.choice((1, 2, 3, 4, 4, 5, 6, 7, 8, 8, 10, 12, 16)),
-                intermediate_size=rng.choice((24, 40, 100, 136, 200, 344, 520, 36, 1000, 44, 28)),
-                vocab_size=rng.choice((97, 256, 301, 1000, 1537, 5003, 33)),
+    head_dim = 16 * rng.choice((1, 2, 3, 4, 4, 5, 6, 7, 8, 8, 10, 12, 16))
+    hidden = rng.choice((24, 40, 56, 72, 88, 104, 136, 200, 264, 520, 100, 36, 1000, 20, 12))
+    intermediate = rng.choice((24, 40, 100, 136, 200, 344, 520, 36, 1000, 44, 28))
+    vocab = rng.choice((97, 256, 301, 1000, 1537, 5003, 33))
+    return dict(model_type="qwen3", num_hidden_layers=rng.choice((1, 2, 3, 4)), hidden_size=hidden,
+                num_attention_heads=kv_heads * group, num_key_value_heads=kv_heads, head_dim=head_dim,
+                intermediate_size=intermediate, vocab_size=vocab,
                 rope_theta=rng.choice((1e4, 5e4, 1e6, 123.0)), rms_norm_eps=rng.choice((1e-6, 1e-5, 1e-4)),
                 attention_bias=rng.random() < 0.4, tie_word_embeddings=rng.random() < 0.5)
 
@@ -45,7 +49,7 @@ def random_trace(rng, vocab):
             step["step"] = len(steps)
             steps.append(step)
 
-    long = rng.choice((130, 257, 400))
+    long = rng.choice((257, 640, 900, 1300))
     add("w", [long, rng.randrange(1, 70)], traces.whole)
     add("t", [long], lambda r: traces.tail_decoded(r, 32))
     sizes = tuple(rng.choice((2, 3, 5, 7, 16, 17, 31, 33, 64, 100)) for _ in range(12))
@@ -84,10 +88,13 @@ def check_configuration(raw, page_size, rng, seed, tmp_path):
 
     print(f"configuration {seed}: page {page_size} {raw}", flush=True)
     folder = str(tmp_path / "model")
-    write_random_model(config_from_dict(dict(raw)), folder, RandomInit(seed=seed, std=rng.choice((0.02, 0.05)), norm_noise=0.1))
+    write_random_model(config_from_dict(dict(raw)), folder, RandomInit(seed=seed, std=rng.choice((0.02, 0.05, 0.1)), norm_noise=0.1))
     steps, requests = random_trace(rng, raw["vocab_size"])
     config, tensors = plain.read_folder(folder)
     expected = {rid: plain.forward(config, tensors, tokens).numpy() for rid, tokens in requests.items()}
+    # what bfloat16 loses on this model and these tokens: the oracle that rounds where the reference's kernels round
+    rounded = [relative_error(row, exact) for rid, tokens in requests.items()
+               for row, exact in zip(plain.forward(config, tensors, tokens, r=BF16).numpy(), expected[rid])]
     for dtype in ("float32", "bfloat16"):
         runner = make_runner(folder, dtype, traces.peak_tokens(steps), page_size)
         out = str(tmp_path / dtype)
@@ -95,19 +102,13 @@ def check_configuration(raw, page_size, rng, seed, tmp_path):
         runner.cache.check_invariants()
         assert not runner.cache.requests, "every request of the trace was ended"
         results = traces.collect(steps, out, raw["vocab_size"])
-        errors = []
-        for rid, tokens in requests.items():
-            for position in range(len(tokens)):
-                want = expected[rid][position]
-                errors.append(float(np.abs(results[(rid, position)] - want).max()) / max(1.0, float(np.abs(want).max())))
-        errors = np.asarray(errors)
+        errors = np.asarray([relative_error(results[(rid, position)], expected[rid][position])
+                             for rid, tokens in requests.items() for position in range(len(tokens))])
         assert np.isfinite(errors).all()
         print(f"  {dtype}: median {np.median(errors):.2e} worst {errors.max():.2e}", flush=True)
         if dtype == "float32":
-            assert errors.max() <= 1e-5, f"{dtype}: {errors.max()} at {int(errors.argmax())}"
+            assert errors.max() <= 2e-5, f"{dtype}: {errors.max()} at {int(errors.argmax())}"
         else:
-            # Rounding to 8 bits at a few places per layer: a smooth spread whose median is near one per cent of the
-            # largest logit and whose tail stays within a few times that; a fault of the cache or a kernel is not smooth.
-            assert np.median(errors) <= 0.012 and errors.max() <= 0.03, f"{dtype}: median {np.median(errors)} worst {errors.max()}"
+            check_against_rounded_oracle(errors, rounded, f"configuration {seed}")
         del runner
         torch.cuda.empty_cache()
