@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_float, c_int, c_long, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_void_p
 from typing import Dict
 
 from . import build
@@ -22,6 +22,7 @@ _SIGNATURES = {
     "lsa_sample_chunks": [c_int],
     "lsa_sample_static": [_P, _P, _P, _P, c_int, c_int, _P],
     "lsa_sample_static_max_rows": [],
+    "lsa_sample_static_error": [c_int],
     "lsa_paged_attention": [_P, c_long, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P, _P, _P, _P, c_int,
                             c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, c_float, _P, c_int, c_int, c_int, _P],
     "lsa_attention_workgroup_tiles": [],
@@ -40,6 +41,8 @@ _SIGNATURES = {
     "lsa_gemm_split_gated_fits": [c_int, c_int, c_int],
     "lsa_gemm_split_gated": [_P, _P, _P, c_int, c_int, c_int, _P],
 }
+
+_RESULT_TYPES = {"lsa_sample_static_error": c_char_p}      # every other entry point returns an int (0 or an error code)
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 
@@ -61,7 +64,7 @@ def load(name: str) -> ctypes.CDLL:
         if hasattr(library, symbol):
             function = getattr(library, symbol)
             function.argtypes = argtypes
-            function.restype = c_int
+            function.restype = _RESULT_TYPES.get(symbol, c_int)
     _loaded[name] = library
     return library
 

@@ -752,8 +752,9 @@ class HipOps(KernelNamespace):
         most = self._sampling.lsa_sample_static_max_rows()
         if n > most:
             raise ValueError(f"sampling without a workspace takes at most {most} rows, got {n}")
-        _launched(self._sampling.lsa_sample_static(_ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), n, vocab, _stream()),
-                  "sample_static")
+        code = self._sampling.lsa_sample_static(_ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), n, vocab, _stream())
+        if code:
+            raise RuntimeError(f"sample_static failed ({code}): {self._sampling.lsa_sample_static_error(code).decode()}")
 
 
 _default = None

@@ -83,7 +83,7 @@ def rope_cos_sin(positions, head_dim, theta, dtype=torch.float64, angle_dtype=No
     part of the formula, so it is kept; cosine and sine of that angle are then taken in ``dtype``.
     ``angle_dtype=torch.float64`` gives the exact product (for invariants that hold only without that rounding)."""
     angle_dtype = angle_dtype or ANGLE_DTYPE
-    frequencies = (positions.to(angle_dtype).unsqueeze(-1) * inverse_frequencies(head_dim, theta, angle_dtype)).to(dtype)
+    frequencies = (positions.to(angle_dtype).unsqueeze(-1) * inverse_frequencies(head_dim, theta, angle_dtype).to(positions.device)).to(dtype)
     angles = torch.cat([frequencies, frequencies], dim=-1)
     return torch.cos(angles), torch.sin(angles)
 
@@ -118,7 +118,7 @@ def causal_attention(q, k, v, scale, window=None, r=exact):
     k = torch.repeat_interleave(k, repeats=group, dim=0)
     v = torch.repeat_interleave(v, repeats=group, dim=0)
     scores = torch.matmul(q, k.transpose(-1, -2)) * scale
-    place = torch.arange(seq)
+    place = torch.arange(seq, device=q.device)
     hidden = place[None, :] > place[:, None]
     if window is not None:
         hidden = hidden | (place[None, :] <= place[:, None] - window)
@@ -182,7 +182,7 @@ def decoder_layer(h, tensors, index, config, positions, window=None, r=exact):
     return r(h + swiglu_mlp(rms_norm(h, tensors[f"{prefix}.post_attention_layernorm.weight"], eps, r), tensors, f"{prefix}.mlp", r))
 
 
-def forward(config, tensors, token_ids, windows=None, layer_order=None, first_position=0, r=exact):
+def forward(config, tensors, token_ids, windows=None, layer_order=None, first_position=0, r=exact, places=None):
     """Logits ``[seq, vocab]`` at every position of one whole sequence
     (utils/model.py:109-158 without cache; tied head rule
     utils/model_loader.py:56-59).
@@ -190,13 +190,17 @@ def forward(config, tensors, token_ids, windows=None, layer_order=None, first_po
     ``windows`` (per layer) and ``layer_order`` (which layer runs when) serve the tests' toy
     arrangements; ``first_position`` shifts all positions.  With a rounding ``r`` everything up to the last norm
     rounds as the reference's bfloat16 run does; the logits themselves stay wide (an engine hands out 32-bit logits,
-    so the rounding of the head's result is not part of what it may lose)."""
-    ids = torch.as_tensor(token_ids, dtype=torch.long)
-    positions = torch.arange(len(ids)) + first_position
+    so the rounding of the head's result is not part of what it may lose).  ``places``: the positions whose logits are
+    wanted (all of them if None; a vocabulary of 150,000 makes the others expensive).  Runs where the tensors live."""
+    device = tensors["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
+    positions = torch.arange(len(ids), device=device) + first_position
     h = tensors["model.embed_tokens.weight"][ids]
     order = layer_order if layer_order is not None else range(config["num_hidden_layers"])
     for index in order:
         h = decoder_layer(h, tensors, index, config, positions, None if windows is None else windows[index], r)
+    if places is not None:
+        h = h[torch.as_tensor(places, dtype=torch.long, device=device)]
     h = rms_norm(h, tensors["model.norm.weight"], config["rms_norm_eps"], r)
     head = tensors["model.embed_tokens.weight"] if config.get("tie_word_embeddings") or "lm_head.weight" not in tensors \
         else tensors["lm_head.weight"]

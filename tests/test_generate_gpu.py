@@ -268,7 +268,7 @@ def test_requests_arriving_over_time_with_shared_prefixes_and_few_pages(case, se
         limits.append(rng.randint(1, 20))
     expected = [plain.greedy_generate(config, tensors, p, n) for p, n in zip(prompts, limits)]
     longest = max(len(p) + n for p, n in zip(prompts, limits))
-    preemptions = hits = 0
+    preemptions_on_the_tight_pool = hits = 0
     for launch_ahead in (True, False):
         for pages in (400, -(-longest // page) + rng.choice((1, 3, 8))):
             engine = Engine(model, None, max_new_tokens=20, max_batch_size=rng.choice((2, 4, 6)), max_num_batched_tokens=rng.choice((16, 32, 128)),
@@ -287,9 +287,11 @@ def test_requests_arriving_over_time_with_shared_prefixes_and_few_pages(case, se
             assert min(engine.kv_cache.available_pages()) == pages and not engine.kv_cache.requests
             for i in range(len(prompts)):
                 assert list(requests[i].generated_token_ids) == expected[i], (launch_ahead, pages, i)
-            preemptions += engine.step_profile["preemptions"]
+            assert pages < 400 or engine.step_profile["preemptions"] == 0
+            preemptions_on_the_tight_pool += engine.step_profile["preemptions"] if pages < 400 else 0
             hits += engine.step_profile["prefix_hit_tokens"]
     assert hits > 0
+    assert preemptions_on_the_tight_pool > 0, "the tight pool (the longest request and a few pages) preempted nobody"
 
 
 def test_calibrate_measures_only_when_asked_and_writes_a_table(tmp_path):
