@@ -119,7 +119,7 @@ class Engine:
                              "decode_by_rows": {}}       # decoding rows of a step -> [steps, seconds] (utils/engine.py:69, 468-471)
         ops = ops if ops is not None else self._default_ops()
         # what the kernels cannot take is refused here, not at the first step
-        ops.check_cache_geometry(model.cache_specs(), config.kv_cache_block_size)
+        ops.check_cache_geometry(model.cache_specs(), config.kv_cache_block_size, config.kv_cache_num_blocks)
         self.kv_cache = CacheManager(model.cache_specs(), config.kv_cache_block_size, config.kv_cache_num_blocks,
                                      num_state_slots=config.max_batch_size, device=self.device, dtype=self.dtype,
                                      model_identity=str(getattr(model, "name", "model")))

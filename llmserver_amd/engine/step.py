@@ -57,6 +57,8 @@ class ModelRunner:
             from ..kernels import default_ops
             ops = default_ops()
         self.model, self.cache, self.ops = model, cache, ops
+        # (whoever made the cache may have asked already, before allocating it; a runner never reads a cache unasked)
+        ops.check_cache_geometry(model.cache_specs(), cache.page_size, [group.pool.num_pages for group in cache.groups] or None)
         self.device, self.dtype = model.device, model.dtype
         self._staging = [Staging(self.device), Staging(self.device)]
         self._flip = 0

@@ -112,10 +112,18 @@ class HipOps(KernelNamespace):
         return self._tuning
 
     @staticmethod
-    def check_cache_geometry(cache_specs, page_size: int) -> None:
-        """Refuse, before anything is allocated, a cache that the attention kernels cannot read."""
+    def check_cache_geometry(cache_specs, page_size: int, num_pages=None) -> None:
+        """Refuse, before anything is allocated, a cache that the attention kernels cannot read.  ``num_pages`` (one
+        number, or one per group of caches) bounds how long a request's context can get."""
         if page_size % 4:
             raise ValueError(f"the attention kernel reads values four keys at a time: page_size must be a multiple of 4, got {page_size}")
+        if num_pages is not None:
+            # A key's page is found as the high half of key * ceil(2^32 / page_size), which is key // page_size only for
+            # keys below 2^32 / page_size; no request can hold more keys than the pool has room for.
+            most = max(num_pages) if isinstance(num_pages, (list, tuple)) else int(num_pages)
+            if most * page_size >= (1 << 32) // page_size:
+                raise ValueError(f"a pool of {most} pages of {page_size} keys lets a context reach {most * page_size} keys; the attention "
+                                 f"kernels find a key's page exactly only below 2^32 / page_size = {(1 << 32) // page_size} keys")
         for spec in cache_specs.values():
             head_dim = getattr(spec, "head_dim", None)
             if head_dim is not None:

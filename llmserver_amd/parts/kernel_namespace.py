@@ -51,8 +51,9 @@ class KernelNamespace:
         raise NotImplementedError
 
     # -- what a namespace may offer; the answers here mean "not offered" --------------------------------------------
-    def check_cache_geometry(self, cache_specs, page_size: int) -> None:
-        """Raise ``ValueError`` for a cache that the kernels cannot read (asked before anything is allocated)."""
+    def check_cache_geometry(self, cache_specs, page_size: int, num_pages=None) -> None:
+        """Raise ``ValueError`` for a cache that the kernels cannot read (asked before anything is allocated):
+        ``page_size`` keys a page, ``num_pages`` pages (one number, or one per group of caches; None: not said)."""
 
     def row_scale_fits(self, x, weight, row_scale) -> bool:
         """Whether the few-row product of these sizes can apply a norm as a scale of its rows."""

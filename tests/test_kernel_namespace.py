@@ -2,9 +2,10 @@
 ``parts.KernelNamespace``: the shipped HIP namespace and the tests' torch twins both answer the required ones, and a
 namespace that offers nothing beyond them (the base class's neutral answers) still runs a model."""
 import inspect
-import re
 import os
+import re
 
+import pytest
 import torch
 
 from llmserver_amd.parts import KernelNamespace
@@ -71,3 +72,27 @@ def test_a_namespace_that_offers_nothing_runs_a_model():
         second = runner.step([StepEntry("r", [5], [0])])
         outs.append(np.concatenate([first.float().cpu().numpy(), second.float().cpu().numpy()]))
     np.testing.assert_allclose(outs[0], outs[1], atol=2e-5, rtol=1e-5)
+
+
+def test_pools_that_let_a_context_outgrow_the_kernels_page_lookup_are_refused():
+    """The attention kernels find a key's page as the high half of key * ceil(2^32 / page_size), exact only for keys
+    below 2^32 / page_size: a pool whose pages could hold a longer context is refused when the engine or a runner
+    is made, with the numbers; page sizes the kernels cannot read, and head sizes, are refused there too."""
+    from llmserver_amd.kernels.ops import HipOps
+    from llmserver_amd.parts.base import PagedKVSpec
+    specs = {0: PagedKVSpec(2, 64, None)}
+    HipOps.check_cache_geometry(specs, 16, (1 << 24) - 1)                  # 2^28 - 16 keys: the last context that is exact
+    HipOps.check_cache_geometry(specs, 500, [17_179, 10])                  # 8,589,500 < 2^32 / 500 = 8,589,934
+    for page_size, pages in ((16, 1 << 24), (500, 17_180), (16, [8, 1 << 24]), (4, 1 << 28)):
+        with pytest.raises(ValueError, match="2\\^32 / page_size"):
+            HipOps.check_cache_geometry(specs, page_size, pages)
+    # the arithmetic the refusal protects: exact below the limit, wrong at some key beyond it
+    for page_size in (500, 12, 16):
+        magic = -(-(1 << 32) // page_size)
+        limit = (1 << 32) // page_size
+        keys = [0, 1, page_size - 1, page_size, limit - 1, limit - page_size, (limit - 1) // page_size * page_size]
+        assert all((key * magic) >> 32 == key // page_size for key in keys)
+    with pytest.raises(ValueError, match="multiple of 4"):
+        HipOps.check_cache_geometry(specs, 6, 10)
+    with pytest.raises(ValueError):
+        HipOps.check_cache_geometry({0: PagedKVSpec(2, 40, None)}, 16, 10)
