@@ -36,41 +36,32 @@ def log(*args):
     print(*args, file=sys.stderr, flush=True)
 
 
-def layer_weights(c):
-    return c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
-        + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
+def decode_step_bytes(model, batch, context):
+    """What a decoding step of ``batch`` rows at ``context`` tokens has to read: every weight it uses once and the
+    cache of its rows, summed over what the model's parts declare (no formula of an architecture stands here)."""
+    from llmserver_amd.engine.cost import StepRow, step_bytes
+    return step_bytes(model, [StepRow(1, context)] * batch, model.dtype)
 
 
-def weight_bytes(config, elem):
-    """What a decode step reads of the weights: every layer's matrices and the head (the embedding table only by row)."""
-    return elem * (config.num_hidden_layers * layer_weights(config) + config.vocab_size * config.hidden_size)
-
-
-def kv_bytes_per_token(config, elem):
-    return 2 * config.num_key_value_heads * config.head_dim * elem * config.num_hidden_layers
-
-
-def prefill_flops(config, tokens):
-    c = config
-    gemm = 2.0 * tokens * layer_weights(c) * c.num_hidden_layers + 2.0 * c.vocab_size * c.hidden_size
-    attention = 2.0 * c.num_attention_heads * c.head_dim * tokens * (tokens + 1) * c.num_hidden_layers
-    return gemm + attention
+def prefill_flops(model, tokens):
+    """Floating-point operations of the step that takes a prompt of ``tokens`` tokens to its first token."""
+    from llmserver_amd.engine.cost import StepRow, step_flops
+    return step_flops(model, [StepRow(tokens, tokens, wanted=1)])
 
 
 def random_model(name, layers, dtype, seed=0):
-    from llmserver_amd.cli.benchmark import RANDOM_CONFIGS
-    from llmserver_amd.config import config_from_dict
+    from llmserver_amd.config import config_from_dict, named_size
     from llmserver_amd.kernels import default_ops
     from llmserver_amd.weights import RandomInit, random_model_on_device
-    raw = dict(RANDOM_CONFIGS[name], model_type="qwen3")
+    raw = named_size(name)
     full = raw["num_hidden_layers"]
     raw["num_hidden_layers"] = min(full, layers) if layers else full
     config = config_from_dict(raw)
     default_ops().preload([config.head_dim], dtype)
-    elem = 2 if str(dtype).endswith("bfloat16") else 4
-    log(f"[bench] {name}: drawing random weights, {weight_bytes(config, elem) / 1e9:.2f} GB")
+    log(f"[bench] {name}: drawing random weights")
     model = random_model_on_device(config, "cuda:0", dtype, RandomInit(seed=seed, std=0.02))
     model.name = f"{name}-random"
+    log(f"[bench] {name}: a decoding step of one row reads {decode_step_bytes(model, 1, 0) / 1e9:.2f} GB of weights")
     return model, config, full
 
 
@@ -178,11 +169,12 @@ def turn_through_engine(model, page_size, cached, fresh, repeats=3, seed=2):
     return best
 
 
-def decode_point(model, config, elem, page_size, batch, context, steps, warmup):
+def decode_point(model, page_size, batch, context, steps, warmup):
+    """Tokens a second, milliseconds a step and GB/s of the bytes a step has to read (at the steps' mean context)."""
     seconds, _ = decode_through_engine(model, page_size, batch, context, steps, warmup)
     ms = 1000.0 * seconds / steps
-    step_bytes = weight_bytes(config, elem) + batch * (context - steps / 2.0) * kv_bytes_per_token(config, elem)
-    return batch * steps / seconds, ms, step_bytes / (ms * 1e-3) / 1e9
+    first, last = decode_step_bytes(model, batch, context - steps + 1), decode_step_bytes(model, batch, context)
+    return batch * steps / seconds, ms, (first + last) / 2.0 / (ms * 1e-3) / 1e9
 
 
 def main() -> int:
@@ -212,11 +204,10 @@ def main() -> int:
 
     dtype = parse_dtype(args.dtype)
     short = "bf16" if dtype == torch.bfloat16 else "fp32"
-    elem = 2 if dtype == torch.bfloat16 else 4
     model, config, full_layers = random_model(MODEL, args.layers, dtype)
 
     log(f"[bench] decode batch {args.batch}: {args.batch} prompts of {args.context - args.steps - args.warmup} tokens, then {args.warmup} + {args.steps} steps")
-    value, ms_per_step, achieved = decode_point(model, config, elem, args.page_size, args.batch, args.context, args.steps, args.warmup)
+    value, ms_per_step, achieved = decode_point(model, args.page_size, args.batch, args.context, args.steps, args.warmup)
     result = {
         "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen3-8B-sized, random weights)", "value": round(value, 2),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
@@ -233,7 +224,7 @@ def main() -> int:
     if not args.no_prefill:
         log(f"[bench] prefill of {args.prefill_tokens} tokens")
         seconds = prefill_through_engine(model, args.page_size, args.prefill_tokens)
-        flops = prefill_flops(config, args.prefill_tokens)
+        flops = prefill_flops(model, args.prefill_tokens)
         result["prefill"] = {"value": round(args.prefill_tokens / seconds, 1), "tokens": args.prefill_tokens,
                              "ms": round(1000.0 * seconds, 3),
                              "frac": round(flops / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)}
@@ -241,7 +232,7 @@ def main() -> int:
     if not args.no_points:
         for batch, steps in ((1, min(args.steps, 64)), (64, min(args.steps, 32))):
             log(f"[bench] decode batch {batch}")
-            rate, ms, gbs = decode_point(model, config, elem, args.page_size, batch, args.context, steps, min(args.warmup, 4))
+            rate, ms, gbs = decode_point(model, args.page_size, batch, args.context, steps, min(args.warmup, 4))
             points[f"decode_b{batch}"] = round(rate, 2)
             points[f"decode_b{batch}_ms_per_step"] = round(ms, 4)
             points[f"decode_b{batch}_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
@@ -250,25 +241,25 @@ def main() -> int:
             log(f"[bench] prefill of {tokens} tokens")
             seconds = prefill_through_engine(model, args.page_size, tokens)
             points[f"prefill_{tokens}_ms"] = round(1000.0 * seconds, 3)
-            points[f"prefill_{tokens}_mfma_frac"] = round(prefill_flops(config, tokens) / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)
+            points[f"prefill_{tokens}_mfma_frac"] = round(prefill_flops(model, tokens) / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)
         log("[bench] 128 new tokens behind 8,064 cached ones")
         points["turn_128_after_8064_ms"] = round(1000.0 * turn_through_engine(model, args.page_size, 8064, 128), 3)
         log("[bench] decode batch 4 at a context of 16,384")
-        rate, ms, gbs = decode_point(model, config, elem, args.page_size, 4, 16384, 32, 4)
+        rate, ms, gbs = decode_point(model, args.page_size, 4, 16384, 32, 4)
         points["decode_b4_ctx16384"] = round(rate, 2)
         points["decode_b4_ctx16384_ms_per_step"] = round(ms, 4)
         points["decode_b4_ctx16384_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
     del model
     torch.cuda.empty_cache()
     if not args.no_points and not args.no_extra_points and dtype == torch.bfloat16 and not args.layers:
-        points.update(extra_points(dtype, elem, args.page_size))
+        points.update(extra_points(dtype, args.page_size))
     if points:
         result["points"] = points
     print(json.dumps(result), flush=True)
     return 0
 
 
-def extra_points(dtype, elem, page_size):
+def extra_points(dtype, page_size):
     """The two other workloads the baseline names, each on a random model of its own size."""
     import torch
 
@@ -294,7 +285,7 @@ def extra_points(dtype, elem, page_size):
     # Batch 16 behind prompts of 8,192 tokens (Qwen3-32B sizes): the decoding steps up to a context of 8,192 + 64.
     model, config, _ = random_model("qwen3-32b", 0, dtype)
     batch, context, steps, warmup = 16, 8192 + 64, 48, 4
-    rate, ms, gbs = decode_point(model, config, elem, page_size, batch, context, steps, warmup)
+    rate, ms, gbs = decode_point(model, page_size, batch, context, steps, warmup)
     points["decode_32b_b16_ctx8192"] = round(rate, 2)
     points["decode_32b_b16_ctx8192_ms_per_step"] = round(ms, 4)
     points["decode_32b_b16_ctx8192_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)

@@ -10,42 +10,33 @@ With ``--prompt`` (text, if the model folder has a ``tokenizer.json``) or ``--pr
 in the manner of the reference's ``benchmark.py`` (benchmark.py:68-88, 339-341): model load, time to
 the first token, generation and decode throughput, medians over ``--repeats``.
 
-For each (prompt length, batch size):
-  * ttft_s  = time to generate 1 token for the whole batch (prefill latency)
-  * total_s = time to generate ``--output-tokens`` tokens for the whole batch
-  * decode tok/s = batch * (output_tokens - 1) / (total_s - ttft_s)
-EOS is ignored, decoding is greedy unless ``--temperature`` is given, and every (prompt length,
-batch size, repeat) gets its own seeded random token ids, so prefix caching cannot help
-(benchmark_cuda.py:13, 32-38).  ``--random-config`` draws seeded random weights
-on the device instead of reading a folder.
+The matrix times two things per (prompt length, batch size), each the median of ``--repeats`` runs on fresh prompts
+(the definitions are the reference's, benchmark_cuda.py:8-13): ``ttft_s``, a run that generates one
+token per request, i.e. the prompts' way to their first tokens; and ``total_s``, a run that generates ``--output-tokens``.
+What lies between them is decoding: ``decode_tok_s = batch * (output_tokens - 1) / (total_s - ttft_s)``.  EOS is
+ignored, decoding is greedy unless ``--temperature`` is given, and every run's prompts are seeded random token ids of
+their own, so that cached prefix pages cannot help.  ``--random-config`` draws seeded random weights on the device
+instead of reading a folder.
 """
 from __future__ import annotations
 
 import argparse
+import dataclasses
 import json
-import math
 import statistics
 import sys
 import time
+from typing import List, Optional
 
-RANDOM_CONFIGS = {
-    "tiny-a": dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
-                   intermediate_size=128, vocab_size=256, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True),
-    "tiny-b": dict(num_hidden_layers=3, hidden_size=96, num_attention_heads=8, num_key_value_heads=2, head_dim=32,
-                   intermediate_size=224, vocab_size=384, rope_theta=1e6, rms_norm_eps=1e-5, attention_bias=True),
-    "qwen3-1.7b": dict(num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
-                       intermediate_size=6144, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=True),
-    "qwen3-8b": dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
-                     intermediate_size=12288, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
-    "qwen3-14b": dict(num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, head_dim=128,
-                      intermediate_size=17408, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
-    "qwen3-32b": dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
-                      intermediate_size=25600, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
-}
+from ..config.named_sizes import NAMED_SIZES
 
 
-def parse_ints(text):
-    return [int(item) for item in text.split(",") if item.strip()]
+def int_list(text: str) -> List[int]:
+    """An option's value ``"128, 1024"`` as ``[128, 1024]`` (an ``argparse`` type: a bad item is the option's error)."""
+    try:
+        return [int(item) for item in text.replace(" ", "").split(",") if item]
+    except ValueError:
+        raise argparse.ArgumentTypeError(f"expected integers separated by commas, got {text!r}") from None
 
 
 def build_prompts(vocab, prompt_tokens, count, tag, seed):
@@ -157,9 +148,38 @@ def profile_engine(engine, vocab, prompt_lengths, batches, seed, out_path) -> No
     print(f"kernel tables written to {out_path}", flush=True)
 
 
+@dataclasses.dataclass
+class PromptRun:
+    """One request from its arrival to its last token."""
+    tokens: List[int]
+    seconds: float
+    first_token_seconds: float
+
+    @property
+    def decode_rate(self) -> Optional[float]:
+        """Tokens a second after the first one; None for a run of one token."""
+        rest = len(self.tokens) - 1
+        return rest / max(self.seconds - self.first_token_seconds, 1e-9) if rest > 0 else None
+
+
+def time_one_prompt(engine, prompt_ids, new_tokens) -> PromptRun:
+    import torch
+    torch.cuda.synchronize()
+    arrived = time.perf_counter()
+    request = engine.add_request(None, prompt_token_ids=prompt_ids, max_new_tokens=new_tokens)
+    first = None
+    while engine.step():
+        if first is None and request.generated_token_ids:
+            first = time.perf_counter()
+    torch.cuda.synchronize()
+    finished = time.perf_counter()
+    return PromptRun(list(request.generated_token_ids), finished - arrived, (first or finished) - arrived)
+
+
 def one_prompt(args, model, load_seconds) -> int:
-    """One prompt, ``--repeats`` fresh requests: the reference's single-prompt statistics
-    (benchmark.py:68-88)."""
+    """One prompt, ``--repeats`` fresh requests, and what the reference's single-prompt benchmark reports of them
+    (benchmark.py:68-88): load time, time to the first token, the whole generation, throughput overall
+    and of decoding alone, medians when there are several runs."""
     import os
 
     import torch
@@ -175,56 +195,146 @@ def one_prompt(args, model, load_seconds) -> int:
         tokenizer = Tokenizer.from_file(path)
         prompt_ids = tokenizer.encode(args.prompt).ids
     else:
-        prompt_ids = parse_ints(args.prompt_token_ids)
+        prompt_ids = args.prompt_token_ids
     if not prompt_ids or args.max_new_tokens <= 0:
         print("the prompt must hold at least one token and --max-new-tokens must be positive", file=sys.stderr)
         return 2
-    blocks = math.ceil((len(prompt_ids) + args.max_new_tokens) / args.block_size) + 8
     engine = Engine(model, None, max_new_tokens=args.max_new_tokens, max_batch_size=1,
                     max_num_batched_tokens=max(args.max_num_batched_tokens, 1), prefill_chunk_size=args.prefill_chunk_size,
-                    kv_cache_num_blocks=blocks, kv_cache_block_size=args.block_size, stream_text=False, max_completed_requests=0,
+                    kv_cache_num_blocks=pool_pages(model, args.block_size, 1, len(prompt_ids) + args.max_new_tokens),
+                    kv_cache_block_size=args.block_size, stream_text=False, max_completed_requests=0,
                     ignore_eos=False, temperature=args.temperature, seed=args.seed, enable_prefix_caching=False)
     run_once(engine, [prompt_ids], min(args.max_new_tokens, 4))               # graphs are captured before the clock starts
-    results = []
-    for _ in range(args.repeats):
-        torch.cuda.synchronize()
-        start = time.perf_counter()
-        request = engine.add_request(None, prompt_token_ids=prompt_ids, max_new_tokens=args.max_new_tokens)
-        first = None
-        while engine.step():
-            if first is None and request.generated_token_ids:
-                first = time.perf_counter() - start
-        torch.cuda.synchronize()
-        seconds = time.perf_counter() - start
-        results.append((list(request.generated_token_ids), seconds, first if first is not None else seconds))
-    tokens, seconds, first = results[-1]
-    print(f"\nPrompt: {args.prompt if args.prompt is not None else prompt_ids}")
-    print(f"Response: {tokenizer.decode(tokens) if tokenizer is not None else tokens}")
-    print(f"\nDevice: {torch.cuda.get_device_name(0)} | Model: {model.name}")
-    print(f"Prompt tokens: {len(prompt_ids)} | Generated tokens: {len(tokens)}")
-    print(f"Model load: {load_seconds:.2f} s | Generation: {seconds:.3f} s")
-    print(f"Time to first token: {first:.4f} s")
-    print(f"Generation throughput: {len(tokens) / seconds:.2f} tokens/s")
-    if len(tokens) > 1:
-        print(f"Decode throughput: {(len(tokens) - 1) / (seconds - first):.2f} tokens/s")
-    if len(results) > 1:
-        print(f"median over {len(results)} runs: Generation: {statistics.median(r[1] for r in results):.3f} s | "
-              f"Time to first token: {statistics.median(r[2] for r in results):.4f} s")
-        speeds = [(len(r[0]) - 1) / (r[1] - r[2]) for r in results if len(r[0]) > 1]
-        if speeds:
-            print(f"median decode throughput: {statistics.median(speeds):.2f} tokens/s")
+    runs = [time_one_prompt(engine, prompt_ids, args.max_new_tokens) for _ in range(args.repeats)]
+    last = runs[-1]
+    shown = {"prompt": args.prompt if args.prompt is not None else prompt_ids,
+             "response": tokenizer.decode(last.tokens) if tokenizer is not None else last.tokens,
+             "model": f"{model.name} ({args.dtype}) on {torch.cuda.get_device_name(0)}",
+             "tokens": f"{len(prompt_ids)} in the prompt, {len(last.tokens)} generated",
+             "load": f"{load_seconds:.2f} s",
+             "first token": f"{last.first_token_seconds * 1000:.2f} ms after the request arrived",
+             "whole run": f"{last.seconds:.3f} s, {len(last.tokens) / last.seconds:.2f} tokens/s"}
+    if last.decode_rate is not None:
+        shown["decoding"] = f"{last.decode_rate:.2f} tokens/s after the first token"
+    if len(runs) > 1:
+        medians = [f"first token {statistics.median(run.first_token_seconds for run in runs) * 1000:.2f} ms",
+                   f"whole run {statistics.median(run.seconds for run in runs):.3f} s"]
+        rates = [run.decode_rate for run in runs if run.decode_rate is not None]
+        if rates:
+            medians.append(f"decoding {statistics.median(rates):.2f} tokens/s")
+        shown[f"medians of {len(runs)} runs"] = ", ".join(medians)
+    print()
+    for label, value in shown.items():
+        print(f"{label:>18}: {value}")
     return 0
+
+
+def pool_pages(model, block_size: int, batch: int, tokens_per_request: int, memory_share: float = 0.85) -> int:
+    """Pages for ``batch`` requests that each grow to ``tokens_per_request`` tokens: their own pages, and the spare page
+    per running request that the scheduler keeps free before it admits another; never more than ``memory_share`` of the
+    device memory that is free now (activations and graphs need the rest)."""
+    import torch
+
+    from ..cache import CacheManager
+    per_request = -(-tokens_per_request // block_size) + 1
+    page_bytes = max(1, CacheManager.bytes_per_token(model.cache_specs(), model.dtype) * block_size)
+    fitting = int(memory_share * torch.cuda.mem_get_info()[0]) // page_bytes
+    return max(1, min(batch * per_request, fitting))
+
+
+@dataclasses.dataclass
+class Measurement:
+    """One cell of the matrix: runs to the first token and runs to ``output_tokens`` tokens, on fresh prompts each."""
+    prompt_tokens: int
+    batch: int
+    output_tokens: int
+    first_token_runs: List[float] = dataclasses.field(default_factory=list)     # seconds of runs that generate one token per request
+    whole_runs: List[float] = dataclasses.field(default_factory=list)           # seconds of runs that generate output_tokens
+    tokens: Optional[List[List[int]]] = None                                    # what the first whole run generated
+    peak_memory_bytes: int = 0
+    failure: Optional[str] = None
+
+    @property
+    def ttft_s(self) -> float:
+        return statistics.median(self.first_token_runs)
+
+    @property
+    def total_s(self) -> float:
+        return statistics.median(self.whole_runs)
+
+    @property
+    def decode_s(self) -> float:
+        """What a whole run takes beyond the first tokens."""
+        return max(self.total_s - self.ttft_s, 1e-9)
+
+    @property
+    def decode_tok_s(self) -> float:
+        return self.batch * (self.output_tokens - 1) / self.decode_s
+
+    @property
+    def prefill_tok_s(self) -> float:
+        return self.batch * self.prompt_tokens / self.ttft_s
+
+    @property
+    def end_to_end_tok_s(self) -> float:
+        return self.batch * self.output_tokens / self.total_s
+
+    def record(self) -> dict:
+        """The cell as it goes into the ``--json`` report."""
+        cell = {"prompt_tokens": self.prompt_tokens, "batch": self.batch, "output_tokens": self.output_tokens}
+        if self.failure is not None:
+            return dict(cell, error=self.failure)
+        return dict(cell, ttft_s=self.ttft_s, total_s=self.total_s, decode_tok_s=self.decode_tok_s, prefill_tok_s=self.prefill_tok_s,
+                    end_to_end_tok_s=self.end_to_end_tok_s, decode_ms_per_token=1000 * self.decode_s / max(self.output_tokens - 1, 1),
+                    tokens=self.tokens, peak_memory_gib=round(self.peak_memory_bytes / 2 ** 30, 2))
+
+    def line(self) -> str:
+        where = f"{self.batch:3d} x {self.prompt_tokens:6d} tokens"
+        if self.failure is not None:
+            return f"{where}: {self.failure}"
+        return (f"{where}: first tokens after {self.ttft_s * 1000:9.2f} ms ({self.prefill_tok_s:10.1f} tok/s), "
+                f"decoding {self.decode_tok_s:10.1f} tok/s, end to end {self.end_to_end_tok_s:10.1f} tok/s")
+
+
+def matrix_prompts(vocab, prompt_tokens, batch, phase, repeat, seed):
+    """The prompts of one run of one cell; ``phase``: "warm-up", "first-token" or "whole-run"."""
+    return build_prompts(vocab, prompt_tokens, batch, f"{phase}/{prompt_tokens}x{batch}/{repeat}", seed)
+
+
+def measure(engine, vocab, prompt_tokens, batch, output_tokens, repeats, seed, pool_tokens) -> Measurement:
+    """Fill one cell.  A cell that cannot run (the pool is too small for it, memory runs out) says so in ``failure``
+    and the matrix goes on."""
+    import torch
+    cell = Measurement(prompt_tokens, batch, output_tokens)
+    needed = batch * (prompt_tokens + output_tokens)
+    if needed > pool_tokens:
+        cell.failure = f"needs {needed} tokens of cache, the pool holds {pool_tokens}"
+        return cell
+    try:
+        # A whole run first, untimed: every graph that the timed runs replay is captured then
+        # (the reference warms up the same way, benchmark_cuda.py:208).
+        run_once(engine, matrix_prompts(vocab, prompt_tokens, batch, "warm-up", 0, seed), output_tokens)
+        for repeat in range(repeats):
+            cell.first_token_runs.append(run_once(engine, matrix_prompts(vocab, prompt_tokens, batch, "first-token", repeat, seed), 1)[0])
+        for repeat in range(repeats):
+            seconds, generated = run_once(engine, matrix_prompts(vocab, prompt_tokens, batch, "whole-run", repeat, seed), output_tokens)
+            cell.whole_runs.append(seconds)
+            cell.tokens = cell.tokens or generated
+        cell.peak_memory_bytes = torch.cuda.max_memory_allocated()
+    except (RuntimeError, MemoryError, BufferError) as error:
+        cell.failure = f"{type(error).__name__}: {error}"
+    return cell
 
 
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     parser.add_argument("--model", default=None, help="model folder (config.json + safetensors)")
-    parser.add_argument("--random-config", default=None, choices=sorted(RANDOM_CONFIGS), help="seeded random weights of a named size instead of --model")
+    parser.add_argument("--random-config", default=None, choices=sorted(NAMED_SIZES), help="seeded random weights of a named size instead of --model")
     parser.add_argument("--prompt", default=None, help="one prompt as text (needs tokenizer.json in the model folder)")
-    parser.add_argument("--prompt-token-ids", default=None, help="one prompt as comma-separated token ids")
+    parser.add_argument("--prompt-token-ids", default=None, type=int_list, help="one prompt as comma-separated token ids")
     parser.add_argument("--max-new-tokens", type=int, default=32, help="tokens to generate for --prompt / --prompt-token-ids")
-    parser.add_argument("--prompt-tokens", default="128,1024")
-    parser.add_argument("--batch-sizes", default="1,8,32")
+    parser.add_argument("--prompt-tokens", default=[128, 1024], type=int_list)
+    parser.add_argument("--batch-sizes", default=[1, 8, 32], type=int_list)
     parser.add_argument("--output-tokens", type=int, default=128)
     parser.add_argument("--repeats", type=int, default=3)
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
@@ -238,7 +348,7 @@ def main(argv=None) -> int:
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--mixed-requests", type=int, default=0,
                         help="instead of the matrix: this many concurrent requests under continuous batching with chunked prefill")
-    parser.add_argument("--mixed-prompt-range", default="16,2048", help="prompt lengths of the mixed workload, uniform in [lo, hi]")
+    parser.add_argument("--mixed-prompt-range", default=[16, 2048], type=int_list, help="prompt lengths of the mixed workload, uniform in [lo, hi]")
     parser.add_argument("--shared-prefix-tokens", type=int, default=512, help="length of the prefix that some mixed requests share")
     parser.add_argument("--shared-fraction", type=float, default=0.5, help="fraction of mixed requests that start with the shared prefix")
     parser.add_argument("--max-batch-size", type=int, default=None, help="requests running at a time (default: the largest batch)")
@@ -253,38 +363,35 @@ def main(argv=None) -> int:
         parser.error("--custom-dtype fp16: this engine computes in bfloat16 (source) or float32 (fp32) only")
     if args.custom_dtype is not None:
         args.dtype = {"source": "bfloat16", "fp32": "float32"}[args.custom_dtype]
+    if len(args.mixed_prompt_range) != 2:
+        parser.error("--mixed-prompt-range takes two numbers: lo,hi")
 
     import torch
 
-    from ..config import config_from_dict
+    from ..config import named_config
     from ..engine import Engine, load_model
     from ..engine.loading import parse_dtype
-    from ..cache import CacheManager
     from ..weights import RandomInit, random_model_on_device
 
     started = time.perf_counter()
     if args.model:
         model = load_model(args.model, args.device, args.dtype)
     else:
-        config = config_from_dict(dict(RANDOM_CONFIGS[args.random_config], model_type="qwen3"))
-        model = random_model_on_device(config, args.device, parse_dtype(args.dtype), RandomInit(seed=args.seed, std=0.02))
+        model = random_model_on_device(named_config(args.random_config), args.device, parse_dtype(args.dtype), RandomInit(seed=args.seed, std=0.02))
         model.name = args.random_config
     torch.cuda.synchronize()
     print(f"loaded {model.name} in {time.perf_counter() - started:.1f} s", flush=True)
     vocab = model.config.vocab_size
     if args.prompt is not None or args.prompt_token_ids is not None:
         return one_prompt(args, model, time.perf_counter() - started)
-    prompt_lengths, batches = parse_ints(args.prompt_tokens), parse_ints(args.batch_sizes)
+    prompt_lengths, batches = args.prompt_tokens, args.batch_sizes
     if args.mixed_requests:
-        low, high = parse_ints(args.mixed_prompt_range)
+        low, high = args.mixed_prompt_range
         prompt_lengths, batches = [high], [args.max_batch_size or args.mixed_requests]
-    max_batch, max_length = max(batches), max(prompt_lengths) + args.output_tokens
-    bytes_per_block = CacheManager.bytes_per_token(model.cache_specs(), model.dtype) * args.block_size
-    wanted = max_batch * math.ceil(max_length / args.block_size) + 8          # benchmark_cuda.py:107-111
-    wanted = min(wanted, int(torch.cuda.mem_get_info()[0] * 0.8 // max(1, bytes_per_block)))
-    engine = Engine(model, None, max_new_tokens=1, max_batch_size=max_batch,
-                    max_num_batched_tokens=max(args.max_num_batched_tokens, max_batch), prefill_chunk_size=args.prefill_chunk_size,
-                    kv_cache_num_blocks=wanted, kv_cache_block_size=args.block_size, stream_text=False, max_completed_requests=0,
+    pages = pool_pages(model, args.block_size, max(batches), max(prompt_lengths) + args.output_tokens)
+    engine = Engine(model, None, max_new_tokens=1, max_batch_size=max(batches),
+                    max_num_batched_tokens=max(args.max_num_batched_tokens, max(batches)), prefill_chunk_size=args.prefill_chunk_size,
+                    kv_cache_num_blocks=pages, kv_cache_block_size=args.block_size, stream_text=False, max_completed_requests=0,
                     ignore_eos=True, temperature=args.temperature, seed=args.seed, enable_prefix_caching=True)
     results = []
     if args.mixed_requests:
@@ -300,38 +407,14 @@ def main(argv=None) -> int:
         prompt_lengths = []
     for prompt_length in prompt_lengths:
         for batch in batches:
-            entry = {"prompt_tokens": prompt_length, "batch": batch, "output_tokens": args.output_tokens}
-            try:
-                if batch * (prompt_length + args.output_tokens) > wanted * args.block_size:
-                    raise MemoryError("KV cache too small for this configuration")
-                # One whole run first, as the reference warms up (benchmark_cuda.py:208 there): every graph the timed
-                # runs replay is captured before the clock starts.
-                run_once(engine, build_prompts(vocab, prompt_length, batch, f"warm-{prompt_length}-{batch}", args.seed), args.output_tokens)
-                ttft, total, tokens = [], [], None
-                for repeat in range(args.repeats):
-                    seconds, _ = run_once(engine, build_prompts(vocab, prompt_length, batch, f"t1-{prompt_length}-{batch}-{repeat}", args.seed), 1)
-                    ttft.append(seconds)
-                for repeat in range(args.repeats):
-                    seconds, generated = run_once(engine, build_prompts(vocab, prompt_length, batch, f"tn-{prompt_length}-{batch}-{repeat}", args.seed), args.output_tokens)
-                    total.append(seconds)
-                    tokens = tokens or generated
-                ttft_s, total_s = statistics.median(ttft), statistics.median(total)
-                decode_s = max(total_s - ttft_s, 1e-9)
-                entry.update(ttft_s=ttft_s, total_s=total_s, decode_tok_s=batch * (args.output_tokens - 1) / decode_s,
-                             e2e_tok_s=batch * args.output_tokens / total_s, prefill_tok_s=batch * prompt_length / ttft_s,
-                             ms_per_token=1000 * decode_s / max(args.output_tokens - 1, 1), tokens=tokens,
-                             peak_alloc_gb=round(torch.cuda.max_memory_allocated() / 2 ** 30, 2))
-                print(f"prompt {prompt_length:6d}  batch {batch:3d}:  ttft {ttft_s * 1000:9.2f} ms   decode {entry['decode_tok_s']:10.1f} tok/s   "
-                      f"prefill {entry['prefill_tok_s']:10.1f} tok/s   end-to-end {entry['e2e_tok_s']:10.1f} tok/s", flush=True)
-            except Exception as error:            # record per-configuration failures (e.g. out of memory) and go on
-                entry["error"] = f"{type(error).__name__}: {error}"
-                print(f"prompt {prompt_length:6d}  batch {batch:3d}:  {entry['error']}", flush=True)
-            results.append(entry)
+            cell = measure(engine, vocab, prompt_length, batch, args.output_tokens, args.repeats, args.seed, pages * args.block_size)
+            print(cell.line(), flush=True)
+            results.append(cell.record())
     if args.profile:
         print("step profile:", json.dumps(engine.step_profile), flush=True)
         engine.max_new_tokens = 64
         profile_engine(engine, vocab, prompt_lengths or [high], batches, args.seed, args.profile_out)
-    report = {"model": model.name, "dtype": args.dtype, "block_size": args.block_size, "kv_blocks": wanted, "gpu": torch.cuda.get_device_name(0),
+    report = {"model": model.name, "dtype": args.dtype, "block_size": args.block_size, "kv_blocks": pages, "gpu": torch.cuda.get_device_name(0),
               "torch": torch.__version__, "results": results, "step_profile": engine.step_profile}
     if args.json:
         with open(args.json, "w") as handle:

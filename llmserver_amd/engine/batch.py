@@ -79,7 +79,6 @@ class StepContext:
         self._computed: Dict[object, object] = {}
         self._tables: Dict[int, torch.Tensor] = {}
         self.static_max_keys: Optional[int] = None      # set when the step's array shapes must be fixed (graph capture)
-        self.short_contexts = False                     # a captured step of single tokens none of whose contexts is long
         self.page_size = None                           # keys a page of the cache holds, if the maker of the step says
 
     # -- building ------------------------------------------------------------------------

@@ -120,6 +120,7 @@ class Engine:
         ops = ops if ops is not None else self._default_ops()
         # what the kernels cannot take is refused here, not at the first step
         ops.check_cache_geometry(model.cache_specs(), config.kv_cache_block_size, config.kv_cache_num_blocks)
+        self._warn_of_slow_page_size(ops, model, config.kv_cache_block_size)
         self.kv_cache = CacheManager(model.cache_specs(), config.kv_cache_block_size, config.kv_cache_num_blocks,
                                      num_state_slots=config.max_batch_size, device=self.device, dtype=self.dtype,
                                      model_identity=str(getattr(model, "name", "model")))
@@ -326,6 +327,18 @@ class Engine:
         self._withdraw_offers()         # offered but not admitted: nothing is held over a step
         return plan
 
+    def _warn_of_slow_page_size(self, ops, model, page_size: int) -> None:
+        """Say so once if these pages keep prompt portions out of the kernel that shares a workgroup's keys between its
+        tiles (the step's plan then gives every tile a wavefront of its own, which reads its keys itself: correct,
+        and about half as fast on long prompts)."""
+        import warnings
+        for head_dim in sorted({spec.head_dim for spec in model.cache_specs().values() if hasattr(spec, "head_dim")}):
+            if ops.attention_workgroup_tiles(self.dtype, head_dim) and not ops.attention_workgroup_tiles(self.dtype, head_dim, page_size):
+                warnings.warn(f"kv_cache_block_size={page_size}: the attention kernel for prompt portions takes pages of a multiple of 8 keys "
+                              f"in {str(self.dtype).split('.')[-1]}; with this page size prompts run through the slower per-tile kernel "
+                              "(a multiple of 16, such as 496 or 512, keeps them on the fast one)", stacklevel=3)
+                return
+
     # -- one step ------------------------------------------------------------------------------
     def warmup_graphs(self, batch_sizes=None, max_context=None) -> int:
         """Capture the decode graphs of these numbers of rows (default: every size that decoding steps of up to
@@ -334,15 +347,16 @@ class Engine:
         reference).  The graphs serve contexts up to the first width of the block table, or, with ``max_context``,
         every width up to that context (the pool has to hold that many tokens for every row meanwhile; sizes it
         cannot hold are left to be captured when they are met)."""
-        from .step import SHORT_CONTEXT, TABLE_WIDTH_STEP
+        from .step import TABLE_WIDTH_STEP
         if not self.runner.use_graphs or self.active_requests:
             return 0
         most = self.scheduler.max_batch_size
         if batch_sizes is None:
             batch_sizes = sorted({min(most, padded_rows(rows)) for rows in range(1, most + 1)})
         tokens_per_width = TABLE_WIDTH_STEP * self.block_size
-        # one token (the shape of short contexts), the first context that is not short, then every width of the table
-        contexts = [1, SHORT_CONTEXT + 1] + [width * tokens_per_width + 1 for width in range(1, -(-(max_context or 1) // tokens_per_width))]
+        # one token, the first context beyond each edge at which a mixer's captured work changes its shape, then every width of the table
+        edges = sorted({edge + 1 for block in self.runner.model.blocks for edge in block.mixer.graph_shape_edges()})
+        contexts = [1] + edges + [width * tokens_per_width + 1 for width in range(1, -(-(max_context or 1) // tokens_per_width))]
         try:
             for context in contexts:
                 pages_per_row = -(-context // self.block_size)

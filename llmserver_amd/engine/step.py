@@ -31,8 +31,6 @@ from ..cache.manager import CacheManager
 from .batch import Staging, StepContext, StepEntry
 
 TABLE_WIDTH_STEP = 64      # captured steps serve block tables up to the next multiple of this many pages
-SHORT_CONTEXT = 512        # captured steps whose contexts all stay within this are a shape of their own (``ctx.short_contexts``):
-                           # mixers may then do with less machinery (attention merges its key ranges inside its workgroups)
 MAX_GRAPHS = 96
 
 
@@ -63,7 +61,8 @@ class ModelRunner:
         self._staging = [Staging(self.device), Staging(self.device)]
         self._flip = 0
         self.vocab = model.head.out_features
-        graph_safe = all(block.mixer.graph_safe for block in model.blocks) and not cache.state_specs
+        self._mixers = list({id(block.mixer): block.mixer for block in model.blocks}.values())
+        graph_safe = all(mixer.graph_safe for mixer in self._mixers) and not cache.state_specs
         if use_graphs is None:
             use_graphs = self.device.type == "cuda" and ops.name == "hip"
         self.use_graphs = bool(use_graphs and graph_safe)
@@ -160,7 +159,9 @@ class ModelRunner:
         rows, wanted = len(entries), sum(len(entry.want) for entry in entries)
         if all(len(entry.want) == 1 for entry in entries):
             rows = wanted = padded_rows(rows)          # decoding: filled up to one of a few sizes
-        return (rows, width, wanted, longest <= SHORT_CONTEXT)
+        # what the mixers' captured work depends on beyond that (each asks itself the same when it prepares the step)
+        shapes = tuple(dict.fromkeys(mixer.graph_shape(rows, longest) for mixer in self._mixers))
+        return (rows, width, wanted, shapes)
 
     @torch.inference_mode()
     def prepare_ahead(self, request_ids: Sequence[object]) -> bool:
@@ -187,7 +188,6 @@ class ModelRunner:
         except BufferError:          # no page for one of them: the step itself will say so, or the caller makes room
             return False
         ctx.static_max_keys = key[1] * self.cache.page_size
-        ctx.short_contexts = key[3]
         self.model.prepare(ctx)
         ctx.stage()
         if ctx.layout != captured.layout:
@@ -265,7 +265,6 @@ class ModelRunner:
         ctx = self.build_context(entries, staging=staging, table_width=key[1], filler_rows=key[0] - len(entries))
         wanted = sum(len(entry.want) for entry in entries)           # the fillers' logits come last and are dropped
         ctx.static_max_keys = key[1] * self.cache.page_size
-        ctx.short_contexts = key[3]
         self.model.prepare(ctx)
         if captured is None:
             ctx.static_max_keys = None           # the first upload may size the staging buffer

@@ -2,7 +2,7 @@
 
     python -m llmserver_amd.kernels.calibrate --model DIR [--model DIR ...] [--out FILE] [--max-batch-size 64]
     python -m llmserver_amd.kernels.calibrate --config config.json [...]      (random weights of those sizes, two layers)
-    python -m llmserver_amd.kernels.calibrate --random-config qwen3-8b [...]  (a size the benchmark command knows by name)
+    python -m llmserver_amd.kernels.calibrate --random-config qwen3-8b [...]  (a size known by name, see llmserver_amd/config/named_sizes.py)
 
 Every product shape of the models is timed both ways (a hand-written kernel with what it folds in; the library's
 product and the kernels it would have absorbed; the library's product whole or in ranges of its inner dimension) at 1
@@ -22,7 +22,7 @@ def main(argv=None) -> int:
     parser = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     parser.add_argument("--model", action="append", default=[], help="a model folder (config.json + safetensors)")
     parser.add_argument("--config", action="append", default=[], help="a config.json whose sizes are measured with random weights")
-    parser.add_argument("--random-config", action="append", default=[], help="a named size of the benchmark command")
+    parser.add_argument("--random-config", action="append", default=[], help="a named size (llmserver_amd/config/named_sizes.py)")
     parser.add_argument("--layers", type=int, default=2, help="layers of a --config model (shapes do not depend on the number)")
     parser.add_argument("--out", default=SHIPPED)
     parser.add_argument("--max-batch-size", type=int, default=64)
@@ -33,8 +33,7 @@ def main(argv=None) -> int:
     import torch
 
     from .. import models  # noqa: F401
-    from ..cli.benchmark import RANDOM_CONFIGS
-    from ..config import config_from_dict
+    from ..config import config_from_dict, named_size
     from ..engine import Engine, load_model, parse_dtype
     from ..weights import random_model_on_device
     total = 0
@@ -44,7 +43,7 @@ def main(argv=None) -> int:
             model = load_model(source, "cuda", args.dtype)
         else:
             if kind == "named":
-                raw = dict(RANDOM_CONFIGS[source], model_type="qwen3")
+                raw = named_size(source)
             else:
                 with open(source) as handle:
                     raw = json.load(handle)

@@ -9,6 +9,8 @@ switched off, on the 32-bit path.
 """
 from __future__ import annotations
 
+import dataclasses
+
 import torch
 
 from ..parts.attention import AttentionTuning, TileLaunchCost, group_tiling
@@ -96,6 +98,7 @@ class HipOps(KernelNamespace):
         self._flush = None
         self._replay_overhead = None
         self._tuning = None
+        self._tuning_f32 = None
 
     @property
     def attention_tuning(self) -> AttentionTuning:
@@ -110,6 +113,15 @@ class HipOps(KernelNamespace):
                      ((False, 2), TileLaunchCost(3.3, 1.11, 2.08)), ((True, 2), TileLaunchCost(8.8, 1.44, 2.84)))
             self._tuning = AttentionTuning(target_waves=4 * units, tile_costs=costs)
         return self._tuning
+
+    def attention_tuning_for(self, dtype) -> AttentionTuning:
+        """The float32 kernels step through 16 keys at a time (16x16x4 products), the bfloat16 ones through 32."""
+        tuning = self.attention_tuning
+        if dtype == torch.float32:
+            if self._tuning_f32 is None:
+                self._tuning_f32 = dataclasses.replace(tuning, key_step=16)
+            return self._tuning_f32
+        return tuning
 
     @staticmethod
     def check_cache_geometry(cache_specs, page_size: int, num_pages=None) -> None:
@@ -492,13 +504,17 @@ class HipOps(KernelNamespace):
                   "gemm_skinny_stream")
         return stream, weighted, square_sums
 
-    def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None):
+    ACTIVATIONS = ("silu",)       # what the activation kernel and the gated products' epilogues compute
+
+    def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None, activation="silu"):
         """``silu(x @ gate^T) * (x @ up^T)`` with ``gate_up_weight [2I, K]`` in one launch for few rows (the
-        activation sits in the product's epilogue), or None if this is not such a case.  ``pairs_per_workgroup``:
+        activation sits in the product's epilogue), or None if this is not such a case (another activation is none).  ``pairs_per_workgroup``:
         1 to 16 pairs of a gate and an up row in two tiles, -1 for 8 pairs in one tile, 0 lets the size decide.
         ``row_scale`` as in :meth:`linear_few_rows`."""
         rows, width = x.shape
         inter = gate_up_weight.shape[0] // 2
+        if activation not in self.ACTIVATIONS:
+            return None
         if rows > self.skinny_rows:
             return self._linear_gated_beyond_few_rows(x, gate_up_weight) if row_scale is None and pairs_per_workgroup == 0 else None
         if not self._few_rows(x, gate_up_weight) or inter % 8 or gate_up_weight.shape[1] != width or rows > 16 \
@@ -566,7 +582,9 @@ class HipOps(KernelNamespace):
         _launched(self._elementwise.lsa_add_rmsnorm(_code(resid), _ptr(resid), _ptr(delta), _ptr(weight), float(eps),
                                                     _ptr(out), _ptr(rows), n_out, width, _stream()), "add_rmsnorm")
 
-    def swiglu(self, gate_up, out):
+    def swiglu(self, gate_up, out, activation="silu"):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"the activation kernel computes {', '.join(self.ACTIVATIONS)}; {activation!r} is not built")
         n, inter = out.shape
         _check(gate_up, "gate_up", out.dtype, (n, 2 * inter))
         _check(out, "out")

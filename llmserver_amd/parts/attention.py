@@ -29,17 +29,20 @@ from .base import VECTOR, Mixer, PagedKVSpec, ParamSpec, PositionEncoding
 from .kernel_namespace import tuning_of
 from .linear import Linear
 
-TILE_ROWS = 16          # rows of (token, group head) pairs one wavefront handles (MFMA N dimension)
+# Neutral defaults of the plan's geometry (AttentionTuning carries them; a kernel namespace may say otherwise per type):
+TILE_ROWS = 16          # rows of (token, group head) pairs that one work item handles
 KEY_ALIGN = 32          # key ranges of split items start at multiples of this
-MAX_SPLITS = 128        # key ranges per tile (the merge kernel's limit, which the kernel namespace checks)
-MIN_KEYS_PER_SPLIT = 64     # shorter key ranges than this are not worth a wavefront of their own
+KEY_STEP = 32           # keys that a workgroup of the prompt-portion kernel takes per trip through its loop
+MAX_SPLITS = 128        # key ranges per tile (what the kernel that merges them takes, which the kernel namespace checks)
+MIN_KEYS_PER_SPLIT = 64     # shorter key ranges than this are not worth a work item of their own
+TILE_WALKS = (512, 256, 128, 64, 32, 16, 8)      # most steps a workgroup may be left with, if its keys are cut
 
 
 @dataclasses.dataclass(frozen=True)
 class TileLaunchCost:
     """What one way of launching the prompt-portion kernel costs: microseconds of start and end, microseconds of one
-    trip of a workgroup through its loop (32 keys; a workgroup makes its trips one after the other, so its longest
-    workgroup bounds a launch), and nanoseconds of one 32-key step of one workgroup per KV head when every compute
+    trip of a workgroup through its loop (``key_step`` keys; a workgroup makes its trips one after the other, so its
+    longest workgroup bounds a launch), and nanoseconds of one such step of one workgroup per KV head when every compute
     unit is busy (the work of all workgroups together bounds a launch, too)."""
     start_us: float = 4.0
     trip_us: float = 1.0
@@ -57,7 +60,12 @@ class AttentionTuning:
     ways, keyed by (takes the most tiles, halves).  Where the kernel can give ranges of a workgroup's keys to
     workgroups of their own, the partial results cost ``merge_us`` and ``slot_ns``, and rows need only
     ``min_tiles_with_ranges`` tiles to go there (without ranges, a short row behind a long context would be a few
-    workgroups' long walk)."""
+    workgroups' long walk).
+
+    The geometry of the kernels' work items stands here, too, so that the plan is cut for the kernels that will run it:
+    ``tile_rows`` (token, head) pairs to an item, key ranges that begin at multiples of ``key_align`` keys, at most
+    ``most_splits`` of them to a tile and none shorter than ``fewest_keys_per_split`` (but the last), ``key_step`` keys
+    per trip of the prompt-portion kernel, and the walks (in steps) that its workgroups' keys may be cut down to."""
     target_waves: int = 1024
     tile_costs: Tuple[Tuple[Tuple[bool, int], TileLaunchCost], ...] = (
         ((False, 1), TileLaunchCost()), ((True, 1), TileLaunchCost()), ((False, 2), TileLaunchCost()), ((True, 2), TileLaunchCost()))
@@ -65,6 +73,12 @@ class AttentionTuning:
     slot_ns: float = 8.0                # ... writing and reading one tile's partial result of one key range, per KV head
     min_tiles_with_ranges: int = 2      # rows with this many tiles go to the prompt-portion kernel if it can cut their keys
                                         # (and if such rows have MIN_TILES_FOR_WORKGROUPS tiles together)
+    tile_rows: int = TILE_ROWS
+    key_align: int = KEY_ALIGN
+    key_step: int = KEY_STEP
+    most_splits: int = MAX_SPLITS
+    fewest_keys_per_split: int = MIN_KEYS_PER_SPLIT
+    tile_walks: Tuple[int, ...] = TILE_WALKS
 
     def tile_cost(self, takes_most: bool, halves: int) -> TileLaunchCost:
         return dict(self.tile_costs).get((bool(takes_most), int(halves)), TileLaunchCost())
@@ -85,10 +99,10 @@ class AttentionNames:
     k_norm: str = "k_norm"
 
 
-def group_tiling(group_size: int):
+def group_tiling(group_size: int, tile_rows: int = TILE_ROWS):
     """(heads of a group per tile, tokens per tile, tiles needed to cover the group)."""
-    heads = min(group_size, TILE_ROWS)
-    return heads, TILE_ROWS // heads, -(-group_size // heads)
+    heads = min(group_size, tile_rows)
+    return heads, tile_rows // heads, -(-group_size // heads)
 
 
 class AttentionPlan:
@@ -117,19 +131,18 @@ class AttentionPlan:
                                              # 2: they are the two ranges of each of two tiles
 
 
-def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: int, target_waves: int = TARGET_WAVES) -> int:
+def fixed_split_count(n_rows: int, group_size: int, n_kv_heads: int, max_keys: int, target_waves: int = TARGET_WAVES,
+                      tuning: AttentionTuning = DEFAULT_TUNING) -> int:
     """Splits per row when the plan's shape must not depend on the rows' contexts (a captured
-    graph of a decode step): enough to fill the chip, never pieces shorter than MIN_KEYS_PER_SPLIT
+    graph of a decode step): enough to fill the chip, never pieces shorter than ``fewest_keys_per_split``
     at the longest context the graph serves."""
-    _, _, group_tiles = group_tiling(group_size)
+    _, _, group_tiles = group_tiling(group_size, tuning.tile_rows)
     waves = max(1, n_rows * n_kv_heads * group_tiles)
-    return max(1, min(MAX_SPLITS, target_waves // waves, max_keys // MIN_KEYS_PER_SPLIT))
+    return max(1, min(tuning.most_splits, target_waves // waves, max_keys // tuning.fewest_keys_per_split))
 
 
 MIN_TILES_FOR_WORKGROUPS = 16      # rows with at least this many tiles go to the prompt-portion kernel (see AttentionTuning for rows with fewer)
 
-
-TILE_WALKS = (512, 256, 128, 64, 32, 16, 8)      # most steps of 32 keys a workgroup may be left with, if its keys are cut
 
 
 def _ranges_of_steps(steps, walk, most_ranges):
@@ -162,7 +175,7 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
     and, where the kernel can (``most_ranges`` > 1), cut into ranges of at most ``walk`` steps for workgroups of
     their own (None: never cut).
 
-    A workgroup walks its keys in steps of 32.  More tiles per workgroup get more out of every step (setting up and
+    A workgroup walks its keys in steps of ``tuning.key_step``.  More tiles per workgroup get more out of every step (setting up and
     draining a workgroup costs about 8 steps more), and two halves halve the trips of the longest workgroup, which
     bounds a launch of few workgroups from below; but steps of larger workgroups take longer, which is what counts
     when every compute unit is busy.  Ranges shorten the longest walk as far as one likes, for the price of a
@@ -177,12 +190,12 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
         if workgroups is not None:
             workgroups[per_workgroup] = of_rows                  # (the caller goes on with those of the way chosen)
         _, _, k_begin, k_end, tiles_of_group = of_rows
-        steps = -(-(k_end - k_begin) // 32)
+        steps = -(-(k_end - k_begin) // tuning.key_step)
         unsplit = int(steps.max(initial=0))
         for halves in sorted({1, max(1, int(most_halves))}):
             cost = tuning.tile_cost(per_workgroup > 4, halves)
             before = None
-            for walk in (None,) + (tuple(w for w in TILE_WALKS if w < unsplit) if most_ranges > 1 else ()):
+            for walk in (None,) + (tuple(w for w in tuning.tile_walks if w < unsplit) if most_ranges > 1 else ()):
                 if walk is None:
                     total, longest, slots = int(steps.sum()) + 8 * len(steps), unsplit, 0
                 else:
@@ -204,9 +217,12 @@ def _workgroup_tiles_that_pay(row_len, row_ctx, tiles_per_row, tokens_per_tile, 
 
 
 WORKGROUP_RANGES = 4    # key ranges of a tile that one workgroup (four wavefronts) walks and merges itself
+SHORT_CONTEXT = 512     # captured steps whose contexts all stay within this are a shape of their own: a workgroup merges
+                        # a tile's four key ranges itself (no partial results in memory, no launch that merges them)
 
 
-def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, merge_in_workgroup: int = 0) -> AttentionPlan:
+def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, merge_in_workgroup: int = 0,
+                       key_align: int = KEY_ALIGN) -> AttentionPlan:
     """The plan of a step in which every row brings one token and every tile gets ``splits`` key ranges: what the
     loop of :func:`build_attention_plan` makes for it, row by row, computed for all rows at once (a decode step of
     many rows is planned thousands of times a second)."""
@@ -220,9 +236,9 @@ def _single_token_plan(row_ctx: np.ndarray, window: Optional[int], splits: int, 
         return AttentionPlan(items, np.full(n_rows, -1, dtype=np.int32), np.zeros((0, 4), dtype=np.int32), 0)
     if merge_in_workgroup:          # four (or two) items a tile; with fewer ranges wanted, the last ones come out empty
         ranges, splits = max(1, min(splits, merge_in_workgroup)), merge_in_workgroup
-    start = (k_begin // KEY_ALIGN) * KEY_ALIGN
+    start = (k_begin // key_align) * key_align
     per = -(-(k_end - start) // (ranges if merge_in_workgroup else splits))
-    per = -(-per // KEY_ALIGN) * KEY_ALIGN
+    per = -(-per // key_align) * key_align
     piece = start[:, None] + np.arange(splits, dtype=np.int64)[None, :] * per[:, None]
     lo = np.maximum(piece, k_begin[:, None])
     hi = np.minimum(piece + per[:, None], k_end[:, None])
@@ -255,7 +271,8 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     workgroup unless there are many), ``tile_key_ranges`` into how many ranges it lets the keys of a workgroup's tiles
     be cut, each for a workgroup of its own (1: it does not; more: rows of few tiles go to it as well, and their
     partial results are merged like those of split items)."""
-    _, tokens_per_tile, group_tiles = group_tiling(group_size)
+    _, tokens_per_tile, group_tiles = group_tiling(group_size, tuning.tile_rows)
+    key_align, key_step, most_splits = tuning.key_align, tuning.key_step, tuning.most_splits
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
     merge_in_workgroup = WORKGROUP_RANGES if merge_in_workgroup is True else int(merge_in_workgroup)
@@ -265,14 +282,14 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
         raise ValueError("a workgroup merges four key ranges of one tile, or two ranges of each of two tiles (an even number of rows)")
     if (merge_in_workgroup or (single_token_shortcut and fixed_splits is not None)) and len(row_len) \
             and int(row_len.min()) == 1 == int(row_len.max()):
-        return _single_token_plan(row_ctx, window, int(fixed_splits or merge_in_workgroup or 1), merge_in_workgroup)
+        return _single_token_plan(row_ctx, window, int(fixed_splits or merge_in_workgroup or 1), merge_in_workgroup, key_align)
     tiles_per_row = -(-row_len // tokens_per_tile)
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
     items, slots, merges, tiles = [], [], [], []
     n_slots = 0
     per_workgroup, halves, walk = 0, 1, None
     workgroups = {}
-    most_ranges = max(1, min(int(tile_key_ranges), MAX_SPLITS))
+    most_ranges = max(1, min(int(tile_key_ranges), most_splits))
     min_tiles = tuning.min_tiles_with_ranges if most_ranges > 1 else MIN_TILES_FOR_WORKGROUPS
     # (rows of few tiles go there only if together they have as many as one row needs without ranges: a launch of its
     # own, and a merge, for a handful of tiles costs more than the items they would be beside the step's other rows)
@@ -292,10 +309,11 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
         rows_in_tiles = np.flatnonzero(tiles_per_row >= min_tiles)
         of_row, starts, k_begin, k_end, tiles_of_group = workgroups.get(per_workgroup) or _workgroups_of_rows(
             rows_in_tiles, row_len, row_ctx, tokens_per_tile, window, per_workgroup)
-        aligned = (k_begin // KEY_ALIGN) * KEY_ALIGN
-        steps = -(-(k_end - aligned) // 32)
-        per = -(-steps // _ranges_of_steps(steps, walk, most_ranges)) * 32
-        ranges = np.maximum(1, -(-(k_end - aligned) // np.maximum(per, 32)))      # (none of them empty)
+        aligned = (k_begin // key_align) * key_align
+        steps = -(-(k_end - aligned) // key_step)
+        per = -(-steps // _ranges_of_steps(steps, walk, most_ranges)) * key_step
+        per = -(-per // key_align) * key_align                                          # (ranges begin at multiples of key_align)
+        ranges = np.maximum(1, -(-(k_end - aligned) // np.maximum(per, key_align)))      # (none of them empty)
         cut = ranges > 1
         first = np.cumsum(np.where(cut, ranges * tiles_of_group, 0)) - np.where(cut, ranges * tiles_of_group, 0)
         n_slots = int(np.where(cut, ranges * tiles_of_group, 0).sum())
@@ -325,14 +343,14 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
             if fixed_splits is not None:
                 splits = fixed_splits
             elif waves_unsplit < target_waves:
-                splits = min(MAX_SPLITS, max(1, target_waves // max(1, waves_unsplit)), max(1, n_keys // MIN_KEYS_PER_SPLIT))
+                splits = min(most_splits, max(1, target_waves // max(1, waves_unsplit)), max(1, n_keys // tuning.fewest_keys_per_split))
             if splits <= 1:
                 items.append((row, q0, k_begin, k_end))
                 slots.append(-1)
                 continue
-            start = (k_begin // KEY_ALIGN) * KEY_ALIGN
+            start = (k_begin // key_align) * key_align
             per = -(-(k_end - start) // splits)
-            per = -(-per // KEY_ALIGN) * KEY_ALIGN        # at most `splits` items, each a multiple of KEY_ALIGN keys
+            per = -(-per // key_align) * key_align        # at most `splits` items, each a multiple of key_align keys
             first_slot = n_slots
             count = 0
             while start < k_end or (fixed_splits is not None and count < splits):
@@ -364,6 +382,9 @@ class GQAttention(Mixer):
             raise ValueError(f"Number of query heads must be divisible by the number of KV heads: query heads: {n_heads}, KV heads: {n_kv_heads}")
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
         self.group_size = n_heads // n_kv_heads
+        if position.rotary_dim is not None and position.rotary_dim != head_dim:
+            raise ValueError(f"the position encoding rotates {position.rotary_dim} of a head's {head_dim} dimensions; this mixer's "
+                             "kernels rotate the whole head or nothing (a rotation of a part of the head is not built)")
         self.position = position
         self.qk_norm_eps = qk_norm_eps
         self.window = window
@@ -408,22 +429,37 @@ class GQAttention(Mixer):
     def plan_key(self):
         return ("paged_attention", self.group_size, self.n_kv_heads, self.window)
 
+    def graph_shape(self, rows: int, longest_context: int):
+        return "short contexts" if longest_context <= SHORT_CONTEXT else None
+
+    def graph_shape_edges(self):
+        return (SHORT_CONTEXT,)
+
+    def mixing_flops(self, new_tokens: int, context: int) -> float:
+        """Scores and weighted values: two products of ``head_dim`` multiply-adds per query head, query and visible key."""
+        first = context - new_tokens
+        if self.window is None:
+            pairs = new_tokens * first + new_tokens * (new_tokens + 1) // 2
+        else:
+            pairs = sum(min(position + 1, self.window) for position in range(first, context))
+        return 4.0 * self.n_heads * self.head_dim * pairs
+
     def prepare(self, ctx):
         key = self.plan_key()
         if ctx.has_plan(key):
             return
         fixed = None
-        tuning = tuning_of(ctx.ops, DEFAULT_TUNING)
+        tuning = tuning_of(ctx.ops, DEFAULT_TUNING, ctx.dtype)
         if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
-            fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves)
+            fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
         # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:
-        #  * short contexts (the step says so, and keeps saying so for as long as its shape is replayed): four ranges a tile;
+        #  * short contexts (a shape of captured steps of its own, see graph_shape): four ranges a tile;
         #  * so many rows that a tile gets four ranges anyway;
         #  * two ranges a tile: two tiles to a workgroup, if the rows come in pairs.  (Two or three ranges in a workgroup
         #    of one tile leave wavefronts idle through the others' walk: a tenth slower at 64 rows behind 4,096 tokens.)
         in_workgroup = 0
         if ctx.n_tokens == ctx.n_rows:
-            if ctx.short_contexts:
+            if ctx.static_max_keys is not None and self.graph_shape(ctx.n_rows, int(np.max(ctx.h_row_ctx))) is not None:
                 in_workgroup = fixed = WORKGROUP_RANGES
             elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
                 in_workgroup = fixed

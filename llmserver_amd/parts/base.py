@@ -27,6 +27,9 @@ class ParamSpec:
     role: str = MATRIX
     init: str = "normal"          # "normal" | "norm" | "bias" | "zeros"
     optional: bool = False         # may be absent from the checkpoint
+    # The share of the tensor that one token's pass uses: 1 for a dense layer's matrix, k/n for one of n experts of
+    # which a token chooses k, 0 for a table of which a token reads a row.  (What a step costs is summed from this.)
+    share_per_token: float = 1.0
 
 
 @dataclasses.dataclass(frozen=True)
@@ -144,7 +147,10 @@ class ResidualSink:
 
 class PositionEncoding(Part):
     """How token positions enter a mixer.  ``rotary_table()`` returns the float32 inverse
-    frequencies ``[rotary_dim/2]`` of a rotate-half rotation, or None if nothing is rotated."""
+    frequencies ``[rotary_dim/2]`` of a rotate-half rotation, or None if nothing is rotated.  ``rotary_dim`` says how
+    many dimensions of a head the encoding rotates (None: none); a mixer checks it against what its kernels rotate."""
+
+    rotary_dim: Optional[int] = None
 
     def rotary_table(self, device) -> Optional[torch.Tensor]:
         return None
@@ -172,6 +178,23 @@ class Mixer(Part):
 
     def prepare(self, ctx) -> None:
         """Stage per-step metadata (host arrays) before the single upload of the step."""
+
+    def graph_shape(self, rows: int, longest_context: int):
+        """What a captured step of ``rows`` single tokens, the longest of whose contexts is ``longest_context``, depends
+        on in this mixer beyond the number of rows and the width of the block tables: anything hashable, None for
+        nothing.  Steps to which every mixer of the model gives equal answers share a graph, so the answer has to be
+        a pure function of the two numbers; the mixer asks itself the same question when it prepares such a step."""
+        return None
+
+    def graph_shape_edges(self):
+        """Contexts at which :meth:`graph_shape` changes its answer (a warm-up captures a graph on either side)."""
+        return ()
+
+    def mixing_flops(self, new_tokens: int, context: int) -> float:
+        """Floating-point operations between the mixer's projections for a row of ``new_tokens`` tokens that ends at a
+        context of ``context`` tokens (attention: scores and weighted values); the projections are counted from
+        ``param_specs``.  Only measurement reads this."""
+        return 0.0
 
     def forward(self, x, ctx, cache):
         """``x [T, H]`` normalised input -> ``[T, H]`` update to add to the residual stream."""

@@ -10,7 +10,7 @@ class TokenEmbedding(Part):
         self.weight = None
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.vocab, self.width), MATRIX, "normal")}
+        return {"weight": ParamSpec((self.vocab, self.width), MATRIX, "normal", share_per_token=0.0)}
 
     def assign(self, name, tensor):
         assert name == "weight"

@@ -30,7 +30,8 @@ class KernelNamespace:
     def add_rmsnorm(self, resid, delta, weight, eps, out, rows=None):
         raise NotImplementedError
 
-    def swiglu(self, gate_up, out):
+    def swiglu(self, gate_up, out, activation="silu"):
+        """``out = act(gate) * up`` with ``gate_up [T, 2I]``, gate first; a namespace refuses an ``activation`` it has not built."""
         raise NotImplementedError
 
     def add_bias_(self, y, bias):
@@ -77,9 +78,14 @@ class KernelNamespace:
     def library_is_faster(self, kind, x, weight, scaled=False, out_float32=False) -> bool:
         return False
 
-    def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None):
-        """Gate and up products with the activation in one launch, or None."""
+    def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None, activation="silu"):
+        """Gate and up products with the activation in one launch, or None (also for an ``activation`` it has not built)."""
         return None
+
+    def attention_tuning_for(self, dtype):
+        """``attention_tuning`` as it holds for tensors of ``dtype`` (kernels of different types may step through their
+        keys differently); here: the same for every type."""
+        return self.attention_tuning
 
     def attention_workgroup_tiles(self, dtype, head_dim, page_size=None) -> int:
         """Most tiles a workgroup of a prompt-portion attention kernel takes together; 0: there is no such kernel."""
@@ -104,6 +110,7 @@ class KernelNamespace:
         return contextlib.nullcontext(None)
 
 
-def tuning_of(ops: KernelNamespace, default):
-    tuning: Optional[object] = ops.attention_tuning
+def tuning_of(ops: KernelNamespace, default, dtype=None):
+    """The namespace's attention tuning for steps of this type, or ``default`` where it has none."""
+    tuning: Optional[object] = ops.attention_tuning_for(dtype) if dtype is not None else ops.attention_tuning
     return tuning if tuning is not None else default

@@ -1,4 +1,4 @@
-"""Gated feed-forward ``down(silu(gate(x)) * up(x))``.
+"""Gated feed-forward ``down(act(gate(x)) * up(x))``; ``act`` is SiLU in every model built so far.
 
 Gate and up are one stacked product, gate first (utils/layers.py:194-218;
 utils/fused_ops.py:59-61, 80-88).  Sigmoid and the product run in 32-bit inside
@@ -25,10 +25,15 @@ class GatedMLP(FeedForward):
     accepts_pending_norm = True
     takes_sink = True
 
+    # config.json's names of an activation -> the name the kernels know it by (utils/layers.py:182 in the
+    # reference lists more; a further one is an entry here and a branch in the activation kernel and the gated epilogues)
+    ACTIVATIONS = {"silu": "silu", "swish": "silu"}
+
     def __init__(self, width: int, intermediate: int, activation: str = "silu", bias: bool = False,
                  names: GatedMLPNames = GatedMLPNames()):
-        if activation not in ("silu", "swish"):
-            raise ValueError(f"Unsupported activation {activation!r}; supported: ['silu', 'swish']")
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"Unsupported activation {activation!r}; supported: {sorted(self.ACTIVATIONS)}")
+        self.activation = self.ACTIVATIONS[activation]
         self.width = width
         self.intermediate = intermediate
         if len(names.gate_up) not in (1, 2):
@@ -65,7 +70,7 @@ class GatedMLP(FeedForward):
                     tensor, row_scale = scaled
                 else:
                     tensor = x.tensor()
-            hidden = ops.linear_gated(tensor, self.gate_up.weight, row_scale=row_scale)
+            hidden = ops.linear_gated(tensor, self.gate_up.weight, row_scale=row_scale, activation=self.activation)
             if hidden is not None:
                 return self.down.forward(hidden, ctx, sink=sink)
             if row_scale is not None:
@@ -73,5 +78,5 @@ class GatedMLP(FeedForward):
             x = tensor
         gate_up = self.gate_up.forward(x, ctx)
         hidden = ctx.empty((gate_up.shape[0], self.intermediate))
-        ops.swiglu(gate_up, hidden)
+        ops.swiglu(gate_up, hidden, activation=self.activation)
         return self.down.forward(hidden, ctx, sink=sink)

@@ -24,15 +24,15 @@ def test_matrix_one_prompt_and_mixed_workload(tmp_path, capsys):
     assert all(r["decode_tok_s"] > 0 and r["ttft_s"] > 0 and len(r["tokens"]) == r["batch"] and len(r["tokens"][0]) == 6 for r in results)
     # the matrix's prompts are seeded: the same ids here, through the plain implementation
     config, tensors = plain_model(case)
-    prompt = benchmark.build_prompts(raw["vocab_size"], 9, 1, "tn-9-1-0", 0)[0]
+    prompt = benchmark.matrix_prompts(raw["vocab_size"], 9, 1, "whole-run", 0, 0)[0]
     assert results[0]["tokens"][0] == plain.greedy_generate(config, tensors, prompt, 6)
     capsys.readouterr()
     prompt = random_tokens(raw["vocab_size"], 7, 3)
     assert benchmark.main(["--model", folder, "--custom-dtype", "fp32", "--prompt-token-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5",
                            "--repeats", "2", "--block-size", str(page)]) == 0
     printed = capsys.readouterr().out
-    assert f"Response: {plain.greedy_generate(config, tensors, prompt, 5)}" in printed
-    assert "Prompt tokens: 7 | Generated tokens: 5" in printed and "Time to first token:" in printed and "median decode throughput:" in printed
+    assert f"response: {plain.greedy_generate(config, tensors, prompt, 5)}" in printed
+    assert "7 in the prompt, 5 generated" in printed and "first token:" in printed and "medians of 2 runs: first token" in printed
     assert benchmark.main(["--model", folder, "--prompt", "text without a tokenizer"]) == 2
     assert benchmark.main(["--random-config", "tiny-b", "--mixed-requests", "6", "--mixed-prompt-range", "4,40", "--shared-prefix-tokens", "16",
                            "--output-tokens", "5", "--block-size", "8", "--max-num-batched-tokens", "64", "--profile",

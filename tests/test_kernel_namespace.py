@@ -96,3 +96,36 @@ def test_pools_that_let_a_context_outgrow_the_kernels_page_lookup_are_refused():
         HipOps.check_cache_geometry(specs, 6, 10)
     with pytest.raises(ValueError):
         HipOps.check_cache_geometry({0: PagedKVSpec(2, 40, None)}, 16, 10)
+
+
+def test_parts_refuse_what_their_kernels_do_not_compute_when_they_are_made():
+    """A position encoding that rotates a part of the head, or an activation that the kernels do not compute, is refused
+    with the reason by the part's constructor, not by a shape check at the first step."""
+    from llmserver_amd.parts import GatedMLP, GQAttention, NoPosition, RotaryPosition
+    with pytest.raises(ValueError, match="rotates 16 of a head's 32 dimensions"):
+        GQAttention(64, 4, 2, 32, RotaryPosition(16, 1e4))
+    assert GQAttention(64, 4, 2, 32, RotaryPosition(32, 1e4)).position.rotary_dim == 32
+    assert GQAttention(64, 4, 2, 32, NoPosition()).position.rotary_dim is None
+    with pytest.raises(ValueError, match="Unsupported activation 'gelu'"):
+        GatedMLP(64, 128, "gelu")
+    assert GatedMLP(64, 128, "swish").activation == "silu"
+    # a namespace's fused product declines an activation it has not built (the caller then takes the separate kernels,
+    # whose activation kernel refuses it by name)
+    from llmserver_amd.kernels.ops import HipOps
+    assert HipOps.linear_gated(HipOps.__new__(HipOps), torch.zeros(2, 8), torch.zeros(16, 8), activation="gelu") is None
+    with pytest.raises(ValueError, match="'gelu' is not built"):
+        HipOps.swiglu(HipOps.__new__(HipOps), torch.zeros(2, 8), torch.zeros(2, 4), activation="gelu")
+
+
+def test_a_mixer_tells_the_step_what_its_captured_work_depends_on():
+    """The step function knows nothing of attention's short contexts: a mixer answers ``graph_shape`` (and names the
+    contexts at which its answer changes), steps with equal answers share a graph."""
+    from llmserver_amd.parts import GQAttention, Mixer, NoPosition
+    from llmserver_amd.parts.attention import SHORT_CONTEXT
+    attention = GQAttention(64, 4, 2, 32, NoPosition())
+    assert attention.graph_shape(8, SHORT_CONTEXT) == attention.graph_shape(1, 1) != attention.graph_shape(8, SHORT_CONTEXT + 1)
+    assert attention.graph_shape(8, 10 ** 6) is None and attention.graph_shape_edges() == (SHORT_CONTEXT,)
+    assert Mixer().graph_shape(3, 5) is None and Mixer().graph_shape_edges() == ()
+    import llmserver_amd.engine.step as step
+    import llmserver_amd.engine.batch as batch
+    assert "SHORT_CONTEXT" not in vars(step) and "short_contexts" not in inspect.getsource(batch)

@@ -57,7 +57,7 @@ class TorchOps(KernelNamespace):
         parts = torch.stack([squares[:, i::3].sum(dim=1) for i in range(3)], dim=1)      # any split of the row will do
         return stream, weighted, parts
 
-    def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None):
+    def linear_gated(self, x, gate_up_weight, pairs_per_workgroup=0, row_scale=None, activation="silu"):
         beyond = self.fused and row_scale is None and 16 < x.shape[0] <= 32            # the kernel for more rows has no row scale
         if not beyond and not self.row_scale_fits(x, gate_up_weight, row_scale):
             return None
@@ -105,7 +105,7 @@ class TorchOps(KernelNamespace):
         normed = total * torch.rsqrt(total.pow(2).mean(dim=-1, keepdim=True) + eps) * weight
         out.copy_(normed.to(out.dtype))
 
-    def swiglu(self, gate_up, out):
+    def swiglu(self, gate_up, out, activation="silu"):
         inter = out.shape[1]
         gate, up = gate_up[:, :inter].float(), gate_up[:, inter:].float()
         out.copy_((gate * torch.sigmoid(gate) * up).to(out.dtype))
