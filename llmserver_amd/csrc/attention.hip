@@ -588,8 +588,17 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
 // stores on the way), into a ring of STAGES buffers: the loads of step i + STAGES - 1 are issued before the products
 // of step i, one barrier a step, and every wavefront reads its MFMA operands from LDS, 16 bytes per lane and read
 // (8-byte reads reach three quarters of the LDS rate at best).  Rows in LDS are padded so that the operand
-// reads of a wavefront spread over the banks.  No key ranges are split here: such
-// rows have many tiles.  `tiles[i]` = {row, first token of the workgroup's tiles, k_begin, k_end}.
+// reads of a wavefront spread over the banks.  `tiles[i]` = {row, first token of the workgroup's tiles, k_begin, k_end}.
+// The wavefronts of a workgroup come in one or two halves (HALVES, see below), each with a ring of its own.
+//
+// Key ranges: an entry of `tiles` may cover only a range [k_begin, k_end) of the keys that its tiles see, the other
+// ranges being other entries (workgroups of their own).  `tile_slots[i]` = {first slot, slots between one tile and the
+// next} then says where entry i leaves its partial results: tile j of the entry writes (max, sum, acc) of every valid
+// pair to slot first + j * stride, in the layout of the wavefront-per-tile kernel, and merge_kernel combines the slots of
+// a tile.  first = -1 (or no `tile_slots` at all): the entry has all keys of its tiles and writes the output itself.
+// What the merge relies on: every slot that a merge entry names is written for every pair the merge reads, also by an
+// entry none of whose keys a pair may see (it writes max = -inf, sum = 0, acc = 0, which the merge weighs with zero);
+// pairs beyond the row's tokens or the group's heads are never read by the merge, and never written here.
 //
 // A load writes 64 lanes x 16 bytes to 1 KB of LDS in lane order, from wherever each lane points: a step's buffer is
 // a row of such 1 KB chunks, and a lane's place in its chunk says which 16 bytes of the step it fetches (the padding

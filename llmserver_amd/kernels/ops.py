@@ -97,31 +97,38 @@ class HipOps(KernelNamespace):
         self._measuring = False
         self._flush = None
         self._replay_overhead = None
-        self._tuning = None
-        self._tuning_f32 = None
+        self._tunings = {}
+
+    # What the prompt-portion kernel's launches cost, per kind of GPU: measured at head size 128 (a launch of one prompt of
+    # 512 to 4,096 tokens, of several, and of portions behind long prefixes; eight tiles to a workgroup do more with each
+    # key they load but start later, two halves shorten the longest workgroup's walk but make every step dearer).  A GPU
+    # that is not listed plans with the attention part's neutral costs; other head sizes scale the trips and steps by
+    # head size / 128 (loads and products of a step grow with the head; untuned beyond that).
+    TILE_COSTS = {"gfx950-256cu": (((False, 1), TileLaunchCost(3.2, 0.89, 1.55)), ((True, 1), TileLaunchCost(8.7, 0.94, 2.45)),
+                                   ((False, 2), TileLaunchCost(3.3, 1.11, 2.08)), ((True, 2), TileLaunchCost(8.8, 1.44, 2.84)))}
+    TILE_COSTS_HEAD_DIM = 128
 
     @property
     def attention_tuning(self) -> AttentionTuning:
         """What the attention plan should know of this GPU: four wavefronts in flight per compute unit (more and shorter
         key ranges cost more in the merge than they gain), and what the prompt-portion kernel costs in each of its four
-        forms (measured on an MI355X at head size 128: a launch of one prompt of 512 to 4,096 tokens, of several, and of
-        portions behind long prefixes; eight tiles to a workgroup do more with each key they load but start later, two
-        halves shorten the longest workgroup's walk but make every step dearer)."""
-        if self._tuning is None:
-            units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-            costs = (((False, 1), TileLaunchCost(3.2, 0.89, 1.55)), ((True, 1), TileLaunchCost(8.7, 0.94, 2.45)),
-                     ((False, 2), TileLaunchCost(3.3, 1.11, 2.08)), ((True, 2), TileLaunchCost(8.8, 1.44, 2.84)))
-            self._tuning = AttentionTuning(target_waves=4 * units, tile_costs=costs)
-        return self._tuning
+        forms on this kind of GPU, if that has been measured."""
+        return self.attention_tuning_for(torch.bfloat16, self.TILE_COSTS_HEAD_DIM)
 
-    def attention_tuning_for(self, dtype) -> AttentionTuning:
+    def attention_tuning_for(self, dtype, head_dim=None) -> AttentionTuning:
         """The float32 kernels step through 16 keys at a time (16x16x4 products), the bfloat16 ones through 32."""
-        tuning = self.attention_tuning
-        if dtype == torch.float32:
-            if self._tuning_f32 is None:
-                self._tuning_f32 = dataclasses.replace(tuning, key_step=16)
-            return self._tuning_f32
-        return tuning
+        head_dim = int(head_dim or self.TILE_COSTS_HEAD_DIM)
+        key = (dtype == torch.float32, head_dim)
+        if key not in self._tunings:
+            units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+            tuning = AttentionTuning(target_waves=4 * units, key_step=16 if dtype == torch.float32 else 32)
+            costs = self.TILE_COSTS.get(self.device_kind)
+            if costs is not None:
+                scale = head_dim / self.TILE_COSTS_HEAD_DIM
+                costs = tuple((form, TileLaunchCost(cost.start_us, cost.trip_us * scale, cost.step_ns * scale)) for form, cost in costs)
+                tuning = dataclasses.replace(tuning, tile_costs=costs)
+            self._tunings[key] = tuning
+        return self._tunings[key]
 
     @staticmethod
     def check_cache_geometry(cache_specs, page_size: int, num_pages=None) -> None:

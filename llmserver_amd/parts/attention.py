@@ -449,7 +449,7 @@ class GQAttention(Mixer):
         if ctx.has_plan(key):
             return
         fixed = None
-        tuning = tuning_of(ctx.ops, DEFAULT_TUNING, ctx.dtype)
+        tuning = tuning_of(ctx.ops, DEFAULT_TUNING, ctx.dtype, self.head_dim)
         if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
             fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
         # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:

@@ -82,9 +82,9 @@ class KernelNamespace:
         """Gate and up products with the activation in one launch, or None (also for an ``activation`` it has not built)."""
         return None
 
-    def attention_tuning_for(self, dtype):
-        """``attention_tuning`` as it holds for tensors of ``dtype`` (kernels of different types may step through their
-        keys differently); here: the same for every type."""
+    def attention_tuning_for(self, dtype, head_dim=None):
+        """``attention_tuning`` as it holds for tensors of ``dtype`` and heads of ``head_dim`` (kernels of different types
+        may step through their keys differently, and costs grow with the head); here: the same for all."""
         return self.attention_tuning
 
     def attention_workgroup_tiles(self, dtype, head_dim, page_size=None) -> int:
@@ -110,7 +110,7 @@ class KernelNamespace:
         return contextlib.nullcontext(None)
 
 
-def tuning_of(ops: KernelNamespace, default, dtype=None):
-    """The namespace's attention tuning for steps of this type, or ``default`` where it has none."""
-    tuning: Optional[object] = ops.attention_tuning_for(dtype) if dtype is not None else ops.attention_tuning
+def tuning_of(ops: KernelNamespace, default, dtype=None, head_dim=None):
+    """The namespace's attention tuning for steps of this type and head size, or ``default`` where it has none."""
+    tuning: Optional[object] = ops.attention_tuning_for(dtype, head_dim) if dtype is not None else ops.attention_tuning
     return tuning if tuning is not None else default

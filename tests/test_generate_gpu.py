@@ -276,13 +276,13 @@ def test_requests_arriving_over_time_with_shared_prefixes_and_few_pages(case, se
     for i in range(14):
         body = random_tokens(raw["vocab_size"], rng.randint(1, 60), 1000 + 50 * seed + i)
         prompts.append(prefix + body if rng.random() < 0.5 else body)
-        limits.append(rng.randint(1, 20))
+        limits.append(rng.randint(1, 40))           # (long enough that running requests outgrow their spare pages on the tight pool)
     expected = [plain.greedy_generate(config, tensors, p, n) for p, n in zip(prompts, limits)]
     longest = max(len(p) + n for p, n in zip(prompts, limits))
     preemptions_on_the_tight_pool = hits = 0
     for launch_ahead in (True, False):
         for pages in (400, -(-longest // page) + rng.choice((1, 3, 8))):
-            engine = Engine(model, None, max_new_tokens=20, max_batch_size=rng.choice((2, 4, 6)), max_num_batched_tokens=rng.choice((16, 32, 128)),
+            engine = Engine(model, None, max_new_tokens=40, max_batch_size=rng.choice((2, 4, 6)), max_num_batched_tokens=rng.choice((16, 32, 128)),
                             kv_cache_num_blocks=pages, kv_cache_block_size=page, ignore_eos=True, launch_ahead=launch_ahead)
             order, requests, steps = list(range(len(prompts))), {}, 0
             while order or engine.scheduler.waiting or engine.scheduler.running:

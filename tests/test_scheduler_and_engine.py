@@ -481,3 +481,38 @@ def test_an_offered_prefix_is_given_back_if_the_request_is_not_admitted_after_al
         pass
     engine.kv_cache.check_invariants()
     assert not engine.kv_cache.requests
+
+
+def test_a_preempted_request_at_the_head_of_the_queue_stalls_admissions_only_until_it_fits():
+    """This engine's own rule (a preempted request is admitted again only when all of it fits beside the running ones)
+    holds back whoever queued behind it meanwhile.  Under steady arrivals, with one long request that is preempted:
+    the stall ends when the running requests have finished (each is bounded by its own length limit), and everybody
+    finishes."""
+    engine, _ = scripted_engine([], max_new_tokens=6, max_batch_size=3, max_num_batched_tokens=16, kv_cache_num_blocks=16,
+                                kv_cache_block_size=2)
+    long = engine.add_request(None, list(range(5, 19)), max_new_tokens=12)           # 14 + 12 tokens: 13 of the 16 pages
+    others = [engine.add_request(None, [30 + i, 40 + i, 50 + i]) for i in range(2)]
+    finished, preempted_at, stalled, steps = [], None, 0, 0
+    arrivals = 0
+    while engine.has_work() or arrivals < 10:
+        if arrivals < 10 and steps % 2 == 0:                                         # a short request every other step
+            others.append(engine.add_request(None, [60 + arrivals, 70 + arrivals], max_new_tokens=4))
+            arrivals += 1
+        waiting_before = len(engine.scheduler.waiting)
+        running_before = len(engine.scheduler.running)
+        engine.step()
+        steps += 1
+        engine.kv_cache.check_invariants()
+        if preempted_at is None and long.preemption_count:
+            preempted_at = steps
+        head = engine.scheduler.waiting[0] if engine.scheduler.waiting else None
+        if head is long and waiting_before > 1 and running_before < 3:
+            stalled += 1                                                             # a place was free, somebody waited behind the long one
+        finished += [r for r in [long] + others if r.status == RequestStatus.FINISHED and r not in finished]
+        assert steps < 300
+    assert preempted_at is not None and long.preemption_count >= 1, "the pool was meant to be too small for all of them"
+    assert long.status == RequestStatus.FINISHED and len(long.generated_token_ids) == 12
+    assert all(r.status == RequestStatus.FINISHED for r in others)
+    # the stall is bounded by what the running requests still had to generate (at most 6 tokens each) plus the plan's own step
+    assert stalled <= 8, stalled
+    assert min(engine.kv_cache.available_pages()) == 16 and not engine.kv_cache.requests
