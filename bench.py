@@ -11,8 +11,10 @@ is decoded tokens per second; ``prefill`` times one engine step that takes a 2,0
 its arrival to its first token; ``roofline`` relates the bytes a decode step has to read (every
 weight once, plus the cache of the live requests) to the published HBM bandwidth; ``points`` holds
 batch 1 and 64 of the same model (tokens per second, with the step's milliseconds and its share of
-the HBM peak beside them), prompts of 512 and 8,192 tokens, a prompt of which all but the last 128 tokens lie in the cache already (8,064 of them: the next turn
-of a conversation) and four requests at a context of 16,384, and, unless ``--no-extra-points``, the two other workloads the baseline
+the HBM peak beside them), prompts of 512, 8,192 and 16,384 tokens, a prompt of which all but the last 128 tokens lie in
+the cache already (8,064 of them: the next turn of a conversation), four requests at a context of 16,384 and eight at
+32,768, the baseline's own decode workload (prompts of 2,048 tokens decoded to 4,096, every step timed, at batch 1, 8
+and 64) and, unless ``--no-extra-points``, the two other workloads the baseline
 names: 64 mixed requests with a shared prefix on Qwen3-1.7B sizes, and batch 16 behind 8,192 tokens
 on Qwen3-32B sizes.  Token ids are seeded uniform random numbers (synthetic data), weights seeded normal.
 """
@@ -242,6 +244,10 @@ def main() -> int:
             seconds = prefill_through_engine(model, args.page_size, tokens)
             points[f"prefill_{tokens}_ms"] = round(1000.0 * seconds, 3)
             points[f"prefill_{tokens}_mfma_frac"] = round(prefill_flops(model, tokens) / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)
+        log("[bench] prefill of 16,384 tokens")
+        seconds = prefill_through_engine(model, args.page_size, 16384, repeats=2)
+        points["prefill_16384_ms"] = round(1000.0 * seconds, 3)
+        points["prefill_16384_mfma_frac"] = round(prefill_flops(model, 16384) / seconds / (MFMA_PEAK_TFLOPS[short] * 1e12), 4)
         log("[bench] 128 new tokens behind 8,064 cached ones")
         points["turn_128_after_8064_ms"] = round(1000.0 * turn_through_engine(model, args.page_size, 8064, 128), 3)
         log("[bench] decode batch 4 at a context of 16,384")
@@ -249,6 +255,19 @@ def main() -> int:
         points["decode_b4_ctx16384"] = round(rate, 2)
         points["decode_b4_ctx16384_ms_per_step"] = round(ms, 4)
         points["decode_b4_ctx16384_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
+        log("[bench] decode batch 8 at a context of 32,768")
+        rate, ms, gbs = decode_point(model, args.page_size, 8, 32768, 32, 4)
+        points["decode_b8_ctx32768"] = round(rate, 2)
+        points["decode_b8_ctx32768_ms_per_step"] = round(ms, 4)
+        points["decode_b8_ctx32768_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
+        # The baseline's own decode workload: prompts of 2,048 tokens decoded greedily to 4,096 tokens in all, every
+        # decoding step of the run timed (2,040 of them after 8 of warm-up; mean context 3,076).
+        if args.context == 4096:
+            for batch in (1, 8, 64):
+                log(f"[bench] prompts of 2,048 tokens decoded to 4,096, batch {batch}")
+                rate, ms, gbs = decode_point(model, args.page_size, batch, 4096, 2040, 8)
+                points[f"decode_2048_to_4096_b{batch}"] = round(rate, 2)
+                points[f"decode_2048_to_4096_b{batch}_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
     del model
     torch.cuda.empty_cache()
     if not args.no_points and not args.no_extra_points and dtype == torch.bfloat16 and not args.layers:

@@ -41,7 +41,13 @@ class LayerCacheView:
     state: Optional[torch.Tensor] = None     # [slots, *shape] for a mixer with per-request state
 
 
-SCRATCH_PAGES = 16      # pages of storage beyond every pool (see CacheGroup.scratch_page)
+SCRATCH_PAGES = 16      # fewest pages of storage beyond every pool (see CacheGroup.scratch_page)
+SCRATCH_TOKENS = 512    # ... and as many as hold this many tokens: the filler tokens of a captured step with prompt portions
+
+
+def scratch_pages(page_size: int) -> int:
+    """Filler rows of one token take pages from the end of the scratch pages, a filler row of several tokens from their start."""
+    return SCRATCH_PAGES + -(-SCRATCH_TOKENS // page_size)
 
 
 class CacheGroup:
@@ -49,14 +55,16 @@ class CacheGroup:
         self.index, self.spec, self.caches = index, spec, caches
         self.pool = PagePool(num_pages, page_size)
         self.page_size = page_size
+        self.scratch_pages = scratch_pages(page_size)
         self.keys = None     # [len(caches), pages + SCRATCH_PAGES, kv_heads, page_size, head_dim]
         self.values = None   # [len(caches), pages + SCRATCH_PAGES, kv_heads, head_dim, page_size]
 
     def scratch_page(self, index: int) -> int:
         """One of the pages behind the pool's, which no request ever holds: rows that a step adds to fill a captured
-        shape write there (each its own page), and nobody reads them."""
-        if not 0 <= index < SCRATCH_PAGES:
-            raise ValueError(f"scratch pages are 0..{SCRATCH_PAGES - 1}, asked for {index}")
+        shape write there (each filler row of one token its own page, a filler row of several tokens as many pages as
+        it needs), and no request reads them."""
+        if not 0 <= index < self.scratch_pages:
+            raise ValueError(f"scratch pages are 0..{self.scratch_pages - 1}, asked for {index}")
         return self.pool.num_pages + index
 
     def first_needed_block(self, num_computed: int) -> int:
@@ -133,7 +141,7 @@ class CacheManager:
     def _allocate_storage(self):
         for group in self.groups:
             spec, n = group.spec, len(group.caches)
-            pages = group.pool.num_pages + SCRATCH_PAGES
+            pages = group.pool.num_pages + group.scratch_pages
             group.keys = torch.zeros((n, pages, spec.n_kv_heads, self.page_size, spec.head_dim), device=self.device, dtype=self.dtype)
             group.values = torch.zeros((n, pages, spec.n_kv_heads, spec.head_dim, self.page_size), device=self.device, dtype=self.dtype)
         for cache, spec in self.state_specs.items():

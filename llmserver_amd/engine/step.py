@@ -22,7 +22,7 @@ from __future__ import annotations
 
 import warnings
 from collections import OrderedDict
-from typing import Optional, Sequence
+from typing import Dict, Optional, Sequence
 
 import numpy as np
 import torch
@@ -32,6 +32,18 @@ from .batch import Staging, StepContext, StepEntry
 
 TABLE_WIDTH_STEP = 64      # captured steps serve block tables up to the next multiple of this many pages
 MAX_GRAPHS = 96
+# Steps that bring portions of prompts are captured too while they are small (there the host's work per launch, not the
+# GPU's, bounds the step): up to this many rows, their tokens filled up to one of these numbers.
+PORTION_ROWS = 16
+PORTION_TOKENS = (8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512)
+PORTION_MEETINGS = 2        # a shape of such a step is captured when it is met for this many times (shapes are many, captures cost a step or two)
+# ... and only where the host is what bounds it.  Launched one by one, a step takes the longer of the host's and the GPU's
+# time; replayed, the GPU's (and somewhat more of that: a captured step's attention cannot choose its kernel by the rows'
+# lengths).  The host's time is about 140 us a layer call (nine or ten launches from Python, a library product 20 us each);
+# the GPU's is estimated from what the step reads and multiplies at the rates that small steps reach.
+HOST_SECONDS_PER_LAYER_CALL = 140e-6
+SMALL_STEP_BYTES_PER_SECOND = 4e12
+SMALL_STEP_FLOPS_PER_SECOND = 1e15
 
 
 def padded_rows(rows: int) -> int:
@@ -42,6 +54,14 @@ def padded_rows(rows: int) -> int:
         return rows
     step = 2 if rows <= 16 else 4 if rows <= 32 else 8 if rows <= 64 else 16
     return -(-rows // step) * step
+
+
+def padded_tokens(tokens: int) -> Optional[int]:
+    """The number of tokens a captured step with portions of ``tokens`` tokens runs with; None: too many to capture."""
+    for size in PORTION_TOKENS:
+        if tokens <= size:
+            return size
+    return None
 
 
 class _CapturedStep:
@@ -66,7 +86,10 @@ class ModelRunner:
         if use_graphs is None:
             use_graphs = self.device.type == "cuda" and ops.name == "hip"
         self.use_graphs = bool(use_graphs and graph_safe)
+        self.capture_portions = True      # small steps that bring prompt portions are replayed from graphs as well
         self._graphs: "OrderedDict[tuple, _CapturedStep]" = OrderedDict()
+        self._met: Dict[tuple, int] = {}  # how often a shape of a step with portions has been met (see PORTION_MEETINGS)
+        self._host_bound: Dict[tuple, bool] = {}
         self.graph_replays = 0
         self._ahead = None          # (graph key, request ids, staged context) of a decoding step prepared ahead
         self._launched = None       # (request ids, their contexts after it, logits) of a step started ahead of its tokens
@@ -74,10 +97,14 @@ class ModelRunner:
         self.steps_launched_ahead = 0
 
     def build_context(self, entries: Sequence[StepEntry], staging: Optional[Staging] = None,
-                      table_width: Optional[int] = None, filler_rows: int = 0) -> StepContext:
+                      table_width: Optional[int] = None, filler_rows: int = 0, filler_tokens: Optional[int] = None,
+                      want_last: Optional[bool] = None) -> StepContext:
         """Check the entries against the cache, allocate their pages, lay out the flat batch.  ``filler_rows`` more rows
         follow the entries', each a first token of nobody's on a scratch page of its own, its logits wanted: they
-        bring a step of single tokens to the shape of a captured one."""
+        bring a step of single tokens to the shape of a captured one.  ``filler_tokens`` (a number, possibly 0): one
+        more row of nobody's with that many tokens, the start of a prompt on scratch pages, which brings the step's
+        tokens to a captured number.  ``want_last``: instead of the entries' own wanted places, the last token of
+        every row (True) or nothing (False), so that the wanted places have a captured shape as well."""
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
@@ -100,7 +127,10 @@ class ModelRunner:
             for place in entry.want:
                 if not 0 <= place < count:
                     raise ValueError(f"wanted place {place} is outside the {count} tokens of request {entry.request_id!r}")
-                logit_idx.append(n_tokens + place)
+                if want_last is None:
+                    logit_idx.append(n_tokens + place)
+            if want_last:
+                logit_idx.append(n_tokens + count - 1)
             row_start.append(n_tokens)
             row_len.append(count)
             row_ctx.append(start + count)
@@ -113,26 +143,42 @@ class ModelRunner:
             self.cache.ensure(entry.request_id, ctx_len)
         if filler_rows:
             fillers = np.arange(filler_rows, dtype=np.int64)
-            logit_idx.extend((n_tokens + fillers).tolist())
+            if want_last is not False:
+                logit_idx.extend((n_tokens + fillers).tolist())
             row_start.extend((n_tokens + fillers).tolist())
             row_len.extend([1] * filler_rows)
             row_ctx.extend([1] * filler_rows)
             token_row.append(len(entries) + fillers)
             token_ids.append(np.zeros(filler_rows, dtype=np.int64))
             positions.append(np.zeros(filler_rows, dtype=np.int64))
+        extra_rows = filler_rows
+        if filler_tokens is not None:
+            first = n_tokens + filler_rows
+            if want_last:
+                logit_idx.append(first + max(filler_tokens, 1) - 1 if filler_tokens else 0)     # (an empty row has no last token: any place will do)
+            row_start.append(first)
+            row_len.append(filler_tokens)
+            row_ctx.append(filler_tokens)
+            token_row.append(np.full(filler_tokens, len(entries) + filler_rows, dtype=np.int64))
+            token_ids.append(np.zeros(filler_tokens, dtype=np.int64))
+            positions.append(np.arange(filler_tokens, dtype=np.int64))
+            extra_rows += 1
         token_ids, positions, token_row = np.concatenate(token_ids), np.concatenate(positions), np.concatenate(token_row)
         tables = []
         records = [self.cache.record(rid) for rid in request_ids]
         for group in self.cache.groups:
             rows_pages = [record.table_array(group.index) for record in records]
             width = table_width if table_width is not None else max(1, max(len(pages) for pages in rows_pages))
-            table = np.full((len(entries) + filler_rows, width), -1, dtype=np.int32)
+            table = np.full((len(entries) + extra_rows, width), -1, dtype=np.int32)
             for row, pages in enumerate(rows_pages):
                 table[row, :len(pages)] = pages
-            for filler in range(filler_rows):
-                table[len(entries) + filler, 0] = group.scratch_page(filler)
+            for filler in range(filler_rows):           # (from the end of the scratch pages: the row of several tokens has their start)
+                table[len(entries) + filler, 0] = group.scratch_page(group.scratch_pages - 1 - filler)
+            if filler_tokens:
+                for block in range(-(-filler_tokens // group.page_size)):
+                    table[len(entries) + filler_rows, block] = group.scratch_page(block)
             tables.append(table)
-        request_ids = request_ids + [None] * filler_rows
+        request_ids = request_ids + [None] * extra_rows
         slots = None
         if self.cache.state_specs:
             slots = np.asarray([self.cache.record(rid).state_slot for rid in request_ids], dtype=np.int32)
@@ -146,8 +192,10 @@ class ModelRunner:
 
     # -- captured single-token steps ---------------------------------------------------------
     def _graph_key(self, entries: Sequence[StepEntry]):
-        if not self.use_graphs or any(len(entry.tokens) != 1 for entry in entries):
+        if not self.use_graphs:
             return None
+        if any(len(entry.tokens) != 1 for entry in entries):
+            return self._portion_key(entries)
         longest = 1
         for entry in entries:
             record = self.cache.requests.get(entry.request_id)
@@ -162,6 +210,56 @@ class ModelRunner:
         # what the mixers' captured work depends on beyond that (each asks itself the same when it prepares the step)
         shapes = tuple(dict.fromkeys(mixer.graph_shape(rows, longest) for mixer in self._mixers))
         return (rows, width, wanted, shapes)
+
+    def _host_bounds_a_step(self, tokens: int, keys: int) -> bool:
+        """Whether a step of ``tokens`` tokens behind up to ``keys`` keys takes the GPU less time than launching its
+        kernels takes the host (an estimate from the model's own sizes: the same answer in every run)."""
+        known = self._host_bound.get((tokens, keys))
+        if known is None:
+            from .cost import StepRow, step_bytes, step_flops
+            row = [StepRow(tokens, keys, 1)]
+            gpu = step_bytes(self.model, row, self.dtype) / SMALL_STEP_BYTES_PER_SECOND + step_flops(self.model, row) / SMALL_STEP_FLOPS_PER_SECOND
+            known = self._host_bound[(tokens, keys)] = gpu < len(self.model.order) * HOST_SECONDS_PER_LAYER_CALL
+        return known
+
+    def _portion_key(self, entries: Sequence[StepEntry]):
+        """The captured shape of a small step that brings portions of prompts (beside single tokens, possibly), or None
+        if it runs eagerly: too many rows or tokens, logits wanted elsewhere than at a row's last token (the engine
+        never asks for others; a trace may), a step that the GPU, not the host, bounds anyway, or a shape that has not
+        been met often enough yet.
+
+        Such a step is filled up with rows of nobody's: rows of one token as in decoding steps, and one more row (empty
+        if the numbers fit) with the tokens that are missing to the captured number, the start of a prompt on scratch
+        pages.  Its wanted places are every row's last token, or none."""
+        if not self.capture_portions or len(entries) > PORTION_ROWS:
+            return None
+        tokens, longest = 0, 1
+        for entry in entries:
+            record = self.cache.requests.get(entry.request_id)
+            want = list(entry.want)
+            if record is None or (want and want != [len(entry.tokens) - 1]):
+                return None
+            tokens += len(entry.tokens)
+            longest = max(longest, record.num_computed + len(entry.tokens))
+        rows = padded_rows(len(entries)) + 1
+        size = padded_tokens(tokens + rows - 1 - len(entries))          # the rows of one token that fill the rows up bring a token each
+        if size is None:
+            return None
+        longest = max(longest, size - tokens - (rows - 1 - len(entries)))
+        blocks = -(-longest // self.cache.page_size)
+        width = -(-blocks // TABLE_WIDTH_STEP) * TABLE_WIDTH_STEP
+        if not self._host_bounds_a_step(size, width * self.cache.page_size):
+            return None
+        wanted = rows if any(entry.want for entry in entries) else 0
+        shapes = tuple(dict.fromkeys(mixer.graph_shape(rows, longest) for mixer in self._mixers))
+        key = ("portions", rows, size, width, wanted, shapes)
+        if key not in self._graphs:
+            met = self._met[key] = self._met.get(key, 0) + 1
+            if len(self._met) > 4 * MAX_GRAPHS:
+                self._met.clear()
+            if met < PORTION_MEETINGS:
+                return None
+        return key
 
     @torch.inference_mode()
     def prepare_ahead(self, request_ids: Sequence[object]) -> bool:
@@ -253,7 +351,8 @@ class ModelRunner:
 
     def _step_captured(self, entries, key) -> torch.Tensor:
         captured = self._graphs.get(key)
-        ctx = self._take_ahead(entries, key) if captured is not None else None
+        portions = key[0] == "portions"
+        ctx = self._take_ahead(entries, key) if captured is not None and not portions else None
         if ctx is not None:
             self._graphs.move_to_end(key)
             ctx.staging.upload()
@@ -262,14 +361,32 @@ class ModelRunner:
             self.steps_prepared_ahead += 1
             return captured.logits[:len(entries)]
         staging = captured.staging if captured is not None else Staging(self.device, capacity=4096)
-        ctx = self.build_context(entries, staging=staging, table_width=key[1], filler_rows=key[0] - len(entries))
-        wanted = sum(len(entry.want) for entry in entries)           # the fillers' logits come last and are dropped
-        ctx.static_max_keys = key[1] * self.cache.page_size
+        if portions:
+            _, rows, size, width, wanted_rows, _ = key
+            tokens = sum(len(entry.tokens) for entry in entries)
+            filler_rows = rows - 1 - len(entries)
+            ctx = self.build_context(entries, staging=staging, table_width=width, filler_rows=filler_rows,
+                                     filler_tokens=size - tokens - filler_rows, want_last=bool(wanted_rows))
+            # every row's last token was computed: the rows that asked are handed out (the fillers' come last)
+            asked = [row for row, entry in enumerate(entries) if entry.want]
+
+            def select(logits):
+                if len(asked) == len(entries) or not len(asked):
+                    return logits[:len(asked)]
+                return logits[torch.tensor(asked, device=logits.device)]
+        else:
+            width = key[1]
+            ctx = self.build_context(entries, staging=staging, table_width=width, filler_rows=key[0] - len(entries))
+            wanted = sum(len(entry.want) for entry in entries)           # the fillers' logits come last and are dropped
+
+            def select(logits):
+                return logits[:wanted]
+        ctx.static_max_keys = width * self.cache.page_size
         self.model.prepare(ctx)
         if captured is None:
             ctx.static_max_keys = None           # the first upload may size the staging buffer
             ctx.upload()
-            ctx.static_max_keys = key[1] * self.cache.page_size
+            ctx.static_max_keys = width * self.cache.page_size
             logits = self.model.forward(ctx, self.cache)              # this step's result, run eagerly
             torch.cuda.synchronize(self.device)
             ctx.forget_computed()                # what the eager run computed on the device must be recorded too
@@ -279,15 +396,15 @@ class ModelRunner:
             self._graphs[key] = _CapturedStep(graph, static_logits, ctx.layout, staging)
             while len(self._graphs) > MAX_GRAPHS:
                 self._graphs.popitem(last=False)
-            return logits[:wanted]
+            return select(logits)
         self._graphs.move_to_end(key)
         ctx.upload()
         if ctx.layout != captured.layout:
             warnings.warn("a captured step met arrays of another shape; running it eagerly")
-            return self.model.forward(ctx, self.cache)[:wanted]
+            return select(self.model.forward(ctx, self.cache))
         captured.graph.replay()
         self.graph_replays += 1
-        return captured.logits[:wanted]
+        return select(captured.logits)
 
     def graph_count(self) -> int:
         return len(self._graphs)
@@ -305,7 +422,7 @@ class ModelRunner:
         if logits is not None or key is not None:
             if logits is None:
                 logits = self._step_captured(entries, key)
-            ctx_rows = [(entry.request_id, self.cache.record(entry.request_id).num_computed + 1) for entry in entries]
+            ctx_rows = [(entry.request_id, self.cache.record(entry.request_id).num_computed + len(entry.tokens)) for entry in entries]
         else:
             self._ahead = None
             ctx = self.build_context(entries)

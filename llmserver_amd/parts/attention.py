@@ -259,7 +259,7 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
                          target_waves: int = TARGET_WAVES, fixed_splits: Optional[int] = None,
                          workgroup_tiles: int = 0, single_token_shortcut: bool = True, merge_in_workgroup: int = 0,
                          tuning: AttentionTuning = DEFAULT_TUNING, tile_halves: int = 1, tile_min_workgroups: int = 0,
-                         tile_key_ranges: int = 1) -> AttentionPlan:
+                         tile_key_ranges: int = 1, fixed_tiles: Optional[int] = None) -> AttentionPlan:
     """Cut the step's rows into tiles of tokens and, where that pays, ranges of keys.
 
     With ``fixed_splits`` every tile gets exactly that many items (some may be empty), so the
@@ -270,7 +270,10 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     workgroups a launch of it needs to be worth while (a kernel whose steps are slow is bounded by its longest
     workgroup unless there are many), ``tile_key_ranges`` into how many ranges it lets the keys of a workgroup's tiles
     be cut, each for a workgroup of its own (1: it does not; more: rows of few tiles go to it as well, and their
-    partial results are merged like those of split items)."""
+    partial results are merged like those of split items).  ``fixed_tiles`` (with ``fixed_splits``): the arrays are
+    filled up to the shape of that many tiles, whatever the rows' lengths are (a captured step of prompt portions:
+    ``fixed_tiles`` is at least the number of tiles any rows of the step's shape can have), with repetitions of the
+    first tile's entries, which compute and write the same numbers once more."""
     _, tokens_per_tile, group_tiles = group_tiling(group_size, tuning.tile_rows)
     key_align, key_step, most_splits = tuning.key_align, tuning.key_step, tuning.most_splits
     row_len = np.asarray(row_len, dtype=np.int64)
@@ -361,6 +364,16 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
                 count += 1
                 start += per
             merges.append((row, q0, first_slot, count))
+    if fixed_tiles is not None:
+        if fixed_splits is None or len(tiles):
+            raise ValueError("a plan is filled up to a number of tiles only where every tile gets a fixed number of key ranges")
+        real = len(items) // fixed_splits
+        if real < 1 or real > fixed_tiles:
+            raise ValueError(f"the step's rows make {real} tiles, the shape it is filled up to holds {fixed_tiles}")
+        items += items[:fixed_splits] * (fixed_tiles - real)
+        slots += slots[:fixed_splits] * (fixed_tiles - real)
+        merges += merges[:1] * (fixed_tiles - real)
+        n_slots = fixed_tiles * fixed_splits if merges else 0
     items = np.asarray(items, dtype=np.int32).reshape(-1, 4)
     merges = np.asarray(merges, dtype=np.int32).reshape(-1, 4)
     tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 6)
@@ -448,17 +461,24 @@ class GQAttention(Mixer):
         key = self.plan_key()
         if ctx.has_plan(key):
             return
-        fixed = None
+        fixed = fixed_tiles = None
         tuning = tuning_of(ctx.ops, DEFAULT_TUNING, ctx.dtype, self.head_dim)
-        if ctx.static_max_keys is not None:          # a step whose shapes must not depend on the contexts
+        single_tokens = ctx.n_tokens == ctx.n_rows
+        if ctx.static_max_keys is not None and single_tokens:          # a step whose shapes must not depend on the contexts
             fixed = fixed_split_count(ctx.n_rows, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
+        elif ctx.static_max_keys is not None:
+            # ... nor on how its tokens are spread over its rows: as many tiles as rows of this many tokens can have at
+            # most (a row's last tile may be partly empty), every tile with the same number of key ranges.
+            _, tokens_per_tile, _ = group_tiling(self.group_size, tuning.tile_rows)
+            fixed_tiles = ctx.n_tokens // tokens_per_tile + ctx.n_rows
+            fixed = fixed_split_count(fixed_tiles, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
         # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:
         #  * short contexts (a shape of captured steps of its own, see graph_shape): four ranges a tile;
         #  * so many rows that a tile gets four ranges anyway;
         #  * two ranges a tile: two tiles to a workgroup, if the rows come in pairs.  (Two or three ranges in a workgroup
         #    of one tile leave wavefronts idle through the others' walk: a tenth slower at 64 rows behind 4,096 tokens.)
         in_workgroup = 0
-        if ctx.n_tokens == ctx.n_rows:
+        if single_tokens:
             if ctx.static_max_keys is not None and self.graph_shape(ctx.n_rows, int(np.max(ctx.h_row_ctx))) is not None:
                 in_workgroup = fixed = WORKGROUP_RANGES
             elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
@@ -470,7 +490,7 @@ class GQAttention(Mixer):
         plan = build_attention_plan(ctx.h_row_len, ctx.h_row_ctx, self.group_size, self.n_kv_heads, self.window,
                                     target_waves=tuning.target_waves, fixed_splits=fixed, workgroup_tiles=per_workgroup,
                                     merge_in_workgroup=in_workgroup, tuning=tuning, tile_halves=halves, tile_min_workgroups=fewest,
-                                    tile_key_ranges=key_ranges)
+                                    tile_key_ranges=key_ranges, fixed_tiles=fixed_tiles)
         ctx.set_plan(key, {
             **({"tile_slots": plan.tile_slots} if plan.tile_slots is not None else {}),
             "items": plan.items, "item_slot": plan.item_slot, "merges": plan.merges, "tiles": plan.tiles,

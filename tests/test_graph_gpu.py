@@ -1,5 +1,7 @@
-"""Captured single-token steps against the same steps run eagerly: every replay is checked, with
-eager work (portions of other prompts) and synchronisations between the replays."""
+"""Captured steps (single tokens; small steps with portions of prompts) against the same steps run eagerly: every
+replay is checked, with eager work (portions of other prompts) and synchronisations between the replays."""
+import random
+
 import pytest
 import torch
 
@@ -25,6 +27,7 @@ def test_replayed_steps_equal_eager_steps(case, n_live, dtype):
     for use_graphs in (True, False):
         cache = CacheManager(model.cache_specs(), page, 500, device="cuda", dtype=model.dtype)
         runners.append(ModelRunner(model, cache, use_graphs=use_graphs))
+        runners[-1].capture_portions = False       # (the portions between the replays are meant to be eager work here)
     lengths = [37, 5, 64, 1, 90, 16, 17, 33, 2, 70, 48, 9, 3, 81, 40, 7, 66, 21, 12, 55, 30, 8, 19, 44][:n_live]
     prompts = {f"r{i}": random_tokens(raw["vocab_size"], n, 1 + i) for i, n in enumerate(lengths)}
     feed = {rid: random_tokens(raw["vocab_size"], 80, 10 + i) for i, rid in enumerate(prompts)}
@@ -153,3 +156,69 @@ def test_steps_started_ahead_of_their_tokens_equal_steps_started_in_time(dtype):
         for rid in prompts:
             runner.cache.close(rid)
         assert all(group.pool.num_available == group.pool.num_pages for group in runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", ["B", "D"])
+def test_replayed_steps_with_portions_equal_eager_steps(case, dtype):
+    """Small steps that bring portions of prompts (alone, several, beside decoded tokens) are captured when their shape
+    has been met twice and replayed afterwards, filled up with rows and tokens of nobody's; whatever the portions'
+    lengths inside a shape, every step gives what the same step gives eagerly (where long rows go through other
+    kernels and key ranges are cut otherwise), also after pages were given back and used again, with the library's
+    products inside the graphs and eager steps between the replays."""
+    from llmserver_amd.cache import CacheManager
+    from llmserver_amd.engine import ModelRunner, StepEntry, load_model
+    print(f"graph replay of steps with portions {case} {dtype}", flush=True)
+    raw, _, page = CASES[case]
+    vocab = raw["vocab_size"]
+    model = load_model(model_folder(case), "cuda", dtype)
+    runners = []
+    for use_graphs in (True, False):
+        cache = CacheManager(model.cache_specs(), page, 300, device="cuda", dtype=model.dtype)
+        runners.append(ModelRunner(model, cache, use_graphs=use_graphs))
+    captured, eager = runners
+    rng = random.Random(11)
+    decoders = {f"d{i}": random_tokens(vocab, n, 1 + i) for i, n in enumerate((37, 5, 64, 1))}
+    feed = {rid: random_tokens(vocab, 200, 10 + i) for i, rid in enumerate(decoders)}
+    for runner in runners:
+        for rid, tokens in decoders.items():
+            runner.cache.open(rid)
+            runner.step([StepEntry(rid, tokens, [])])
+    prompts, fed, opened, worst, scale, compared = {}, {}, 0, 0.0, 0.0, 0
+    for turn in range(150):
+        while len(prompts) < 2:                                        # two prompts under way at any time
+            rid = f"p{opened}"
+            prompts[rid], fed[rid] = random_tokens(vocab, rng.choice((9, 30, 64, 100, 150)), 100 + opened), 0
+            opened += 1
+            for runner in runners:
+                runner.cache.open(rid)
+        entries = [StepEntry(rid, [feed[rid][turn]], [0]) for rid in rng.sample(sorted(decoders), rng.choice((0, 0, 1, 2, 4)))]
+        ended = []
+        for rid in sorted(prompts)[:rng.choice((1, 1, 2))]:
+            size = min(len(prompts[rid]) - fed[rid], rng.choice((2, 3, 7, 16, 31, 40)))
+            reaches_end = fed[rid] + size == len(prompts[rid])
+            entries.append(StepEntry(rid, prompts[rid][fed[rid]:fed[rid] + size], [size - 1] if reaches_end else []))
+            fed[rid] += size
+            if reaches_end:
+                ended.append(rid)
+        outs = [runner.step(entries).clone() for runner in runners]
+        torch.cuda.synchronize()
+        assert outs[0].shape == outs[1].shape == (sum(len(entry.want) for entry in entries), vocab)
+        if outs[1].numel():
+            worst, scale, compared = max(worst, float((outs[0] - outs[1]).abs().max())), max(scale, float(outs[1].abs().max())), compared + 1
+        for rid in ended:                                               # its pages go back and are used again by the next prompts
+            del prompts[rid]
+            for runner in runners:
+                runner.cache.close(rid)
+        if turn % 11 == 5:                                             # an eager step between the replays: too many tokens to be captured
+            for runner in runners:
+                runner.cache.open("long")
+                runner.step([StepEntry("long", random_tokens(vocab, 600, turn), [599])])
+                runner.cache.close("long")
+    kinds = [key[0] for key in captured._graphs]
+    print(f"  {captured.graph_replays} replays of {len(kinds)} graphs ({kinds.count('portions')} with portions); worst difference {worst:.2e} "
+          f"of logits up to {scale:.2e} in {compared} steps", flush=True)
+    assert kinds.count("portions") >= 4 and captured.graph_replays >= 60 and eager.graph_replays == 0
+    assert worst <= (2e-5 if dtype == "float32" else 1.5e-2) * scale, (worst, scale)
+    for runner in runners:
+        runner.cache.check_invariants()

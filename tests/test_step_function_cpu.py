@@ -119,6 +119,49 @@ def test_filler_rows_of_a_captured_shape(tmp_path):
     assert list(filled.h_row_ctx) == [6, 21, 1, 1, 1] and list(filled.h_row_len) == [1] * 5
     table = filled.h_tables[0]
     assert (table[:2, :plain.h_tables[0].shape[1]] == plain.h_tables[0]).all()
-    assert list(table[2:, 0]) == [pool_pages, pool_pages + 1, pool_pages + 2] and (table[2:, 1:] == -1).all()
-    assert runner.cache.groups[0].keys.shape[1] > pool_pages + 2
+    scratch = runner.cache.groups[0].scratch_pages          # (rows of one token take the last of the scratch pages)
+    assert list(table[2:, 0]) == [pool_pages + scratch - 1, pool_pages + scratch - 2, pool_pages + scratch - 3] and (table[2:, 1:] == -1).all()
+    assert runner.cache.groups[0].keys.shape[1] == pool_pages + scratch and scratch >= 16 + 512 // 16
+    runner.cache.check_invariants()
+
+
+def test_a_step_with_portions_filled_up_to_a_captured_shape():
+    """A small step that brings a portion of a prompt beside a decoded token is filled up to fixed numbers of rows and
+    tokens: rows of one token of nobody's, and one more row of nobody's with the tokens that are missing, the start of
+    a prompt on the first scratch pages (or no tokens at all, if the numbers fit).  The requests' own rows come out
+    as without the fillers, the attention plan has the shape that any rows of these numbers would give, and the
+    wanted places are every row's last token."""
+    import numpy as np
+    from llmserver_amd.engine import StepEntry
+    runner = make_runner(model_folder("A"), "float32", 256, 16, device="cpu", ops=TorchOps())
+    tokens = {"a": list(range(1, 41)), "b": list(range(50, 63))}
+    for name in tokens:
+        runner.cache.open(name)
+    runner.step([StepEntry("a", tokens["a"][:20], [])])
+    runner.step([StepEntry("b", tokens["b"][:12], [])])
+    entries = [StepEntry("a", tokens["a"][20:31], [10]), StepEntry("b", tokens["b"][12:], [0])]        # 11 + 1 tokens
+    plain = runner.build_context(entries)
+    shapes = []
+    for filler_tokens in (19, 0):                     # filled up to 32 tokens (with one filler row of one token); or the numbers fit
+        filled = runner.build_context(entries, table_width=64, filler_rows=1, filler_tokens=filler_tokens, want_last=True)
+        assert filled.n_rows == 4 and filled.n_tokens == 13 + filler_tokens and filled.n_out == 4
+        assert list(filled.h_row_len) == [11, 1, 1, filler_tokens] and list(filled.h_row_ctx) == [31, 13, 1, filler_tokens]
+        assert list(filled.h_logit_idx[:3]) == [10, 11, 12] and 0 <= filled.h_logit_idx[3] < filled.n_tokens
+        assert list(filled.h_token_ids[:12]) == list(plain.h_token_ids) and list(filled.h_positions[13:]) == list(range(filler_tokens))
+        table, pool_pages = filled.h_tables[0], runner.cache.groups[0].pool.num_pages
+        assert (table[:2, :plain.h_tables[0].shape[1]] == plain.h_tables[0]).all()
+        assert list(table[3, :2]) == ([pool_pages, pool_pages + 1] if filler_tokens else [-1, -1])
+        filled.static_max_keys = 64 * 16
+        runner.model.prepare(filled)
+        plan = filled.get_plan(runner.model.blocks[0].mixer.plan_key())
+        shapes.append((plan["items"].shape, plan["merges"].shape, plan["n_slots"], plan["n_tiles"]))
+        # every token of every row meets its keys: the tiles of a row cover its tokens, each tile's ranges its keys
+        covered = {}
+        for row, q0, k_begin, k_end in plan["items"].tolist():
+            covered.setdefault((row, q0), set()).update(range(k_begin, k_end))
+        for row, (length, context) in enumerate(zip(filled.h_row_len, filled.h_row_ctx)):
+            for q0 in range(0, int(length), 8):       # (two query heads to a KV head: eight tokens to a tile)
+                assert covered[(row, q0)] == set(range(int(context) - int(length) + min(q0 + 8, int(length)))), (row, q0)
+    # (the second has 19 tokens fewer: its shape is that of a smaller captured number of tokens, but rows and ranges agree)
+    assert shapes[0][0][0] == (32 // 8 + 4) * (shapes[0][0][0] // (32 // 8 + 4)) and shapes[0][3] == 0 and shapes[1][3] == 0
     runner.cache.check_invariants()
