@@ -8,8 +8,8 @@
 //   normalised, rotated and stored at keys[page][kv_head][slot][:]; v heads are stored transposed
 //   at values[page][kv_head][:][slot].  The page of a token is table[row][position / page_size];
 //   nothing is allocated here.
-// value_tiles: for long portions, the v heads go through LDS in tiles of 64 tokens so that the
-//   transposed stores of neighbouring tokens (neighbouring slots of a page) coalesce.
+//   For long portions, the v heads go through LDS in tiles of 64 tokens so that the transposed stores of
+//   neighbouring tokens (neighbouring slots of a page) coalesce: further workgroups of the same launch.
 // Norm sums, angles, cos/sin and the rotation are 32-bit; results are rounded once.
 #include "common.hpp"
 
@@ -68,7 +68,8 @@ __device__ inline void store8(T* p, const float (&v)[8]) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
+__device__ __forceinline__ void qk_norm_rope_kv_write_block(
+    const int block,
     T* __restrict__ qkv,                 // [tokens, (Hq + 2 Hkv) * d]
     T* __restrict__ keys,                // [pages, Hkv, page_size, d]
     T* __restrict__ values,              // [pages, Hkv, d, page_size]
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     const float* __restrict__ cos_sin,   // [tokens, d] (cos of the d/2 pairs, then sin) or nullptr
     int page_size, int n_q, int n_kv, int d, int write_cache, int n_heads, int n_tokens) {
     const int lanes_per_pair = d >> 4, pairs_per_wave = 64 / lanes_per_pair;
-    const int lane = threadIdx.x & 63, wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, wave = block * 4 + (threadIdx.x >> 6);
     const int slot_in_wave = lane / lanes_per_pair, j = lane % lanes_per_pair;
     const long pair = (long)wave * pairs_per_wave + slot_in_wave;
     const bool active = slot_in_wave < pairs_per_wave && pair < (long)n_tokens * n_heads;
@@ -151,15 +152,15 @@ constexpr int VT_TOKENS = 64;
 // dimension at a time (8 or 16 bytes) where four tokens are neighbours in one page, which is the
 // rule inside a portion; a page's [d][page_size] block is contiguous, so these stores coalesce.
 template <typename T>
-__global__ __launch_bounds__(256) void value_tiles_kernel(
+__device__ __forceinline__ void value_tiles_block(
+    const int tile_index, const int kv_head, unsigned char* tile_bytes,          // tile_bytes: [VT_TOKENS][d + VEC] elements of T in LDS
     const T* __restrict__ qkv, T* __restrict__ values, const int* __restrict__ table, int table_stride,
     const int* __restrict__ token_row, const int* __restrict__ positions, int page_size, int n_q, int n_kv, int d, int n_tokens) {
     constexpr int VEC = Elem<T>::kVec;
-    extern __shared__ unsigned char tile_bytes[];          // [VT_TOKENS][d + VEC] elements of T
     __shared__ long group_base[VT_TOKENS / 4];             // element offset of the group's first slot in `values`, or -1
     __shared__ unsigned char covered[VT_TOKENS];           // token goes out with its group
     T* tile = reinterpret_cast<T*>(tile_bytes);
-    const int token0 = blockIdx.x * VT_TOKENS, kv_head = blockIdx.y;
+    const int token0 = tile_index * VT_TOKENS;
     const int pitch = d + VEC;
     const int width = (n_q + 2 * n_kv) * d;
     const int pieces = d / VEC;
@@ -211,6 +212,24 @@ __global__ __launch_bounds__(256) void value_tiles_kernel(
     }
 }
 
+// One launch for both: the first `qk_blocks` workgroups take the (token, head) pairs of the q and k heads (and of the v
+// heads, unless these go in tiles), the others a tile of 64 tokens of one KV head's values each.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
+    T* __restrict__ qkv, T* __restrict__ keys, T* __restrict__ values, const int* __restrict__ table, int table_stride,
+    const int* __restrict__ token_row, const int* __restrict__ positions, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight, float eps, const float* __restrict__ cos_sin, int page_size, int n_q, int n_kv, int d,
+    int write_cache, int n_heads, int n_tokens, int qk_blocks) {
+    extern __shared__ unsigned char tile_bytes[];          // (none unless values go in tiles)
+    if ((int)blockIdx.x < qk_blocks) {
+        qk_norm_rope_kv_write_block<T>((int)blockIdx.x, qkv, keys, values, table, table_stride, token_row, positions, q_weight, k_weight, eps,
+                                       cos_sin, page_size, n_q, n_kv, d, write_cache, n_heads, n_tokens);
+        return;
+    }
+    const int tile = ((int)blockIdx.x - qk_blocks) / n_kv, kv_head = ((int)blockIdx.x - qk_blocks) % n_kv;
+    value_tiles_block<T>(tile, kv_head, tile_bytes, qkv, values, table, table_stride, token_row, positions, page_size, n_q, n_kv, d, n_tokens);
+}
+
 template <typename T>
 static int launch(void* qkv, void* keys, void* values, const int* table, int table_stride, const int* token_row,
                   const int* positions, const float* q_weight, const float* k_weight, float eps, const float* cos_sin,
@@ -222,15 +241,13 @@ static int launch(void* qkv, void* keys, void* values, const int* table, int tab
     if (d % 16 != 0 || d > 1024) return -1;
     const long pairs = (long)n_tokens * n_heads;
     const int pairs_per_block = 4 * (64 / (d / 16));
-    dim3 grid((unsigned)((pairs + pairs_per_block - 1) / pairs_per_block));
-    qk_norm_rope_kv_write_kernel<T><<<grid, 256, 0, stream>>>((T*)qkv, (T*)keys, (T*)values, table, table_stride, token_row,
-                                                              positions, q_weight, k_weight, eps, cos_sin, page_size,
-                                                              n_q, n_kv, d, write_cache, n_heads, n_tokens);
-    int err = (int)hipGetLastError();
-    if (err || !tiled_values) return err;
-    dim3 vgrid((n_tokens + VT_TOKENS - 1) / VT_TOKENS, n_kv);
-    value_tiles_kernel<T><<<vgrid, 256, VT_TOKENS * (d + Elem<T>::kVec) * sizeof(T), stream>>>((const T*)qkv, (T*)values, table, table_stride,
-                                                                                  token_row, positions, page_size, n_q, n_kv, d, n_tokens);
+    const long qk_blocks = (pairs + pairs_per_block - 1) / pairs_per_block;
+    const long value_blocks = tiled_values ? (long)((n_tokens + VT_TOKENS - 1) / VT_TOKENS) * n_kv : 0;
+    if (qk_blocks + value_blocks > 0x7fffffffL) return -1;
+    const size_t tile_bytes = tiled_values ? (size_t)VT_TOKENS * (d + Elem<T>::kVec) * sizeof(T) : 0;
+    qk_norm_rope_kv_write_kernel<T><<<dim3((unsigned)(qk_blocks + value_blocks)), 256, tile_bytes, stream>>>(
+        (T*)qkv, (T*)keys, (T*)values, table, table_stride, token_row, positions, q_weight, k_weight, eps, cos_sin, page_size,
+        n_q, n_kv, d, write_cache, n_heads, n_tokens, (int)qk_blocks);
     LSA_LAUNCH_CHECK();
 }
 

@@ -165,3 +165,42 @@ def test_a_step_with_portions_filled_up_to_a_captured_shape():
     # (the second has 19 tokens fewer: its shape is that of a smaller captured number of tokens, but rows and ranges agree)
     assert shapes[0][0][0] == (32 // 8 + 4) * (shapes[0][0][0] // (32 // 8 + 4)) and shapes[0][3] == 0 and shapes[1][3] == 0
     runner.cache.check_invariants()
+
+
+def test_which_steps_with_portions_are_captured():
+    """The shape a small step with portions is filled up to, and the steps that stay eager: too many rows or tokens,
+    logits wanted elsewhere than at a row's end, a shape met for the first time, and steps that the GPU bounds anyway
+    (estimated from the model's own sizes, so every run decides alike)."""
+    from llmserver_amd.engine import StepEntry
+    from llmserver_amd.engine.step import PORTION_ROWS, PORTION_TOKENS, padded_tokens
+    assert [padded_tokens(n) for n in (1, 8, 9, 100, 512, 513)] == [8, 8, 16, 128, 512, None] and list(PORTION_TOKENS) == sorted(PORTION_TOKENS)
+    runner = make_runner(model_folder("A"), "float32", 2048, 16, device="cpu", ops=TorchOps())
+    runner.use_graphs = True                      # (only the keys are asked for here; nothing is captured on the CPU)
+    for name in ("a", "b", "c"):
+        runner.cache.open(name)
+    runner.cache.advance("a", 0)
+    step = [StepEntry("a", list(range(40)), [39]), StepEntry("b", [5], [0])]
+    assert runner._graph_key(step) is None        # met for the first time
+    key = runner._graph_key(step)
+    assert key == ("portions", 3, 48, 64, 3, ("short contexts",))      # two rows and one of fillers; 41 tokens filled up to 48; all rows' ends wanted
+    assert runner._graph_key([StepEntry("a", list(range(44)), [43]), StepEntry("c", [1, 2, 3], [2])]) == key       # other lengths, the same shape
+    assert runner._graph_key([StepEntry("a", list(range(40)), []), StepEntry("b", [5, 6], [])]) is None            # nothing wanted: another shape, first meeting
+    assert runner._graph_key([StepEntry("a", list(range(40)), []), StepEntry("b", [5, 6], [])])[4] == 0
+    assert runner._graph_key([StepEntry("a", list(range(40)), [3])]) is None and runner._graph_key([StepEntry("a", list(range(40)), [3])]) is None   # a place inside the portion
+    many = [StepEntry(f"r{i}", [1, 2], [1]) for i in range(PORTION_ROWS + 1)]
+    for entry in many:
+        runner.cache.open(entry.request_id)
+    assert runner._graph_key(many) is None and runner._graph_key(many) is None
+    assert runner._graph_key([StepEntry("a", list(range(513)), [512])]) is None and runner._graph_key([StepEntry("a", list(range(513)), [512])]) is None
+    runner.capture_portions = False
+    assert runner._graph_key(step) is None
+    # the GPU's time against the host's: a tiny model is always the host's; at Qwen3-8B sizes a step of 128 tokens is the GPU's
+    import llmserver_amd.models  # noqa: F401
+    from llmserver_amd.config import named_config
+    from llmserver_amd.weights.random_init import build_model
+    assert runner._host_bounds_a_step(512, 1024)
+    runner.model, runner._host_bound = build_model(named_config("qwen3-8b")), {}
+    runner.dtype = torch.bfloat16
+    assert runner._host_bounds_a_step(16, 1024) and not runner._host_bounds_a_step(128, 1024) and not runner._host_bounds_a_step(32, 16384)
+    runner.model, runner._host_bound = build_model(named_config("qwen3-1.7b")), {}
+    assert runner._host_bounds_a_step(512, 1024)
