@@ -13,7 +13,7 @@ from safetensors.torch import load_file, save_file
 
 import plain_qwen3 as plain
 import traces
-from helpers import random_tokens
+from helpers import BF16, check_against_rounded_oracle, random_tokens, relative_error
 from llmserver_amd.config import config_from_dict
 from llmserver_amd.weights import RandomInit, write_random_model
 
@@ -41,7 +41,10 @@ def sharp_model(tmp_path_factory):
     with torch.no_grad():
         expected = {"main": plain.forward(config, tensors, main).numpy()}
         expected.update({rid: plain.forward(config, tensors, tokens).numpy() for rid, tokens in others.items()})
-    return folder, main, others, expected
+        # what bfloat16 loses on these sequences (sharp scores make the rounding of q and k count): the rounded oracle
+        lost = [relative_error(row, exact) for rid, tokens in dict(others, main=main).items()
+                for row, exact in zip(plain.forward(config, tensors, tokens, r=BF16).numpy(), expected[rid])]
+    return folder, main, others, expected, lost
 
 
 def build_steps(main, others):
@@ -65,7 +68,7 @@ def build_steps(main, others):
 def test_sharp_attention_over_a_long_context(sharp_model, dtype, tmp_path, monkeypatch):
     from llmserver_amd.engine.replay import make_runner, replay
     print(f"sharp attention over {LENGTH} tokens, {dtype}", flush=True)
-    folder, main, others, expected = sharp_model
+    folder, main, others, expected, lost = sharp_model
     steps, owner = build_steps(main, others)
     runner = make_runner(folder, dtype, traces.peak_tokens(steps), 16)
     out = str(tmp_path / "out")
@@ -82,7 +85,7 @@ def test_sharp_attention_over_a_long_context(sharp_model, dtype, tmp_path, monke
     errors = {}
     for (rid, position), logits in results.items():
         want = expected[owner[rid]][position]
-        errors.setdefault(rid, []).append(float(np.abs(logits - want).max()) / max(1.0, float(np.abs(want).max())))
+        errors.setdefault(rid, []).append(relative_error(logits, want))
     assert sum(len(v) for v in errors.values()) == 4 * LENGTH + sum(len(t) for t in others.values())
     worst = {rid: max(v) for rid, v in errors.items()}
     print("  worst by request:", {rid: f"{e:.2e}" for rid, e in worst.items()}, flush=True)
@@ -90,8 +93,7 @@ def test_sharp_attention_over_a_long_context(sharp_model, dtype, tmp_path, monke
         assert max(worst.values()) <= 3e-5, worst
     else:
         # rounding of q and k to 8 bits moves sharp scores by a tenth of a unit: several per cent of the largest logit
-        # at the worst places, a per cent at the median; a lost key moves them by tens of per cent
-        assert max(worst.values()) <= 0.12 and float(np.median(np.concatenate([np.asarray(v) for v in errors.values()]))) <= 0.03, worst
-        same_tokens = [float(np.abs(results[("w", p)] - results[(other, p)]).max()) / max(1.0, float(np.abs(results[("w", p)]).max()))
-                       for other in ("t", "p", "q") for p in range(LENGTH)]
-        assert max(same_tokens) <= 0.08, max(same_tokens)
+        # at the worst places, a per cent at the median, as the rounded oracle shows; a lost key moves them by tens of per cent
+        check_against_rounded_oracle(np.concatenate([np.asarray(v) for v in errors.values()]), lost, "sharp attention")
+        same_tokens = [relative_error(results[(other, p)], results[("w", p)]) for other in ("t", "p", "q") for p in range(LENGTH)]
+        check_against_rounded_oracle(same_tokens, lost, "sharp attention, the same request cut in other ways", factor=2.0)
