@@ -17,6 +17,9 @@ Such a step can be laid out on the host while the GPU still runs the step before
 the token ids is known then), and started before the host has seen those tokens (``launch_ahead``: the ids are copied
 on the device from the sampler's output); ``step`` then finds its work done, or drops it if the step that comes is
 another one.
+
+Small steps that bring portions of prompts are captured too, where launching their kernels one by one would take the
+host longer than running them takes the GPU (``_portion_key``).
 """
 from __future__ import annotations
 
