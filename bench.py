@@ -299,7 +299,12 @@ def extra_points(dtype, page_size):
     points["mixed_1p7b_64req_total_s"] = round(entry["total_s"], 3)
     points["mixed_1p7b_64req_prefix_hit_tokens"] = int(entry["prefix_hit_tokens"])
     points["mixed_1p7b_64req_prompt_tokens"] = int(entry["prompt_tokens_total"])
-    del engine, model
+    del engine
+    # Short prompts on the same model, from a request's arrival to its first token: steps of this size are replayed from
+    # graphs (launched one by one, the host would bound them).
+    for tokens in (32, 128):
+        points[f"first_token_1p7b_{tokens}_ms"] = round(1000.0 * prefill_through_engine(model, page_size, tokens, repeats=4), 3)
+    del model
     torch.cuda.empty_cache()
     # Batch 16 behind prompts of 8,192 tokens (Qwen3-32B sizes): the decoding steps up to a context of 8,192 + 64.
     model, config, _ = random_model("qwen3-32b", 0, dtype)
