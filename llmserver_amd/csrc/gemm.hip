@@ -376,12 +376,17 @@ static int compute_units() {
 // which costs no launch.
 constexpr int SPLIT_TILE_ROWS = 16 * GEMM_WAVES;       // rows of W per workgroup
 constexpr int SPLIT_MOST_ROWS = 128;                    // most rows of X
+constexpr int SPLIT_AHEAD_FROM_SLABS = 4;               // slabs of 256 columns a workgroup from which W is asked for a slab ahead (beyond 64 rows)
 
 // SLAB: columns of X staged at a time (512 up to 64 rows, 256 beyond: two slabs have to fit into LDS).
 // GATED: W stacks a gate matrix on an up matrix ([N, K], gate rows first) and the result wanted is
 // silu(x . gate^T) * (x . up^T) in bfloat16, [M, N / 2]: four wavefronts take 64 gate rows, the other four the up rows
 // that belong to them, and the two halves meet in the epilogue; one range of K only (nothing is left to add up).
-template <int MT, int SLAB, bool GATED>
+// AHEAD: the W of a slab is asked for a whole slab before it is met instead of half a slab.  With many rows of X a slab
+// takes long to multiply, and a request made only half a slab ahead is waited for at every slab; it costs the registers
+// of a second slab of W and a longer start, so it pays from four slabs a workgroup on (measured at 128 rows:
+// 4096 x 12288 36.5 -> 33 us, 5120 x 25600 89 -> 73 us; two slabs a workgroup 16.2 -> 16.8 us).
+template <int MT, int SLAB, bool GATED, bool AHEAD>
 __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                      void* __restrict__ out, int M, int N, int K, int k_range) {
     constexpr int SPLIT_PITCH = SLAB * 2 + 16;          // bytes per staged row: 16 rows apart are 64 banks apart
@@ -404,16 +409,23 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_
 #pragma unroll
         for (int u = 0; u < SPLIT_CHUNK; ++u) c.a[u] = *reinterpret_cast<const bf16x8*>(wp + min(k0 + 32 * u + 8 * quad, k_safe) - 8 * quad);
     };
+    // The operands of X for the next k step are read from LDS while the products of this one run.
+    struct Operands { bf16x8 b[MT]; };
+    auto read_operands = [&](Operands& o, const unsigned char* slab, int k_in_slab) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) o.b[t] = *reinterpret_cast<const bf16x8*>(slab + (16 * t + col) * SPLIT_PITCH + 2 * (k_in_slab + 8 * quad));
+    };
     auto multiply_chunk = [&](const Chunk& c, int k0, const unsigned char* slab, int k_in_slab) {
+        Operands even, odd;
+        read_operands(even, slab, k_in_slab);
 #pragma unroll
         for (int u = 0; u < SPLIT_CHUNK; ++u) {
+            if (u + 1 < SPLIT_CHUNK) read_operands((u & 1) ? even : odd, slab, k_in_slab + 32 * (u + 1));
+            const Operands& o = (u & 1) ? odd : even;
             bf16x8 a = c.a[u];
             if (k0 + 32 * u + 8 * quad >= k_last) a = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                const bf16x8 b = *reinterpret_cast<const bf16x8*>(slab + (16 * t + col) * SPLIT_PITCH + 2 * (k_in_slab + 32 * u + 8 * quad));
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
-            }
+            for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, o.b[t], acc[t], 0, 0, 0);
         }
     };
     // A slab of X: rows beyond M and columns beyond K are staged as zeros (their loads read a valid address).
@@ -434,8 +446,54 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_split_kernel(const bf16_
             *reinterpret_cast<bf16x8*>(slab + m * SPLIT_PITCH + 16 * piece) = v;
         }
     };
-    if (k_first < k_last) {
-        constexpr int HALF = 32 * SPLIT_CHUNK;          // a slab is two chunks of W
+    constexpr int HALF = 32 * SPLIT_CHUNK;          // a slab is two chunks of W
+    if (AHEAD && k_first < k_last) {
+        // Every load of the loop is issued whether or not its slab exists (a slab past the last one is the last one again,
+        // from cache): the number of loads in flight at each wait is then the same on every path, and no wait is for more
+        // than it needs.
+        const int n_slabs = (k_last - k_first + SLAB - 1) / SLAB, k_end = k_first + (n_slabs - 1) * SLAB;
+        Chunk p0, q0, p1, q1;
+        Slab next;
+        load_slab(next, k_first);
+        load_chunk(p0, k_first);
+        load_chunk(q0, k_first + HALF);
+        store_slab(next, k_first, staged);
+        __syncthreads();
+        load_chunk(p1, min(k_first + SLAB, k_end));
+        load_chunk(q1, min(k_first + SLAB, k_end) + HALF);
+        // The scheduler would move loads down to just before their use (fewer registers live): they stay where they are.
+        __builtin_amdgcn_sched_barrier(0);
+        int buffer = 0, k0 = k_first;
+        // A slab that another follows: its successor's X travels through registers to the other buffer while it is
+        // multiplied, and the W of the slab after that is asked for, a chunk as soon as the registers of one are free.
+        auto slab_and_next = [&](Chunk& p, Chunk& q) {
+            load_slab(next, k0 + SLAB);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply_chunk(p, k0, staged + buffer * BUFFER, 0);
+            load_chunk(p, min(k0 + 2 * SLAB, k_end));
+            __builtin_amdgcn_sched_barrier(0);
+            multiply_chunk(q, k0 + HALF, staged + buffer * BUFFER, HALF);
+            load_chunk(q, min(k0 + 2 * SLAB, k_end) + HALF);
+            __builtin_amdgcn_sched_barrier(0);
+            store_slab(next, k0 + SLAB, staged + (buffer ^ 1) * BUFFER);
+            __syncthreads();
+            buffer ^= 1;
+            k0 += SLAB;
+        };
+        int left = n_slabs;
+        for (; left > 2; left -= 2) {
+            slab_and_next(p0, q0);
+            slab_and_next(p1, q1);
+        }
+        if (left == 2) {
+            slab_and_next(p0, q0);
+            multiply_chunk(p1, k0, staged + buffer * BUFFER, 0);
+            multiply_chunk(q1, k0 + HALF, staged + buffer * BUFFER, HALF);
+        } else {
+            multiply_chunk(p0, k0, staged + buffer * BUFFER, 0);
+            multiply_chunk(q0, k0 + HALF, staged + buffer * BUFFER, HALF);
+        }
+    } else if (k_first < k_last) {
         Chunk p, q;
         Slab next;
         // Loads are issued in the order in which they are waited for: X of a slab before the W it meets.
@@ -684,26 +742,28 @@ LSA_EXPORT int lsa_gemm_split(const void* x, const void* w, float* partial, int 
     // More LDS than a kernel gets by default: asked for once per kernel and device.
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -1;
-#define LSA_SPLIT(MT, SLAB, GATED)                                                                                             \
+#define LSA_SPLIT(MT, SLAB, GATED, AHEAD)                                                                                      \
     {                                                                                                                          \
         static bool sized[64] = {};                                                                                            \
         constexpr int bytes = 2 * 16 * MT * (2 * SLAB + 16);                                                                   \
         if (!sized[device]) {                                                                                                  \
-            const hipError_t e = hipFuncSetAttribute((const void*)gemm_split_kernel<MT, SLAB, GATED>,                          \
+            const hipError_t e = hipFuncSetAttribute((const void*)gemm_split_kernel<MT, SLAB, GATED, AHEAD>,                   \
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, bytes);                       \
             if (e != hipSuccess) return (int)e;                                                                                \
             sized[device] = true;                                                                                              \
         }                                                                                                                      \
-        gemm_split_kernel<MT, SLAB, GATED><<<grid, block, bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, range); \
+        gemm_split_kernel<MT, SLAB, GATED, AHEAD><<<grid, block, bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, range); \
     }
     // Slabs of 512 columns where two of them fit into LDS and the range is made of whole ones (a slab is loaded whole).
     const bool wide = range % 512 == 0;
+    // Beyond 64 rows, W a whole slab ahead where a workgroup has four slabs or more (see the kernel).
+    const bool ahead = ((range < K ? range : K) + 255) / 256 >= SPLIT_AHEAD_FROM_SLABS;
     void* out = partial;
-    if (M <= 32) { if (wide) LSA_SPLIT(2, 512, false) else LSA_SPLIT(2, 256, false) }
-    else if (M <= 48) { if (wide) LSA_SPLIT(3, 512, false) else LSA_SPLIT(3, 256, false) }
-    else if (M <= 64) { if (wide) LSA_SPLIT(4, 512, false) else LSA_SPLIT(4, 256, false) }
-    else if (M <= 96) LSA_SPLIT(6, 256, false)
-    else LSA_SPLIT(8, 256, false)
+    if (M <= 32) { if (wide) LSA_SPLIT(2, 512, false, false) else LSA_SPLIT(2, 256, false, false) }
+    else if (M <= 48) { if (wide) LSA_SPLIT(3, 512, false, false) else LSA_SPLIT(3, 256, false, false) }
+    else if (M <= 64) { if (wide) LSA_SPLIT(4, 512, false, false) else LSA_SPLIT(4, 256, false, false) }
+    else if (M <= 96) { if (ahead) LSA_SPLIT(6, 256, false, true) else LSA_SPLIT(6, 256, false, false) }
+    else { if (ahead) LSA_SPLIT(8, 256, false, true) else LSA_SPLIT(8, 256, false, false) }
     LSA_LAUNCH_CHECK();
 }
 
@@ -727,7 +787,7 @@ LSA_EXPORT int lsa_gemm_split_gated(const void* x, const void* w, void* hidden, 
     if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -1;
     void* out = hidden;
     const bool wide = range % 512 == 0;
-    if (wide) LSA_SPLIT(2, 512, true) else LSA_SPLIT(2, 256, true)
+    if (wide) LSA_SPLIT(2, 512, true, false) else LSA_SPLIT(2, 256, true, false)
 #undef LSA_SPLIT
     LSA_LAUNCH_CHECK();
 }

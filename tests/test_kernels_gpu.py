@@ -537,11 +537,13 @@ def test_product_with_bias_is_rounded_once(ops, rows, n, k):
 
 
 @pytest.mark.parametrize("rows", [9, 16, 17, 32, 33, 48, 49, 64, 65, 96, 97, 128])
-@pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (2050, 1000), (200, 5128), (8192, 64), (5120, 520), (127, 264)])
+@pytest.mark.parametrize("n, k", [(48, 72), (301, 4096), (4096, 12288), (2050, 1000), (200, 5128), (8192, 64), (5120, 520), (127, 264),
+                                  (10880, 3840), (8192, 4104)])
 def test_product_in_partial_sums(ops, rows, n, k):
     """The product for 17 to 128 rows, which leaves partial sums over ranges of the inner dimension, against a float64
     product of the same bfloat16 values: one range and many, ranges that end inside a staged slab, sizes that are no
-    multiple of the tiles.  Then the kernel that adds them up, adds the result to a residual stream and normalises,
+    multiple of the tiles; ranges of six, five (an odd number) and four slabs and a last range of one whole slab and a
+    ragged one, which beyond 64 rows go through the form that asks for the weights a slab ahead.  Then the kernel that adds them up, adds the result to a residual stream and normalises,
     against its twin."""
     print(f"product in partial sums rows {rows} n {n} k {k}", flush=True)
     torch.manual_seed(rows * n + k)
