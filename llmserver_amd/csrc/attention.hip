@@ -91,7 +91,10 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
     const Item* __restrict__ items, const int* __restrict__ item_slot, int n_items,
     float* __restrict__ part_acc, float* __restrict__ part_ml, Geometry g, DecodeFusion fusion) {
     const int lane = threadIdx.x & 63;
-    const int item_index = blockIdx.x * 4 + (threadIdx.x >> 6);
+    // The wavefront's number, told to the compiler to be the same in all lanes: the item, its row and the key loop's bounds
+    // then live in scalar registers and the loop's branches are scalar ones (a hundred branches on the execution mask
+    // otherwise; batch 8 at context 4,096: 4.56 -> 4.53 ms a step).
+    const int item_index = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     constexpr bool WG_MERGE = WG_RANGES > 0;
     if (!WG_MERGE && item_index >= n_items) return;      // with WG_MERGE every wavefront has to reach the barrier at the end
     // The start of an item is a chain of loads, each of which needs the one before it (the item, its row, the row's

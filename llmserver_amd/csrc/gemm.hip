@@ -166,11 +166,19 @@ __global__ __launch_bounds__(GEMM_WAVES * 64) void gemm_skinny_kernel(const bf16
         int k0 = k_begin;
         int chunks = (k_end - k_begin + SPAN - 1) / SPAN;
         load_chunk(p, k0);
+        // The scheduling barriers keep a chunk's loads together and ahead of the products of the chunk before: left to
+        // itself the compiler spreads them between those products, a few at a time, each group waited for (down to "no
+        // load in flight") right behind the products it was issued between (output product of 4096 x 4096 at 8 rows
+        // 9.9 -> 8.8 us, down product 25.0 -> 24.0 us; in the two-tile kernel below they gain nothing).
         while (chunks >= 3) {
             load_chunk(q, k0 + SPAN);
+            __builtin_amdgcn_sched_barrier(0);
             multiply_chunk(p, k0);
+            __builtin_amdgcn_sched_barrier(0);
             load_chunk(p, k0 + 2 * SPAN);
+            __builtin_amdgcn_sched_barrier(0);
             multiply_chunk(q, k0 + SPAN);
+            __builtin_amdgcn_sched_barrier(0);
             k0 += 2 * SPAN;
             chunks -= 2;
         }
