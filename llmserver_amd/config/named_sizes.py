@@ -13,9 +13,15 @@ NAMED_SIZES = {
                    intermediate_size=128, vocab_size=256, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True),
     "tiny-b": dict(model_type="qwen3", num_hidden_layers=3, hidden_size=96, num_attention_heads=8, num_key_value_heads=2, head_dim=32,
                    intermediate_size=224, vocab_size=384, rope_theta=1e6, rms_norm_eps=1e-5, attention_bias=True),
+    "qwen3-0.6b": dict(model_type="qwen3", num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8,
+                       head_dim=128, intermediate_size=3072, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
+                       tie_word_embeddings=True),
     "qwen3-1.7b": dict(model_type="qwen3", num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, num_key_value_heads=8,
                        head_dim=128, intermediate_size=6144, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
                        tie_word_embeddings=True),
+    "qwen3-4b": dict(model_type="qwen3", num_hidden_layers=36, hidden_size=2560, num_attention_heads=32, num_key_value_heads=8,
+                     head_dim=128, intermediate_size=9728, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
+                     tie_word_embeddings=True),
     "qwen3-8b": dict(model_type="qwen3", num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
                      head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6),
     "qwen3-14b": dict(model_type="qwen3", num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,

@@ -3,7 +3,7 @@
 For most shapes the hand-written few-row products win, for some the library's product plus the kernels around it
 does.  Which, is measured (``HipOps.measuring()``: ``Engine.calibrate`` and ``python -m llmserver_amd.kernels.calibrate``
 run it), never while a request is served, and kept per kind of GPU (architecture and number of compute units, such as ``gfx950-256cu``) in JSON files: the table that ships with the package
-(``choices.json`` beside this file, measured for the sizes the benchmarks use) and, if the environment variable
+(``choices.json`` beside this file, measured for the shapes of the sizes that ``config/named_sizes.py`` knows by name) and, if the environment variable
 ``LLMSERVER_AMD_CHOICES`` names one, a table of the user's own, whose entries win.  A shape that no table knows goes
 the hand-written way.  The same tables give the same kernels, so two runs round alike.
 """
