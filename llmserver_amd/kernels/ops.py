@@ -745,10 +745,10 @@ class HipOps(KernelNamespace):
                 _check(cos_sin, "cos_sin", torch.float32, (n, head_dim))
             fusion_mode = 3 if write_cache else 1
         merge_in_workgroup = int(plan.get("merge_in_workgroup", 0))
-        if merge_in_workgroup and (n_items % 4 or n_merges or n_slots or n_tiles or n != rows
+        if merge_in_workgroup and (n_items % 4 or n_merges or n_slots or n_tiles or (merge_in_workgroup == 2 and n != rows)
                                    or (decode_fusion is not None and (q_weight is None or cos_sin is None))):
-            raise ValueError("merging in the workgroup takes steps of one token per row whose plan gives every tile four key ranges "
-                             "(or two, with tiles in pairs) and no slots, and, with decode fusion, both norm weights and a rotation")
+            raise ValueError("merging in the workgroup takes a plan that gives every tile four key ranges (or, in steps of one token "
+                             "per row, two, with tiles in pairs) and no slots, and, with decode fusion, both norm weights and a rotation")
         lib = self._attention_library(qkv.dtype, head_dim)
         if n_tiles and int(plan.get("tile_halves", 1)) not in (1, lib.lsa_attention_tile_halves()):
             raise ValueError(f"the plan splits a workgroup's keys into {plan['tile_halves']} halves, this kernel takes 1 or {lib.lsa_attention_tile_halves()}")

@@ -273,19 +273,25 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     partial results are merged like those of split items).  ``fixed_tiles`` (with ``fixed_splits``): the arrays are
     filled up to the shape of that many tiles, whatever the rows' lengths are (a captured step of prompt portions:
     ``fixed_tiles`` is at least the number of tiles any rows of the step's shape can have), with repetitions of the
-    first tile's entries, which compute and write the same numbers once more."""
+    first tile's entries, which compute and write the same numbers once more.  ``merge_in_workgroup`` (4, or 2 in steps
+    of one token per row with an even number of rows): every tile gets that many ranges, the items of a workgroup, which
+    merges them itself: no slots, no merges, no workgroups of tiles."""
     _, tokens_per_tile, group_tiles = group_tiling(group_size, tuning.tile_rows)
     key_align, key_step, most_splits = tuning.key_align, tuning.key_step, tuning.most_splits
     row_len = np.asarray(row_len, dtype=np.int64)
     row_ctx = np.asarray(row_ctx, dtype=np.int64)
     merge_in_workgroup = WORKGROUP_RANGES if merge_in_workgroup is True else int(merge_in_workgroup)
-    if merge_in_workgroup and not (len(row_len) and int(row_len.min()) == 1 == int(row_len.max())):
-        raise ValueError("key ranges are merged in the workgroup only in steps of one token per row")
+    single_tokens = bool(len(row_len)) and int(row_len.min()) == 1 == int(row_len.max())
+    if merge_in_workgroup == 2 and not single_tokens:
+        raise ValueError("two key ranges of each of two tiles are merged in a workgroup only in steps of one token per row")
     if merge_in_workgroup not in (0, 2, WORKGROUP_RANGES) or (merge_in_workgroup == 2 and len(row_len) % 2):
         raise ValueError("a workgroup merges four key ranges of one tile, or two ranges of each of two tiles (an even number of rows)")
-    if (merge_in_workgroup or (single_token_shortcut and fixed_splits is not None)) and len(row_len) \
-            and int(row_len.min()) == 1 == int(row_len.max()):
+    if (merge_in_workgroup or (single_token_shortcut and fixed_splits is not None)) and single_tokens:
         return _single_token_plan(row_ctx, window, int(fixed_splits or merge_in_workgroup or 1), merge_in_workgroup, key_align)
+    if merge_in_workgroup:
+        # Rows of several tokens: every tile of every row gets exactly four ranges (the last ones may be empty), four
+        # neighbouring items, which their workgroup merges: no slots, no merge, and no workgroups of tiles.
+        fixed_splits, workgroup_tiles = merge_in_workgroup, 0
     tiles_per_row = -(-row_len // tokens_per_tile)
     waves_unsplit = int(tiles_per_row.sum()) * n_kv_heads * group_tiles
     items, slots, merges, tiles = [], [], [], []
@@ -359,11 +365,12 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
             while start < k_end or (fixed_splits is not None and count < splits):
                 lo, hi = max(start, k_begin), min(start + per, k_end)
                 items.append((row, q0, lo, max(lo, hi)) if lo < k_end else (row, q0, k_end, k_end))
-                slots.append(n_slots)
-                n_slots += 1
+                slots.append(-1 if merge_in_workgroup else n_slots)
+                n_slots += 0 if merge_in_workgroup else 1
                 count += 1
                 start += per
-            merges.append((row, q0, first_slot, count))
+            if not merge_in_workgroup:
+                merges.append((row, q0, first_slot, count))
     if fixed_tiles is not None:
         if fixed_splits is None or len(tiles):
             raise ValueError("a plan is filled up to a number of tiles only where every tile gets a fixed number of key ranges")
@@ -379,8 +386,10 @@ def build_attention_plan(row_len, row_ctx, group_size: int, n_kv_heads: int, win
     tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 6)
     tiles = tiles[np.argsort(tiles[:, 2] - tiles[:, 3], kind="stable")]       # most keys first: the long tiles must not start last
     tile_slots = np.ascontiguousarray(tiles[:, 4:]) if len(tiles) and int(tiles[:, 4].max()) >= 0 else None
-    return AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, np.ascontiguousarray(tiles[:, :4]),
+    plan = AttentionPlan(items, np.asarray(slots, dtype=np.int32), merges, n_slots, np.ascontiguousarray(tiles[:, :4]),
                          per_workgroup if len(tiles) else 0, halves if len(tiles) else 1, tile_slots)
+    plan.merge_in_workgroup = merge_in_workgroup
+    return plan
 
 
 class GQAttention(Mixer):
@@ -473,7 +482,8 @@ class GQAttention(Mixer):
             fixed_tiles = ctx.n_tokens // tokens_per_tile + ctx.n_rows
             fixed = fixed_split_count(fixed_tiles, self.group_size, self.n_kv_heads, ctx.static_max_keys, tuning.target_waves, tuning)
         # Where a workgroup can merge a tile's key ranges itself, the merge launch and the partial results go:
-        #  * short contexts (a shape of captured steps of its own, see graph_shape): four ranges a tile;
+        #  * short contexts (a shape of captured steps of its own, see graph_shape): four ranges a tile, in steps of
+        #    single tokens and in captured steps with portions alike;
         #  * so many rows that a tile gets four ranges anyway;
         #  * two ranges a tile: two tiles to a workgroup, if the rows come in pairs.  (Two or three ranges in a workgroup
         #    of one tile leave wavefronts idle through the others' walk: a tenth slower at 64 rows behind 4,096 tokens.)
@@ -483,6 +493,8 @@ class GQAttention(Mixer):
                 in_workgroup = fixed = WORKGROUP_RANGES
             elif fixed == WORKGROUP_RANGES or (fixed == 2 and ctx.n_rows % 2 == 0):
                 in_workgroup = fixed
+        elif ctx.static_max_keys is not None and self.graph_shape(ctx.n_rows, int(np.max(ctx.h_row_ctx))) is not None:
+            in_workgroup = fixed = WORKGROUP_RANGES
         per_workgroup = ctx.ops.attention_workgroup_tiles(ctx.dtype, self.head_dim, ctx.page_size)
         halves = ctx.ops.attention_tile_halves(ctx.dtype, self.head_dim) if per_workgroup else 1
         fewest = ctx.ops.attention_tile_min_workgroups(ctx.dtype) if per_workgroup else 0

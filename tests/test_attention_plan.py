@@ -175,6 +175,47 @@ def test_plan_whose_key_ranges_are_merged_in_the_workgroup(seed):
         assert [(b, e) for _, _, b, e in ranges][len(filled):] == [(context, context)] * (per_tile - len(filled))
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_plan_of_portions_whose_key_ranges_are_merged_in_the_workgroup(seed):
+    """Rows of several tokens: every tile of every row gets four neighbouring items (its key ranges, the last ones may be
+    empty) without slots or merges; the ranges of a tile follow one another from the first key its first token may see to
+    its last token, at multiples of KEY_ALIGN; filled up to a number of tiles, the arrays have that shape and the
+    additions repeat the first tile."""
+    rng = random.Random(seed)
+    rows = rng.randint(1, 6)
+    lens = [rng.choice((1, 2, 7, 8, 9, 40, 128)) for _ in range(rows)]
+    contexts = [n + rng.choice((0, 0, 5, 64, 300)) for n in lens]
+    window = rng.choice((None, None, 40))
+    group_size, n_kv = rng.choice((1, 2, 4, 20)), rng.choice((1, 8))
+    if all(n == 1 for n in lens):
+        lens[0], contexts[0] = 3, contexts[0] + 2
+    _, tokens_per_tile, _ = group_tiling(group_size)
+    real = sum(-(-n // tokens_per_tile) for n in lens)
+    fixed_tiles = rng.choice((None, real, real + 3))
+    plan = build_attention_plan(lens, contexts, group_size, n_kv, window, merge_in_workgroup=4, workgroup_tiles=8, fixed_tiles=fixed_tiles,
+                                **({"fixed_splits": 4} if fixed_tiles else {}))
+    tiles = fixed_tiles or real
+    assert plan.merge_in_workgroup == 4 and plan.items.shape == (4 * tiles, 4) and plan.n_slots == 0 and plan.merges.shape == (0, 4)
+    assert (plan.item_slot == -1).all() and plan.tiles.shape == (0, 4) and plan.tile_slots is None
+    at = 0
+    for row, (n, context) in enumerate(zip(lens, contexts)):
+        for q0 in range(0, n, tokens_per_tile):
+            ranges = plan.items[4 * at:4 * at + 4].tolist()
+            at += 1
+            assert all(r == row and q == q0 for r, q, _, _ in ranges)
+            last = context - n + min(q0 + tokens_per_tile, n)                # one past the last key the tile's last token sees
+            first = 0 if window is None else max(0, context - n + q0 - window + 1)
+            filled = [(b, e) for _, _, b, e in ranges if b < e]
+            assert filled and filled[0][0] == first and filled[-1][1] == last
+            assert all(a[1] == b[0] and b[0] % KEY_ALIGN == 0 for a, b in zip(filled, filled[1:]))
+            assert [(b, e) for _, _, b, e in ranges][len(filled):] == [(last, last)] * (4 - len(filled))
+    assert at == real
+    for extra in range(real, tiles):                                         # the filling repeats the first tile
+        assert (plan.items[4 * extra:4 * extra + 4] == plan.items[:4]).all()
+    with pytest.raises(ValueError):                                          # two ranges a tile: single tokens only
+        build_attention_plan(lens, contexts, group_size, n_kv, window, merge_in_workgroup=2)
+
+
 def test_four_or_eight_tiles_per_workgroup_whole_or_in_halves():
     """With the costs measured on an MI355X: one prompt is bounded by its longest workgroup, whose walk two halves
     shorten (eight tiles at 2,048 tokens, four below); long rows and many rows keep every compute unit busy and take eight

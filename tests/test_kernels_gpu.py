@@ -234,8 +234,18 @@ def test_attention_key_ranges_merged_in_the_workgroup(ops, dtype, n_q, n_kv, d, 
     assert plan.merge_in_workgroup == per_tile and len(plan.items) == per_tile * len(ctxs) and plan.n_slots == 0 and len(plan.merges) == 0
     if window is None:
         assert float(ref[-1, :d].float().mean()) > 5.0           # the far key won the last row's first head
-    with pytest.raises(ValueError):                              # a row of two tokens
-        build_attention_plan([1, 2], [5, 9], n_q // n_kv, n_kv, window, merge_in_workgroup=per_tile)
+    if per_tile == 2:
+        with pytest.raises(ValueError):                          # a row of two tokens: tiles in pairs are for single tokens only
+            build_attention_plan([1, 2], [5, 9], n_q // n_kv, n_kv, window, merge_in_workgroup=per_tile)
+        return
+    # Rows of several tokens (portions of prompts, as captured steps of short contexts have them): every tile of every row
+    # gets four ranges, some of them empty, and the workgroup merges them; portions with and without a prefix, tiles that
+    # are not full, a row of one token among them.
+    lens = [17, 1, 40, 2, 128, 5]
+    ctxs = [17, 33, 140, 65, 512, 300]
+    plan, _ = attention_case(ops, dtype, n_q, n_kv, d, page, lens, ctxs, window=window, seed=n_q * d + 2, merge_in_workgroup=per_tile)
+    assert plan.merge_in_workgroup == 4 and len(plan.items) % 4 == 0 and plan.n_slots == 0 and len(plan.merges) == 0
+    assert (plan.item_slot == -1).all() and len(plan.tiles) == 0
 
 
 @pytest.mark.parametrize("n_q, n_kv, d, page", [(32, 8, 128, 16), (4, 2, 64, 8), (20, 1, 64, 16), (6, 3, 192, 12), (2, 1, 256, 64)])
