@@ -7,7 +7,10 @@ into the residual stream as partial sums (two layers, so that the feed-forward's
 
 A second test runs a mixed trace at these widths (a portion of 300 tokens and one of 40 beside 24 and 64 rows of one token
 each, pages given back and used again), a third all 36 layers of Qwen3-8B once: what the depth does to bfloat16, and
-to the 32-bit path, against the plain implementation run on the GPU."""
+to the 32-bit path, against the plain implementation run on the GPU.
+
+The first two run at the widths of Qwen3-4B as well (2560, 32/8 heads, intermediate 9728: no powers of two, products
+whose ranges of the inner dimension end in a shorter one, 20 tiles of weight rows where 8B has 32)."""
 import random
 
 import numpy as np
@@ -26,10 +29,13 @@ REAL = dict(model_type="qwen3", num_hidden_layers=2, hidden_size=4096, num_atten
             attention_bias=False, tie_word_embeddings=True)
 
 
-@pytest.fixture(scope="module")
-def real_model(tmp_path_factory):
+OTHER_WIDTHS = dict(REAL, hidden_size=2560, intermediate_size=9728)
+
+
+@pytest.fixture(scope="module", params=[REAL, OTHER_WIDTHS], ids=["widths of 8B", "widths of 4B"])
+def real_model(request, tmp_path_factory):
     folder = str(tmp_path_factory.mktemp("real_size"))
-    write_random_model(config_from_dict(dict(REAL)), folder, RandomInit(seed=2, std=0.02, norm_noise=0.1))
+    write_random_model(config_from_dict(dict(request.param)), folder, RandomInit(seed=2, std=0.02, norm_noise=0.1))
     config, tensors = plain.read_folder(folder, dtype=torch.float32)
     tokens = random_tokens(REAL["vocab_size"], 83, 77)
     with torch.no_grad():
