@@ -245,6 +245,41 @@ __global__ __launch_bounds__(256, LSA_MIN_WAVES) void paged_attention_kernel(
             return none ? (size_t)0 : page;
         };
 #if LSA_BF16
+        // A step that lies inside the item's range, with pages of a multiple of 16 keys: each half of the step lies in
+        // one page, the same for all lanes, which one lane's table entry names (no exchange between lanes, and the
+        // page's address is a scalar).
+        if ((ps & 15) == 0 && kt >= k_begin && kt + KEY_STEP <= k_end) {
+            size_t page[2];
+            int slot0[2];
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                const int first = kt + 16 * t2;
+                const int block = (int)__umulhi((unsigned)first, g.page_magic);
+                slot0[t2] = first - block * ps;
+                page[t2] = (size_t)__builtin_amdgcn_readlane(pages_cur, block - 64 * chunk) * page_elems;
+            }
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                const elem_t* kp = keys + page[t2] + kv_head_keys + (size_t)(slot0[t2] + col) * D + 8 * quad;
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    if (32 * s + 32 <= D) {
+                        f.k[t2][s] = *reinterpret_cast<const bf16x8*>(kp + 32 * s);
+                    } else {
+                        bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + 32 * s - (quad >= 2 ? 16 : 0));
+                        if (quad >= 2) kf = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+                        f.k[t2][s] = kf;
+                    }
+                }
+            }
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                const elem_t* vp = values + page[t2] + kv_head_values + (size_t)col * ps + slot0[t2] + 4 * quad;
+#pragma unroll
+                for (int c = 0; c < ND; ++c) f.v[c][t2] = *reinterpret_cast<const bf16x4*>(vp + (size_t)(16 * c) * ps);
+            }
+            return;
+        }
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
             int slot;
